@@ -1,0 +1,364 @@
+// Memory-aware row aggregation over a block CSR, and the block transpose that lets the
+// backward pass run as the same gather (stands in for the reference's forward kernels,
+// cuda_operators/aggregate_acc_kernel.cu:270-331,375-427, and -- on the transposed block --
+// for its atomic-scatter backward kernels, :467-517,554-596).
+//
+// Mapping: one LPR-lane group per (output row, column slice); LPR in {8,16,32,64} is the
+// smallest power of two that covers the row with one 16-byte (or narrower, if the row
+// length or stride forbids it) vector load per lane, so a 128-float row is one
+// global_load_dwordx4 from each of 32 lanes and a wave streams two rows at a time.  The
+// group's lanes first load up to LPR neighbour ids (and their per-edge weights) in one
+// coalesced read, then broadcast them lane by lane; the row loads are issued four at a
+// time before the first FMA so that each lane keeps several 16-byte loads in flight.
+// Accumulation is fp32, in CSR order, in registers: no shared-memory read-modify-write
+// and no redundant staging of the id list as in the reference kernel.
+#include "fgl_common.hpp"
+#include "fgl_kernels.hpp"
+
+namespace fgl {
+
+template <int N>
+struct VecF32 { float v[N]; };
+
+// ---- vector load / store of VEC elements as fp32 -----------------------------------
+template <typename T, int VEC>
+struct RowIO;
+
+template <int VEC>
+struct RowIO<float, VEC> {
+    using Raw = float __attribute__((ext_vector_type(VEC)));
+    static __device__ __forceinline__ Raw load(const float* p) { return *reinterpret_cast<const Raw*>(p); }
+    static __device__ __forceinline__ void fma(float (&acc)[VEC], float w, Raw r)
+    {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += w * r[i];
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&acc)[VEC])
+    {
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) r[i] = acc[i];
+        *reinterpret_cast<Raw*>(p) = r;
+    }
+};
+template <>
+struct RowIO<float, 1> {
+    using Raw = float;
+    static __device__ __forceinline__ Raw load(const float* p) { return *p; }
+    static __device__ __forceinline__ void fma(float (&acc)[1], float w, Raw r) { acc[0] += w * r; }
+    static __device__ __forceinline__ void store(float* p, const float (&acc)[1]) { *p = acc[0]; }
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (u >> 16) | 0x40u;  // quiet NaN
+    u += 0x7FFFu + ((u >> 16) & 1u);                                                       // round to nearest even
+    return u >> 16;
+}
+
+// bf16 rows are moved as 32-bit words holding two elements (VEC is even) or as single halfwords.
+template <int VEC>
+struct RowIO<uint16_t, VEC> {
+    static_assert(VEC % 2 == 0, "bf16 vectors hold an even number of elements");
+    using Raw = uint32_t __attribute__((ext_vector_type(VEC / 2)));
+    static __device__ __forceinline__ Raw load(const uint16_t* p) { return *reinterpret_cast<const Raw*>(p); }
+    static __device__ __forceinline__ void fma(float (&acc)[VEC], float w, Raw r)
+    {
+#pragma unroll
+        for (int i = 0; i < VEC / 2; ++i) {
+            acc[2 * i] += w * bf16_bits_to_f32(r[i] & 0xFFFFu);
+            acc[2 * i + 1] += w * bf16_bits_to_f32(r[i] >> 16);
+        }
+    }
+    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[VEC])
+    {
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < VEC / 2; ++i) r[i] = f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16);
+        *reinterpret_cast<Raw*>(p) = r;
+    }
+};
+template <>
+struct RowIO<uint16_t, 2> {
+    using Raw = uint32_t;
+    static __device__ __forceinline__ Raw load(const uint16_t* p) { return *reinterpret_cast<const uint32_t*>(p); }
+    static __device__ __forceinline__ void fma(float (&acc)[2], float w, Raw r)
+    {
+        acc[0] += w * bf16_bits_to_f32(r & 0xFFFFu);
+        acc[1] += w * bf16_bits_to_f32(r >> 16);
+    }
+    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[2])
+    {
+        *reinterpret_cast<uint32_t*>(p) = f32_to_bf16_bits(acc[0]) | (f32_to_bf16_bits(acc[1]) << 16);
+    }
+};
+template <>
+struct RowIO<uint16_t, 1> {
+    using Raw = uint16_t;
+    static __device__ __forceinline__ Raw load(const uint16_t* p) { return *p; }
+    static __device__ __forceinline__ void fma(float (&acc)[1], float w, Raw r) { acc[0] += w * bf16_bits_to_f32(r); }
+    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[1]) { *p = (uint16_t)f32_to_bf16_bits(acc[0]); }
+};
+
+// per-edge weight, evaluated by the lane that loaded the neighbour id
+template <int MODE>
+__device__ __forceinline__ float edge_weight(int col, float row_factor, const int32_t* __restrict__ col_norm)
+{
+    if (MODE == FGL_AGG_GCN) return row_factor * (1.0f / sqrtf((float)col_norm[col]));
+    if (MODE == FGL_AGG_COLMEAN) {
+        const int c = col_norm[col];
+        return 1.0f / (float)(c > 1 ? c : 1);
+    }
+    return row_factor;  // SUM: 1, MEAN: 1/deg(row)
+}
+
+template <typename T, int VEC, int LPR, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __restrict__ indptr,
+                                                           const int32_t* __restrict__ indices, int64_t n_rows_max,
+                                                           const int32_t* __restrict__ d_n_rows,
+                                                           const T* __restrict__ X, int64_t ldx, int D, int zero_policy,
+                                                           const int32_t* __restrict__ row_norm,
+                                                           const int32_t* __restrict__ col_norm, T* __restrict__ out,
+                                                           int64_t ldo)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int kGroups = kBlock / LPR;
+    const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
+    const int gl = (int)threadIdx.x % LPR;  // lane within the group
+    const int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
+    if (row >= n_rows) return;  // uniform per group: the cross-lane reads below stay inside the group
+    const int col0 = ((int)blockIdx.y * LPR + gl) * VEC;
+    const bool live = col0 < D;
+
+    const int a = indptr[row], b = indptr[row + 1];
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+
+    if (a == b) {
+        if (live) {
+            if (zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, IO::load(X + row * ldx + col0));
+            IO::store(out + row * ldo + col0, acc);
+        }
+        return;
+    }
+
+    float row_factor = 1.0f;
+    if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
+    if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)row_norm[row]);
+
+    for (int base = a; base < b; base += LPR) {
+        const int cnt = (b - base) < LPR ? (b - base) : LPR;
+        int my_col = 0;
+        float my_w = 0.0f;
+        if (gl < cnt) {
+            my_col = indices[base + gl];
+            my_w = edge_weight<MODE>(my_col, row_factor, col_norm);
+        }
+        int t = 0;
+        for (; t + 4 <= cnt; t += 4) {
+            const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
+            const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
+            const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
+            const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
+            if (live) {
+                const typename IO::Raw r0 = IO::load(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r1 = IO::load(X + (int64_t)c1 * ldx + col0);
+                const typename IO::Raw r2 = IO::load(X + (int64_t)c2 * ldx + col0);
+                const typename IO::Raw r3 = IO::load(X + (int64_t)c3 * ldx + col0);
+                IO::fma(acc, w0, r0);
+                IO::fma(acc, w1, r1);
+                IO::fma(acc, w2, r2);
+                IO::fma(acc, w3, r3);
+            }
+        }
+        for (; t < cnt; ++t) {
+            const int c0 = __shfl(my_col, t, LPR);
+            const float w0 = __shfl(my_w, t, LPR);
+            if (live) IO::fma(acc, w0, IO::load(X + (int64_t)c0 * ldx + col0));
+        }
+    }
+    if (live) IO::store(out + row * ldo + col0, acc);
+}
+
+// ---- block transpose ---------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* __restrict__ indptr,
+                                                                 const int32_t* __restrict__ indices, int64_t n_rows_max,
+                                                                 const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
+                                                                 int64_t n_cols_max, int32_t* __restrict__ counts,
+                                                                 int32_t* __restrict__ rank)
+{
+    const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
+    int64_t n_e = n_rows > 0 ? (int64_t)indptr[n_rows] : 0;
+    if (n_e > n_edges_max) n_e = n_edges_max;
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n_e) return;
+    const int32_t c = indices[e];
+    if (c >= 0 && (int64_t)c < n_cols_max) rank[e] = atomicAdd(&counts[c], 1);
+    else rank[e] = -1;
+}
+
+__global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* __restrict__ indptr,
+                                                                const int32_t* __restrict__ indices, int64_t n_rows_max,
+                                                                const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
+                                                                const int32_t* __restrict__ t_indptr,
+                                                                const int32_t* __restrict__ rank,
+                                                                int32_t* __restrict__ t_indices)
+{
+    const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r >= n_rows) return;
+    int64_t a = indptr[r], b = indptr[r + 1];
+    if (b > n_edges_max) b = n_edges_max;
+    for (int64_t e = a; e < b; ++e) {
+        const int32_t k = rank[e];
+        if (k >= 0) t_indices[(int64_t)t_indptr[indices[e]] + k] = (int32_t)r;
+    }
+}
+
+size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
+{
+    Carver c(nullptr);
+    c.take<int32_t>((size_t)n_edges_max);
+    c.take<char>(scan_workspace_bytes(n_cols_max));
+    return c.used();
+}
+
+// ---- dispatch ----------------------------------------------------------------------
+template <typename T, int VEC, int LPR>
+static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const int32_t* indptr, const int32_t* indices,
+                           int64_t n_rows_max, const int32_t* d_n_rows, const T* X, int64_t ldx, int D, int zero_policy,
+                           const int32_t* row_norm, const int32_t* col_norm, T* out, int64_t ldo)
+{
+#define FGL_LAUNCH_MODE(M)                                                                                            \
+    hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, indptr, indices, n_rows_max, \
+                       d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo)
+    switch (mode) {
+        case FGL_AGG_SUM: FGL_LAUNCH_MODE(FGL_AGG_SUM); break;
+        case FGL_AGG_MEAN: FGL_LAUNCH_MODE(FGL_AGG_MEAN); break;
+        case FGL_AGG_GCN: FGL_LAUNCH_MODE(FGL_AGG_GCN); break;
+        default: FGL_LAUNCH_MODE(FGL_AGG_COLMEAN); break;
+    }
+#undef FGL_LAUNCH_MODE
+    FGL_CHECK_LAUNCH("aggregate_kernel");
+    return FGL_OK;
+}
+
+template <typename T, int VEC>
+static int launch_agg_vec(int mode, hipStream_t stream, const int32_t* indptr, const int32_t* indices, int64_t n_rows_max,
+                          const int32_t* d_n_rows, const T* X, int64_t ldx, int D, int zero_policy,
+                          const int32_t* row_norm, const int32_t* col_norm, T* out, int64_t ldo)
+{
+    const int lanes_needed = (D + VEC - 1) / VEC;
+    int lpr = 8;
+    while (lpr < 64 && lpr < lanes_needed) lpr <<= 1;
+    const int64_t groups = kBlock / lpr;
+    const int64_t gx = ceil_div(n_rows_max, groups);
+    const int64_t gy = ceil_div(lanes_needed, lpr);
+    if (gx > 0x7FFFFFFF || gy > 65535) {
+        set_error("aggregate: grid too large (%lld x %lld)", (long long)gx, (long long)gy);
+        return FGL_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)gx, (unsigned)gy);
+    switch (lpr) {
+        case 8: return launch_agg_mode<T, VEC, 8>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
+        case 16: return launch_agg_mode<T, VEC, 16>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
+        case 32: return launch_agg_mode<T, VEC, 32>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
+        default: return launch_agg_mode<T, VEC, 64>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
+    }
+}
+
+// widest vector (in elements) that the row length, both strides and both base addresses allow
+static int pick_vec(int D, int64_t ldx, int64_t ldo, const void* x, const void* out, int elem_bytes)
+{
+    int vec = 16 / elem_bytes;
+    while (vec > 1) {
+        const uintptr_t bytes = (uintptr_t)vec * elem_bytes;
+        if (D % vec == 0 && ldx % vec == 0 && ldo % vec == 0 && ((uintptr_t)x % bytes) == 0 && ((uintptr_t)out % bytes) == 0) break;
+        vec >>= 1;
+    }
+    return vec;
+}
+
+}  // namespace fgl
+
+using namespace fgl;
+
+FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
+                             const int32_t* d_n_rows, const void* d_x, int64_t ldx, int D, int dtype, int mode,
+                             int zero_policy, const int32_t* d_row_norm, const int32_t* d_col_norm, void* d_out,
+                             int64_t ldo, void* stream)
+{
+    FGL_REQUIRE(n_rows_max >= 0, "aggregate: negative row count");
+    FGL_REQUIRE(D >= 1, "aggregate: feature length %d < 1", D);
+    FGL_REQUIRE(ldx >= D && ldo >= D, "aggregate: row stride smaller than the row length");
+    FGL_REQUIRE(dtype == FGL_F32 || dtype == FGL_BF16, "aggregate: unknown dtype %d", dtype);
+    FGL_REQUIRE(mode >= FGL_AGG_SUM && mode <= FGL_AGG_COLMEAN, "aggregate: unknown mode %d", mode);
+    FGL_REQUIRE(zero_policy == FGL_ZERO_COPY_SELF || zero_policy == FGL_ZERO_ZEROS, "aggregate: unknown zero policy %d", zero_policy);
+    FGL_REQUIRE(mode != FGL_AGG_GCN || (d_row_norm && d_col_norm), "aggregate: gcn mode needs row_norm and col_norm");
+    FGL_REQUIRE(mode != FGL_AGG_COLMEAN || d_col_norm, "aggregate: colmean mode needs col_norm");
+    if (n_rows_max == 0) return FGL_OK;
+    FGL_REQUIRE(d_indptr && d_indices && d_x && d_out, "aggregate: null pointer");
+    FGL_REQUIRE(d_x != d_out, "aggregate: output aliases the input");
+    hipStream_t s = as_stream(stream);
+    if (dtype == FGL_F32) {
+        const float* X = static_cast<const float*>(d_x);
+        float* O = static_cast<float*>(d_out);
+        switch (pick_vec(D, ldx, ldo, d_x, d_out, 4)) {
+            case 4: return launch_agg_vec<float, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+            case 2: return launch_agg_vec<float, 2>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+            default: return launch_agg_vec<float, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+        }
+    }
+    const uint16_t* X = static_cast<const uint16_t*>(d_x);
+    uint16_t* O = static_cast<uint16_t*>(d_out);
+    switch (pick_vec(D, ldx, ldo, d_x, d_out, 2)) {
+        case 8: return launch_agg_vec<uint16_t, 8>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+        case 4: return launch_agg_vec<uint16_t, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+        case 2: return launch_agg_vec<uint16_t, 2>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+        default: return launch_agg_vec<uint16_t, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+    }
+}
+
+FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
+{
+    if (n_cols_max < 0 || n_edges_max < 0) return 0;
+    return transpose_workspace_bytes(n_cols_max, n_edges_max);
+}
+
+FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
+                                   const int32_t* d_n_rows, int64_t n_cols_max, const int32_t* d_n_cols,
+                                   int64_t n_edges_max, int32_t* d_t_indptr, int32_t* d_t_indices, void* d_ws,
+                                   size_t ws_bytes, void* stream)
+{
+    FGL_REQUIRE(n_rows_max >= 0 && n_cols_max >= 0 && n_edges_max >= 0, "block_transpose: negative size");
+    FGL_REQUIRE(n_edges_max <= 0x7FFFFFFF, "block_transpose: edge count exceeds int32 offsets");
+    FGL_REQUIRE(d_t_indptr != nullptr, "block_transpose: null output");
+    FGL_REQUIRE(n_edges_max == 0 || (d_indptr && d_indices && d_t_indices), "block_transpose: null pointer");
+    if (d_ws == nullptr || ws_bytes < transpose_workspace_bytes(n_cols_max, n_edges_max)) {
+        set_error("block_transpose: workspace too small (%zu < %zu)", ws_bytes, transpose_workspace_bytes(n_cols_max, n_edges_max));
+        return FGL_ERR_WORKSPACE;
+    }
+    hipStream_t s = as_stream(stream);
+    Carver c(d_ws);
+    int32_t* rank = c.take<int32_t>((size_t)n_edges_max);
+    char* scan_ws = c.take<char>(scan_workspace_bytes(n_cols_max));
+    // the counts live in t_indptr and are scanned in place
+    int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(d_t_indptr), n_cols_max + 1, 0u, s);
+    if (rc != FGL_OK) return rc;
+    if (n_edges_max > 0 && n_rows_max > 0) {
+        hipLaunchKernelGGL(transpose_count_kernel, dim3((unsigned)ceil_div(n_edges_max, kBlock)), dim3(kBlock), 0, s,
+                           d_indptr, d_indices, n_rows_max, d_n_rows, n_edges_max, n_cols_max, d_t_indptr, rank);
+        FGL_CHECK_LAUNCH("transpose_count_kernel");
+    }
+    rc = launch_exclusive_sum(d_t_indptr, n_cols_max, d_n_cols, d_t_indptr, nullptr, scan_ws, scan_workspace_bytes(n_cols_max), s);
+    if (rc != FGL_OK) return rc;
+    if (n_edges_max > 0 && n_rows_max > 0) {
+        hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)ceil_div(n_rows_max, kBlock)), dim3(kBlock), 0, s, d_indptr,
+                           d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices);
+        FGL_CHECK_LAUNCH("transpose_fill_kernel");
+    }
+    return FGL_OK;
+}

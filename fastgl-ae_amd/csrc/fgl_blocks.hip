@@ -1,0 +1,165 @@
+// All hops of one mini-batch in a single enqueue (stands in for the layer loop of the
+// reference's FusedMapSampler.sample_blocks, FusedMapSampler.py:63-109, which synchronises
+// with the host at least four times per hop and rebuilds its hash table per hop,
+// id_map.cu:408-409,454).  Here the table and the numbering persist across hops -- hop h's
+// unique list is hop h+1's seed list with the same local ids -- node and edge counts stay on
+// the device, and each launch is sized by a host-side bound and reads the actual count.
+//
+// Also: the seeded R-MAT key generator used to build the synthetic benchmark graphs.
+#include "fgl_common.hpp"
+#include "fgl_kernels.hpp"
+
+namespace fgl {
+
+__global__ void blocks_init_counts_kernel(int32_t* __restrict__ counts, int n_entries, int32_t n_seeds)
+{
+    const int i = (int)threadIdx.x;
+    if (i < n_entries) counts[i] = (i == 0) ? n_seeds : 0;
+}
+
+struct BlocksPlan {
+    int64_t cap_dst[32];
+    int64_t cap_edges[32];
+    int64_t cap_uniq;
+    int64_t table_slots;
+    size_t ws_bytes;
+};
+
+static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops, BlocksPlan* p)
+{
+    FGL_REQUIRE(n_hops >= 1 && n_hops <= 32, "sample_blocks: %d hops outside [1, 32]", n_hops);
+    FGL_REQUIRE(n_nodes >= 0 && n_seeds >= 0 && fanouts != nullptr, "sample_blocks: bad sizes");
+    int64_t cur = n_seeds;
+    size_t ws = 0;
+    for (int h = 0; h < n_hops; ++h) {
+        FGL_REQUIRE(fanouts[h] >= 1 && fanouts[h] <= FGL_MAX_FANOUT, "sample_blocks: fanout %d outside [1, %d]", fanouts[h], FGL_MAX_FANOUT);
+        p->cap_dst[h] = cur;
+        p->cap_edges[h] = cur * fanouts[h];
+        FGL_REQUIRE(p->cap_edges[h] <= 0x7FFFFFFF, "sample_blocks: hop %d may produce %lld edges, beyond int32 offsets", h, (long long)p->cap_edges[h]);
+        size_t w = sample_workspace_bytes(p->cap_dst[h], fanouts[h]) + idmap_map_src_workspace_bytes(p->cap_edges[h]);
+        if (w > ws) ws = w;
+        // every node is numbered once; repeated seeds are the only way past n_nodes
+        int64_t next = cur + p->cap_edges[h];
+        if (next > n_nodes + n_seeds) next = n_nodes + n_seeds;
+        cur = next;
+    }
+    p->cap_uniq = cur;
+    p->table_slots = fgl_idmap_slots(cur);
+    FGL_REQUIRE(p->table_slots <= ((int64_t)1 << 31), "sample_blocks: table too large");
+    p->ws_bytes = ws;
+    return FGL_OK;
+}
+
+// ---- R-MAT -------------------------------------------------------------------------
+constexpr uint32_t kCutA = 0x91EB851Eu;  // floor(0.57 * 2^32)
+constexpr uint32_t kCutB = 0xC28F5C28u;  // floor(0.76 * 2^32)
+constexpr uint32_t kCutC = 0xF3333333u;  // floor(0.95 * 2^32)
+
+__global__ __launch_bounds__(kBlock) void rmat_keys_kernel(int64_t first_edge, int64_t n_edges, int scale, int64_t n_nodes,
+                                                           uint32_t seed_lo, uint32_t seed_hi, int64_t* __restrict__ keys)
+{
+    const int64_t x = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (x >= n_edges) return;
+    const uint64_t e = (uint64_t)(first_edge + x);
+    uint64_t u = 0, v = 0;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+    for (int lvl = 0; lvl < scale; ++lvl) {
+        if ((lvl & 3) == 0) philox4x32_10((uint32_t)e, (uint32_t)(e >> 32), (uint32_t)(lvl >> 2), 0x524D4154u, seed_lo, seed_hi, o);
+        const uint32_t r = o[lvl & 3];
+        const uint32_t ub = r >= kCutB;
+        const uint32_t vb = (r >= kCutA && r < kCutB) || r >= kCutC;
+        u = (u << 1) | ub;
+        v = (v << 1) | vb;
+    }
+    int64_t k0 = INT64_MAX, k1 = INT64_MAX;
+    if (u != v && u < (uint64_t)n_nodes && v < (uint64_t)n_nodes) {
+        k0 = (int64_t)((v << 32) | u);
+        k1 = (int64_t)((u << 32) | v);
+    }
+    keys[2 * x] = k0;
+    keys[2 * x + 1] = k1;
+}
+
+}  // namespace fgl
+
+using namespace fgl;
+
+FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
+                                      int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq, int64_t* table_slots,
+                                      size_t* ws_bytes)
+{
+    BlocksPlan p;
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, &p);
+    if (rc != FGL_OK) return rc;
+    for (int h = 0; h < n_hops; ++h) {
+        if (cap_dst) cap_dst[h] = p.cap_dst[h];
+        if (cap_edges) cap_edges[h] = p.cap_edges[h];
+    }
+    if (cap_uniq) *cap_uniq = p.cap_uniq;
+    if (table_slots) *table_slots = p.table_slots;
+    if (ws_bytes) *ws_bytes = p.ws_bytes;
+    return FGL_OK;
+}
+
+FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                                 const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
+                                 uint64_t rng_seed, uint32_t stream_base, void* d_table, int64_t table_slots,
+                                 int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
+                                 int32_t* const* src_local, int32_t* const* src_global, int32_t* d_counts, void* d_ws,
+                                 size_t ws_bytes, void* stream)
+{
+    BlocksPlan p;
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, &p);
+    if (rc != FGL_OK) return rc;
+    FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
+    FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
+    FGL_REQUIRE(table_slots >= p.table_slots, "sample_blocks: table has %lld slots, plan needs %lld", (long long)table_slots, (long long)p.table_slots);
+    FGL_REQUIRE(uniq_capacity >= p.cap_uniq, "sample_blocks: unique list holds %lld, plan needs %lld", (long long)uniq_capacity, (long long)p.cap_uniq);
+    if (d_ws == nullptr || ws_bytes < p.ws_bytes) {
+        set_error("sample_blocks: workspace too small (%zu < %zu)", ws_bytes, p.ws_bytes);
+        return FGL_ERR_WORKSPACE;
+    }
+    for (int h = 0; h < n_hops; ++h) FGL_REQUIRE(block_ptr[h] && src_local[h], "sample_blocks: null output for hop %d", h);
+
+    hipStream_t s = as_stream(stream);
+    const int n_counts = 2 * n_hops + 2;
+    uint32_t* d_status = reinterpret_cast<uint32_t*>(d_counts + 2 * n_hops + 1);
+    hipLaunchKernelGGL(blocks_init_counts_kernel, dim3(1), dim3(128), 0, s, d_counts, n_counts, (int32_t)n_seeds);
+    FGL_CHECK_LAUNCH("blocks_init_counts_kernel");
+    rc = launch_idmap_reset(d_table, table_slots, s);
+    if (rc != FGL_OK) return rc;
+    rc = launch_idmap_insert_dst(d_table, table_slots, d_seeds, n_seeds, nullptr, d_uniq, d_status, s);
+    if (rc != FGL_OK) return rc;
+
+    for (int h = 0; h < n_hops; ++h) {
+        const int32_t* hop_seeds = (h == 0) ? d_seeds : d_uniq;
+        int32_t* d_n_dst = d_counts + h;
+        int32_t* d_n_edges = d_counts + n_hops + 1 + h;
+        int32_t* sampled = (src_global && src_global[h]) ? src_global[h] : src_local[h];
+        char* ws = static_cast<char*>(d_ws);
+        const size_t ws_sample = sample_workspace_bytes(p.cap_dst[h], fanouts[h]);
+        rc = launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], rng_seed,
+                           stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s);
+        if (rc != FGL_OK) return rc;
+        rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
+                                  d_counts + h + 1, d_uniq, uniq_capacity, FGL_IDMAP_ORDERED, d_status, ws + ws_sample,
+                                  ws_bytes - ws_sample, s);
+        if (rc != FGL_OK) return rc;
+    }
+    return FGL_OK;
+}
+
+FGL_EXPORT int fgl_rmat_keys(int64_t first_edge, int64_t n_edges, int scale, int64_t n_nodes, uint64_t seed,
+                             int64_t* d_keys, void* stream)
+{
+    FGL_REQUIRE(first_edge >= 0 && n_edges >= 0 && n_nodes >= 0, "rmat_keys: negative size");
+    FGL_REQUIRE(scale >= 1 && scale <= 31, "rmat_keys: scale %d outside [1, 31]", scale);
+    if (n_edges == 0) return FGL_OK;
+    FGL_REQUIRE(d_keys != nullptr, "rmat_keys: null output");
+    const int64_t blocks = ceil_div(n_edges, kBlock);
+    FGL_REQUIRE(blocks <= 0x7FFFFFFF, "rmat_keys: too many edges in one call");
+    hipLaunchKernelGGL(rmat_keys_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream), first_edge, n_edges,
+                       scale, n_nodes, (uint32_t)seed, (uint32_t)(seed >> 32), d_keys);
+    FGL_CHECK_LAUNCH("rmat_keys_kernel");
+    return FGL_OK;
+}

@@ -1,0 +1,210 @@
+// CSR neighbour sampling without replacement (stands in for the reference's
+// sample_node_cuda, cuda_operators/sample.cu:102-203).
+//
+// Three launches, no host synchronisation:
+//   1. sample_degree_kernel   one lane per seed: two offsets of the row, k = min(fanout, deg),
+//                             staged row start / degree, per-tile sum of k
+//   2. tile prefix            single workgroup; also writes block_ptr[n] and the edge count
+//   3. sample_edges_kernel    per tile of TS seeds: wave64 scan of k -> output offsets,
+//                             Floyd subset selection for rows longer than the fanout (one lane
+//                             per seed, picks kept in LDS, conflict-free [pick][seed] layout),
+//                             then a flat pass over the tile's output edges so that the
+//                             src/dst writes are fully coalesced and the copy-all rows read
+//                             `indices` contiguously.
+#include "fgl_common.hpp"
+#include "fgl_kernels.hpp"
+
+namespace fgl {
+
+template <int TS>
+__global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restrict__ indptr, int is64, int64_t n_nodes,
+                                                           const int32_t* __restrict__ seeds, int64_t n_max,
+                                                           const int32_t* __restrict__ d_n, int fanout,
+                                                           int64_t* __restrict__ row_start, int32_t* __restrict__ deg_out,
+                                                           int32_t* __restrict__ tile_sums, uint32_t* __restrict__ d_status)
+{
+    __shared__ int smem[TS / kWave + 1];
+    const int64_t n = actual_count(n_max, d_n);
+    const int64_t i = (int64_t)blockIdx.x * TS + threadIdx.x;
+    int k = 0;
+    if (i < n) {
+        const int64_t s = seeds[i];
+        int64_t a = 0, deg = 0;
+        if (s >= 0 && s < n_nodes) {
+            if (is64) {
+                const int64_t* p = static_cast<const int64_t*>(indptr);
+                a = p[s];
+                deg = p[s + 1] - a;
+            } else {
+                const int32_t* p = static_cast<const int32_t*>(indptr);
+                a = p[s];
+                deg = (int64_t)p[s + 1] - a;
+            }
+            if (deg < 0) deg = 0;
+            if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
+        } else if (d_status) {
+            atomicOr(d_status, FGL_STATUS_BAD_SEED);
+        }
+        row_start[i] = a;
+        deg_out[i] = (int32_t)deg;
+        k = deg < fanout ? (int)deg : fanout;
+    }
+    int total;
+    (void)block_exclusive_scan<TS>(k, smem, &total);
+    if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+template <int TS>
+__global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restrict__ indices,
+                                                          const int32_t* __restrict__ seeds, int64_t n_max,
+                                                          const int32_t* __restrict__ d_n, int fanout,
+                                                          const int64_t* __restrict__ row_start,
+                                                          const int32_t* __restrict__ deg_arr,
+                                                          const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
+                                                          uint32_t seed_hi, uint32_t stream_id,
+                                                          int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
+                                                          int32_t* __restrict__ block_ptr)
+{
+    extern __shared__ uint32_t s_sel[];  // [fanout][TS] picked positions
+    __shared__ int s_scan[TS / kWave + 1];
+    __shared__ int s_off[TS + 1];
+    __shared__ int64_t s_row[TS];
+    __shared__ int s_deg[TS];
+    __shared__ int s_seed[TS];
+
+    const int tid = (int)threadIdx.x;
+    const int64_t n = actual_count(n_max, d_n);
+    const int64_t i = (int64_t)blockIdx.x * TS + tid;
+    int deg = 0, seed = 0;
+    int64_t row = 0;
+    if (i < n) {
+        deg = deg_arr[i];
+        row = row_start[i];
+        seed = seeds[i];
+    }
+    const int k = deg < fanout ? deg : fanout;
+    int total;
+    const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
+    const int base = tile_prefix[blockIdx.x];
+    s_off[tid] = ex;
+    if (tid == 0) s_off[TS] = total;
+    s_row[tid] = row;
+    s_deg[tid] = deg;
+    s_seed[tid] = seed;
+    if (i < n) block_ptr[i] = base + ex;
+
+    if (deg > fanout) {
+        // Floyd: for j = deg-k .. deg-1 draw t in [0, j]; take t unless already taken, else j.
+        uint32_t o[4];
+        for (int m = 0; m < fanout; ++m) {
+            if ((m & 1) == 0) philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32), stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
+            const uint64_t r = (m & 1) ? ((uint64_t)o[2] | ((uint64_t)o[3] << 32)) : ((uint64_t)o[0] | ((uint64_t)o[1] << 32));
+            const uint32_t j = (uint32_t)(deg - fanout + m);
+            const uint32_t t = (uint32_t)__umul64hi(r, (uint64_t)j + 1u);
+            bool dup = false;
+            for (int q = 0; q < m; ++q) dup |= (s_sel[q * TS + tid] == t);
+            s_sel[m * TS + tid] = dup ? j : t;
+        }
+    }
+    __syncthreads();
+
+    for (int x = tid; x < total; x += TS) {
+        int lo = 0, hi = TS;  // s_off[lo] <= x < s_off[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_off[mid] <= x) lo = mid; else hi = mid;
+        }
+        const int j = x - s_off[lo];
+        const int64_t pos = s_deg[lo] <= fanout ? (int64_t)j : (int64_t)s_sel[j * TS + lo];
+        src_out[(int64_t)base + x] = indices[s_row[lo] + pos];
+        if (dst_out) dst_out[(int64_t)base + x] = s_seed[lo];
+    }
+}
+
+static inline int tile_seeds_for(int fanout) { return fanout <= 48 ? 256 : 64; }
+
+size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
+{
+    const int ts = tile_seeds_for(fanout);
+    const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, ts);
+    Carver c(nullptr);
+    c.take<int64_t>((size_t)n_seeds_max);
+    c.take<int32_t>((size_t)n_seeds_max);
+    c.take<int32_t>((size_t)tiles);
+    c.take<int32_t>((size_t)tiles);
+    return c.used();
+}
+
+template <int TS>
+static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                            const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                            uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
+                            int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws,
+                            hipStream_t stream)
+{
+    const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, TS);
+    Carver c(d_ws);
+    int64_t* row_start = c.take<int64_t>((size_t)n_seeds_max);
+    int32_t* deg = c.take<int32_t>((size_t)n_seeds_max);
+    int32_t* sums = c.take<int32_t>((size_t)tiles);
+    int32_t* prefix = c.take<int32_t>((size_t)tiles);
+
+    hipLaunchKernelGGL(sample_degree_kernel<TS>, dim3((unsigned)tiles), dim3(TS), 0, stream, d_indptr, indptr_is64,
+                       n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
+    FGL_CHECK_LAUNCH("sample_degree_kernel");
+    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds,
+                                stream);
+    if (rc != FGL_OK) return rc;
+    const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
+    hipLaunchKernelGGL(sample_edges_kernel<TS>, dim3((unsigned)tiles), dim3(TS), lds, stream, d_indices, d_seeds,
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,
+                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr);
+    FGL_CHECK_LAUNCH("sample_edges_kernel");
+    return FGL_OK;
+}
+
+int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                  const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                  uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
+                  int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws, size_t ws_bytes,
+                  hipStream_t stream)
+{
+    FGL_REQUIRE(n_seeds_max >= 0 && n_nodes >= 0, "sample_node: negative size");
+    FGL_REQUIRE(fanout >= 1 && fanout <= FGL_MAX_FANOUT, "sample_node: fanout %d outside [1, %d]", fanout, FGL_MAX_FANOUT);
+    FGL_REQUIRE(n_seeds_max * (int64_t)fanout <= 0x7FFFFFFF, "sample_node: %lld seeds x fanout %d overflows int32 edge offsets",
+                (long long)n_seeds_max, fanout);
+    FGL_REQUIRE(d_block_ptr != nullptr, "sample_node: null block_ptr");
+    FGL_REQUIRE(n_seeds_max == 0 || (d_indptr && d_indices && d_seeds && d_src_out), "sample_node: null pointer");
+    if (d_ws == nullptr || ws_bytes < sample_workspace_bytes(n_seeds_max, fanout)) {
+        set_error("sample_node: workspace too small (%zu < %zu)", ws_bytes, sample_workspace_bytes(n_seeds_max, fanout));
+        return FGL_ERR_WORKSPACE;
+    }
+    if (tile_seeds_for(fanout) == 256)
+        return launch_sample_ts<256>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
+                                     rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status,
+                                     d_ws, stream);
+    return launch_sample_ts<64>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
+                                rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws,
+                                stream);
+}
+
+}  // namespace fgl
+
+using namespace fgl;
+
+FGL_EXPORT size_t fgl_sample_workspace_bytes(int64_t n_seeds_max, int fanout)
+{
+    if (n_seeds_max < 0 || fanout < 1) return 0;
+    return sample_workspace_bytes(n_seeds_max, fanout);
+}
+
+FGL_EXPORT int fgl_sample_node(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                               const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                               uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
+                               int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws,
+                               size_t ws_bytes, void* stream)
+{
+    return launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, rng_seed,
+                         stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws, ws_bytes,
+                         as_stream(stream));
+}

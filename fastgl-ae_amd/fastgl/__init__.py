@@ -1,0 +1,41 @@
+"""``fastgl`` -- MI355X (gfx950) implementation of FastGL's hot path, importable under the
+name of the reference's extension module so that ``import fastgl`` in the reference's
+sampler and layer code resolves to it.
+
+Operators with the reference's signatures: ``sample_node``, ``transfer_edge_id``, ``cal_deg``,
+``exclusive_sum``, ``forward_gcn``, ``backward_gcn``, ``forwaed_gin`` (sic), ``backward_gin``.
+Everything runs in hand-written HIP kernels behind ``libfastgl_hip.so``; there is no CPU path.
+"""
+from ._lib import LIB_PATH, build, lib  # noqa: F401
+from .ops import (  # noqa: F401
+    BlocksPlan,
+    aggregate,
+    backward_gat,
+    backward_gcn,
+    backward_gin,
+    block_transpose,
+    cal_deg,
+    exclusive_sum,
+    forwaed_gin,
+    forward_gat,
+    forward_gcn,
+    manual_seed,
+    rmat_keys,
+    sample_blocks_fused,
+    sample_node,
+    table_size,
+    transfer_edge_id,
+)
+from .sampler import Block, FusedMapSampler  # noqa: F401
+from .conv import (  # noqa: F401
+    GCN,
+    GIN,
+    SAGE,
+    GCNConv,
+    GINConv,
+    MA_Function,
+    MA_Function_GIN,
+    MA_Function_Mean,
+    SAGEConv,
+)
+from . import graph  # noqa: F401

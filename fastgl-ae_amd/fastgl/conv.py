@@ -1,0 +1,234 @@
+"""GNN layers over the memory-aware aggregation operators, with the class names, call
+signatures and autograd wiring of the reference's GraphConv.py (MA_Function, GCNConv, GCN,
+MA_Function_GIN, GINConv, GIN; GraphConv.py:19-195), plus a mean aggregator (GraphSAGE),
+which the reference's benchmark configurations name but its kernels do not provide.
+
+The reference's quirks are kept where they define results: weights are drawn from
+U(-1/sqrt(out), 1/sqrt(out)) (GraphConv.py:52-55), dropout sits between layers, no activation
+is applied by GCN / GIN (the ``activation`` argument is ignored, GraphConv.py:69,86-99), the
+backward of GCN receives (dst_norm, src_norm) in the slots the extension calls
+(src_norm_degs, dst_norm_degs) (GraphConv.py:37), and destination rows without edges pass
+their input through in the forward pass and receive no gradient from it.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import nn
+
+from . import ops
+from .sampler import Block
+
+
+def _block_csr(graph):
+    """(edge_ptr, src_edges, raw_dst_degs) of a block.  A ``Block`` carries its CSR; any other
+    object with ``edges()`` goes through cal_deg + exclusive_sum like GraphConv.py:93-98."""
+    dst_nodes = graph.num_dst_nodes()
+    if isinstance(graph, Block):
+        return graph.edge_ptr, graph.src_local, graph.in_degrees()
+    raw = ops.cal_deg(graph.edges()[1].int(), dst_nodes)
+    return ops.exclusive_sum(raw), graph.edges()[0].int(), raw
+
+
+class MA_Function(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat, weight, neighbor_num,
+                transposed=None):
+        ctx.save_for_backward(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat)
+        ctx.transposed = transposed
+        return ops.forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, weight, neighbor_num,
+                               dst_nodes)[0]
+
+    @staticmethod
+    def backward(ctx, d_input):
+        edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat = ctx.saved_tensors
+        d_input = d_input.contiguous()
+        if ctx.transposed is None:
+            d_x, d_w = ops.backward_gcn(edge_ptr, src_edges, dst_norm_degs, src_norm_degs, d_input, weight, input_feat)
+        else:  # same arithmetic, with the block's cached transpose
+            t_ptr, t_idx = ctx.transposed
+            g = ops.aggregate(t_ptr, t_idx, d_input, mode="gcn", zero_policy="zeros", row_norm=src_norm_degs,
+                              col_norm=dst_norm_degs, n_rows=int(input_feat.size(0)))
+            d_x = torch.mm(g, weight.transpose(0, 1))
+            d_w = torch.mm(input_feat.transpose(0, 1), g)
+        return None, None, None, None, None, d_x, d_w, None, None
+
+
+class _Conv(nn.Module):
+    def __init__(self, input_dim, output_dim, weight=False):
+        super().__init__()
+        if weight:
+            self.weights = nn.Parameter(torch.randn(input_dim, output_dim))
+        else:
+            self.weights = self.register_parameter('weight', None)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.weights is not None:
+            stdv = 1. / math.sqrt(self.weights.size(1))
+            self.weights.data.uniform_(-stdv, stdv)
+
+    def _weight(self):
+        if self.weights is None:
+            raise RuntimeError("layer was built with weight=False")
+        return self.weights
+
+
+class GCNConv(_Conv):
+    def forward(self, edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat, neighbor_num,
+                transposed=None):
+        return MA_Function.apply(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat,
+                                 self._weight(), neighbor_num, transposed)
+
+
+def _stack(conv, in_feats, n_hidden, n_classes, n_layers, weight):
+    layers = nn.ModuleList()
+    layers.append(conv(in_feats, n_hidden, weight=weight))
+    for _ in range(1, n_layers - 1):
+        layers.append(conv(n_hidden, n_hidden, weight=weight))
+    layers.append(conv(n_hidden, n_classes, weight=weight))
+    return layers
+
+
+class GCN(nn.Module):
+    def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, weight, dropout):
+        super().__init__()
+        self.layers = _stack(GCNConv, in_feats, n_hidden, n_classes, n_layers, weight)
+        self.dropout = nn.Dropout(p=dropout)
+
+    def forward(self, blocks, features, neighbor_list=[5, 10, 15]):
+        h = features
+        for i, layer in enumerate(self.layers):
+            if i != 0:
+                h = self.dropout(h)
+            graph = blocks[i]
+            dst_nodes = graph.num_dst_nodes()
+            edge_ptr, src_edges, raw_dst_norm_degs = _block_csr(graph)
+            if isinstance(graph, Block):
+                src_norm_degs = graph.out_degrees().clamp(min=1)
+                transposed = graph.transposed() if torch.is_grad_enabled() else None
+            else:
+                src_norm_degs = ops.cal_deg(src_edges, graph.num_src_nodes()).clamp(min=1)
+                transposed = None
+            dst_norm_degs = raw_dst_norm_degs.clamp(min=1)
+            h = layer(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, h, neighbor_list[i], transposed)
+        return h
+
+
+class MA_Function_GIN(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, edge_ptr, src_edges, dst_nodes, input_feat, weight, neighbor_num, transposed=None):
+        X_prime, tmp = ops.forwaed_gin(edge_ptr, src_edges, input_feat, weight, neighbor_num, dst_nodes)
+        ctx.src_nodes = input_feat.size(0)
+        ctx.neighbor_num = neighbor_num
+        ctx.transposed = transposed
+        ctx.save_for_backward(edge_ptr, src_edges, weight, tmp)
+        return X_prime
+
+    @staticmethod
+    def backward(ctx, d_input):
+        edge_ptr, src_edges, weight, tmp = ctx.saved_tensors
+        d_input = d_input.contiguous()
+        if ctx.transposed is None:
+            d_x, d_w = ops.backward_gin(edge_ptr, src_edges, d_input, weight, tmp, ctx.src_nodes)
+        else:
+            t_ptr, t_idx = ctx.transposed
+            d_tmp = torch.mm(d_input, weight.transpose(0, 1))
+            d_w = torch.mm(tmp.transpose(0, 1), d_input)
+            d_x = ops.aggregate(t_ptr, t_idx, d_tmp, mode="sum", zero_policy="zeros", n_rows=int(ctx.src_nodes))
+        return None, None, None, d_x, d_w, None, None
+
+
+class GINConv(_Conv):
+    def forward(self, edge_ptr, src_edges, dst_nodes, input_feat, neighbor_num, transposed=None):
+        return MA_Function_GIN.apply(edge_ptr, src_edges, dst_nodes, input_feat, self._weight(), neighbor_num, transposed)
+
+
+class GIN(nn.Module):
+    def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, weight, dropout):
+        super().__init__()
+        self.layers = _stack(GINConv, in_feats, n_hidden, n_classes, n_layers, weight)
+        self.dropout = nn.Dropout(p=dropout)
+
+    def forward(self, blocks, features, neighbor_list=[5, 10, 15]):
+        h = features
+        for i, layer in enumerate(self.layers):
+            if i != 0:
+                h = self.dropout(h)
+            graph = blocks[i]
+            dst_nodes = graph.num_dst_nodes()
+            edge_ptr, src_edges, _ = _block_csr(graph)
+            transposed = graph.transposed() if isinstance(graph, Block) and torch.is_grad_enabled() else None
+            h = layer(edge_ptr, src_edges, dst_nodes, h, neighbor_list[i], transposed)
+        return h
+
+
+# ---------------------------------------------------------------------------------------
+# mean aggregation (GraphSAGE-mean)
+# ---------------------------------------------------------------------------------------
+class MA_Function_Mean(torch.autograd.Function):
+    """``out[d] = mean of feat[src] over the edges into d`` (zeros if there are none).
+    ``indices`` may hold block-local ids (``feat`` = the block's source rows) or graph ids
+    (``feat`` = the whole resident feature table: the input-row gather fused into the first
+    layer).  The gradient w.r.t. ``feat`` is produced only in the block-local form."""
+
+    @staticmethod
+    def forward(ctx, block, feat, use_global):
+        indices = block.src_global if use_global else block.src_local
+        ctx.block = block
+        ctx.use_global = use_global
+        ctx.n_src = block.num_src_nodes()
+        return ops.aggregate(block.edge_ptr, indices, feat, mode="mean", zero_policy="zeros", n_rows=block.num_dst_nodes())
+
+    @staticmethod
+    def backward(ctx, d_out):
+        if ctx.use_global or not ctx.needs_input_grad[1]:
+            return None, None, None
+        block = ctx.block
+        t_ptr, t_idx = block.transposed()
+        d_feat = ops.aggregate(t_ptr, t_idx, d_out.contiguous(), mode="colmean", zero_policy="zeros",
+                               col_norm=block.in_degrees().contiguous(), n_rows=ctx.n_src)
+        return None, d_feat, None
+
+
+class SAGEConv(nn.Module):
+    """``h_dst W_self + mean(h_src) W_neigh + b`` (the mean aggregator of GraphSAGE)."""
+
+    def __init__(self, input_dim, output_dim, bias=True):
+        super().__init__()
+        self.fc_self = nn.Linear(input_dim, output_dim, bias=False)
+        self.fc_neigh = nn.Linear(input_dim, output_dim, bias=bias)
+
+    def forward(self, block, feat_src, feat_dst=None, use_global=False):
+        h_neigh = MA_Function_Mean.apply(block, feat_src, use_global)
+        if feat_dst is None:
+            feat_dst = feat_src[:block.num_dst_nodes()]
+        return self.fc_self(feat_dst) + self.fc_neigh(h_neigh)
+
+
+class SAGE(nn.Module):
+    def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation=torch.relu, dropout=0.0):
+        super().__init__()
+        dims = [in_feats] + [n_hidden] * (n_layers - 1) + [n_classes]
+        self.layers = nn.ModuleList(SAGEConv(dims[i], dims[i + 1]) for i in range(n_layers))
+        self.activation = activation
+        self.dropout = nn.Dropout(p=dropout)
+
+    def forward(self, blocks, features, input_nodes=None):
+        """``features``: the rows of the input nodes, or -- with ``input_nodes`` given -- the
+        whole feature table, in which case the first layer gathers straight from it."""
+        h = features
+        for i, (layer, block) in enumerate(zip(self.layers, blocks)):
+            if i == 0 and input_nodes is not None:
+                if block.src_global is None:
+                    raise RuntimeError("the outermost block does not carry graph ids")
+                dst_ids = input_nodes[:block.num_dst_nodes()].long()
+                h = layer(block, features, feat_dst=features.index_select(0, dst_ids), use_global=True)
+            else:
+                h = layer(block, h)
+            if i != len(self.layers) - 1:
+                if self.activation is not None:
+                    h = self.activation(h)
+                h = self.dropout(h)
+        return h

@@ -1,0 +1,381 @@
+"""The operator functions of the reference's ``fastgl`` extension module, with the same
+names, positional arguments, return lists and error type (cuda_operators/aggregate_acc.cpp:
+601-621 lists them; only the ones its Python code calls are provided), implemented over
+the HIP C ABI.  Extensions that the reference does not have (mean aggregation, the
+transposed block, the all-hops sampler) follow at the end.
+
+Index tensors are int32 and must be contiguous device tensors (``RuntimeError`` otherwise,
+as the reference's CHECK_INPUT, aggregate_acc.cpp:4-6); ``edge_ptr`` of the full graph may
+also be int64.  Features are fp32 or bf16.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib as L
+
+_rng_state = {"seed": 0, "calls": 0}
+
+
+def manual_seed(seed: int) -> None:
+    """Seed of the sampler's Philox streams; also resets the per-call stream counter.
+    (The reference's picks come from one constant stream, sample.cu:70.)"""
+    _rng_state["seed"] = int(seed) & 0xFFFFFFFFFFFFFFFF
+    _rng_state["calls"] = 0
+
+
+def _check_input(t, name, dtypes=None):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError("%s must be a tensor" % name)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+    if dtypes is not None and t.dtype not in dtypes:
+        raise RuntimeError("%s must have dtype in %s, got %s" % (name, [str(d) for d in dtypes], t.dtype))
+
+
+def _same_device(*tensors):
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t is not None and t.device != dev:
+            raise RuntimeError("all tensors must live on the same device")
+    return dev
+
+
+_I32 = (torch.int32,)
+_PTR = (torch.int32, torch.int64)
+_FEAT = (torch.float32, torch.bfloat16)
+
+
+def _raise_status(bits: int, where: str):
+    if bits:
+        raise RuntimeError("fastgl.%s: %s" % (where, L.status_message(bits)))
+
+
+# ---------------------------------------------------------------------------------------
+# drop-in operators
+# ---------------------------------------------------------------------------------------
+def sample_node(src_edges, dst_edges, edge_ptr, seed_nodes, dst_nodes, neighbor_num):
+    """fastgl.sample_node (aggregate_acc.cpp:491-512): ``-> [src_out, dst_out, edges_num]``.
+
+    ``src_edges`` is the CSR ``indices`` of the in-neighbour graph, ``edge_ptr`` its
+    ``indptr``; ``dst_edges`` is accepted and, as in the reference kernels, never read.
+    Outputs hold global ids, each seed's edges contiguous, seeds in order.
+    """
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(dst_edges, "dst_edges")
+    _check_input(edge_ptr, "edge_ptr", _PTR)
+    _check_input(seed_nodes, "seed_nodes", _I32)
+    dev = _same_device(src_edges, edge_ptr, seed_nodes)
+    n_seeds = int(seed_nodes.size(0))
+    dst_nodes = int(dst_nodes)
+    fanout = int(neighbor_num)
+    if dst_nodes < n_seeds:
+        raise RuntimeError("dst_nodes (%d) is smaller than the number of seeds (%d)" % (dst_nodes, n_seeds))
+    lib = L.lib()
+    with torch.cuda.device(dev):
+        src_out = torch.empty(max(dst_nodes * fanout, 1), dtype=torch.int32, device=dev)
+        dst_out = torch.empty(max(dst_nodes * fanout, 1), dtype=torch.int32, device=dev)
+        block_ptr = torch.empty(n_seeds + 1, dtype=torch.int32, device=dev)
+        meta = torch.zeros(2, dtype=torch.int32, device=dev)  # [edge count, status]
+        ws_bytes = lib.fgl_sample_workspace_bytes(n_seeds, fanout)
+        ws = L.workspace(ws_bytes, dev)
+        stream_id = _rng_state["calls"] & 0xFFFFFFFF
+        _rng_state["calls"] += 1
+        L.check(lib.fgl_sample_node(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(src_edges),
+                                    int(edge_ptr.size(0)) - 1, L.ptr(seed_nodes), n_seeds, None, fanout,
+                                    _rng_state["seed"], stream_id, L.ptr(src_out), L.ptr(dst_out), L.ptr(block_ptr),
+                                    meta.data_ptr(), meta.data_ptr() + 4, L.ptr(ws), ws.numel(), L.stream_handle()))
+        n_edges, status = meta.tolist()  # the host read-back the reference also does (sample.cu:202)
+    _raise_status(status, "sample_node")
+    edges_num = meta[:1]
+    out = [src_out[:n_edges], dst_out[:n_edges], edges_num]
+    sample_node.last_block_ptr = block_ptr  # CSR offsets of the block just sampled
+    return out
+
+
+sample_node.last_block_ptr = None
+
+
+def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_items, unique_num, edge_nums):
+    """fastgl.transfer_edge_id (aggregate_acc.cpp:467-489, id_map.cu:386-493): the fused
+    id-map.  Rewrites ``src_edges`` / ``dst_edges`` in place to local ids and returns
+    ``[src_edges, dst_edges, uniq]`` with ``uniq = cat(dst_edges_unique, new source ids)``.
+    New ids are numbered in first-occurrence order."""
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(dst_edges, "dst_edges", _I32)
+    _check_input(dst_edges_unique, "dst_edges_unique", _I32)
+    dev = _same_device(src_edges, dst_edges, dst_edges_unique)
+    n_dst = int(dst_nodes)
+    n_edges = int(edge_nums)
+    if n_dst > dst_edges_unique.size(0):
+        raise RuntimeError("dst_nodes (%d) exceeds len(dst_edges_unique) (%d)" % (n_dst, dst_edges_unique.size(0)))
+    if n_edges > src_edges.size(0) or n_edges > dst_edges.size(0):
+        raise RuntimeError("edge_nums (%d) exceeds the edge arrays" % n_edges)
+    if int(total_items) - n_dst != n_edges:
+        raise RuntimeError("total_items - dst_nodes must equal edge_nums (id_map.cu:308)")
+    lib = L.lib()
+    max_new = max(0, min(int(unique_num), n_edges))
+    capacity = n_dst + max_new
+    slots = lib.fgl_idmap_slots(capacity)
+    with torch.cuda.device(dev):
+        table = _table(slots, dev)
+        uniq = torch.empty(max(capacity, 1), dtype=torch.int32, device=dev)
+        meta = torch.zeros(2, dtype=torch.int32, device=dev)  # [n_total, status]
+        ws_bytes = lib.fgl_idmap_map_src_workspace_bytes(n_edges)
+        ws = L.workspace(ws_bytes, dev)
+        st = L.stream_handle()
+        status_ptr = meta.data_ptr() + 4
+        L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+        L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dst_edges_unique), n_dst, None, L.ptr(uniq),
+                                         status_ptr, st))
+        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(src_edges), L.ptr(src_edges), n_edges, None, n_dst,
+                                      None, meta.data_ptr(), L.ptr(uniq), capacity, L.IDMAP_ORDERED, status_ptr,
+                                      L.ptr(ws), ws.numel(), st))
+        L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(dst_edges), n_edges, None, status_ptr, st))
+        n_total, status = meta.tolist()  # host read-back, as id_map.cu:454,491
+    _raise_status(status, "transfer_edge_id")
+    return [src_edges, dst_edges, uniq[:n_total]]
+
+
+_tables = {}
+
+
+def _table(slots: int, dev) -> torch.Tensor:
+    """Hash-table storage, cached per (device, stream) and grown on demand (the reference
+    cudaMallocs, memsets and cudaFrees one per call, id_map.cu:45-59)."""
+    key = (torch.device(dev).index, L.stream_handle())
+    t = _tables.get(key)
+    if t is None or t.numel() < slots:
+        t = torch.empty(int(slots), dtype=torch.int64, device=dev)
+        _tables[key] = t
+    return t
+
+
+def cal_deg(edges, nodes_num):
+    """fastgl.cal_deg (aggregate_acc.cpp:522-529): int32 histogram of ``edges`` over ``nodes_num`` bins."""
+    _check_input(edges, "edges", _I32)
+    n = int(nodes_num)
+    dev = edges.device
+    with torch.cuda.device(dev):
+        deg = torch.empty(max(n, 1), dtype=torch.int32, device=dev)[:n]
+        L.check(L.lib().fgl_cal_deg(L.ptr(edges), int(edges.numel()), None, L.ptr(deg), n, L.stream_handle()))
+    return deg
+
+
+def exclusive_sum(in_degs):
+    """fastgl.exclusive_sum (aggregate_acc.cpp:514-520): ``len+1`` exclusive prefix sums (int32)."""
+    _check_input(in_degs, "in_degs", _I32)
+    n = int(in_degs.numel())
+    dev = in_degs.device
+    lib = L.lib()
+    with torch.cuda.device(dev):
+        out = torch.empty(n + 1, dtype=torch.int32, device=dev)
+        ws = L.workspace(lib.fgl_exclusive_sum_workspace_bytes(n), dev)
+        L.check(lib.fgl_exclusive_sum_i32(L.ptr(in_degs), n, None, L.ptr(out), L.ptr(ws), ws.numel(), L.stream_handle()))
+    return out
+
+
+def forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, weight, neighbor_num, dst_nodes):
+    """fastgl.forward_gcn (aggregate_acc.cpp:133-160): ``[A_norm (X W)]`` with
+    ``A_norm[d, s] = 1/sqrt(dst_norm[d]) * 1/sqrt(src_norm[s])``; a dst row without edges
+    passes ``(X W)[d]`` through (aggregate_acc_kernel.cu:307-309)."""
+    for t, n in ((edge_ptr, "edge_ptr"), (src_edges, "src_edges"), (src_norm_degs, "src_norm_degs"),
+                 (dst_norm_degs, "dst_norm_degs")):
+        _check_input(t, n, _I32)
+    _check_input(input_feat, "input_feat", _FEAT)
+    _check_input(weight, "weight", _FEAT)
+    tmp = torch.mm(input_feat, weight)
+    out = aggregate(edge_ptr, src_edges, tmp, mode="gcn", zero_policy="self", row_norm=dst_norm_degs,
+                    col_norm=src_norm_degs, n_rows=int(dst_nodes))
+    return [out]
+
+
+def backward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, d_input, weight, input_feat):
+    """fastgl.backward_gcn (aggregate_acc.cpp:349-376): ``[d_x, d_w]``.
+
+    Positional meaning as in the reference kernel (aggregate_acc_kernel.cu:494,509): the
+    third argument is indexed by destination id and the fourth by source id -- the caller
+    passes ``(dst_norm, src_norm)`` there (GraphConv.py:37)."""
+    by_dst, by_src = src_norm_degs, dst_norm_degs
+    for t, n in ((edge_ptr, "edge_ptr"), (src_edges, "src_edges"), (by_dst, "src_norm_degs"), (by_src, "dst_norm_degs")):
+        _check_input(t, n, _I32)
+    _check_input(d_input, "d_input", _FEAT)
+    _check_input(weight, "weight", _FEAT)
+    _check_input(input_feat, "input_feat", _FEAT)
+    n_src = int(input_feat.size(0))
+    n_dst = int(d_input.size(0))
+    t_ptr, t_idx = block_transpose(edge_ptr, src_edges, n_dst, n_src)
+    g = aggregate(t_ptr, t_idx, d_input, mode="gcn", zero_policy="zeros", row_norm=by_src, col_norm=by_dst, n_rows=n_src)
+    d_x = torch.mm(g, weight.transpose(0, 1))
+    d_w = torch.mm(input_feat.transpose(0, 1), g)
+    return [d_x, d_w]
+
+
+def forwaed_gin(edge_ptr, src_edges, input_feat, weight, neighbor_num, dst_nodes):
+    """fastgl.forwaed_gin (sic; aggregate_acc.cpp:173-199, exported at :613): ``[tmp W, tmp]``
+    with ``tmp[d] = sum of X[s] over the edges into d`` (``X[d]`` if there are none)."""
+    _check_input(edge_ptr, "edge_ptr", _I32)
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(input_feat, "input_feat", _FEAT)
+    _check_input(weight, "weight", _FEAT)
+    tmp = aggregate(edge_ptr, src_edges, input_feat, mode="sum", zero_policy="self", n_rows=int(dst_nodes))
+    return [torch.mm(tmp, weight), tmp]
+
+
+def backward_gin(edge_ptr, src_edges, d_input, weight, input_feat, src_nodes):
+    """fastgl.backward_gin (aggregate_acc.cpp:387-409): ``[d_x, d_w]``; ``input_feat`` is the
+    ``tmp`` that forwaed_gin returned."""
+    _check_input(edge_ptr, "edge_ptr", _I32)
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(d_input, "d_input", _FEAT)
+    _check_input(weight, "weight", _FEAT)
+    _check_input(input_feat, "input_feat", _FEAT)
+    d_tmp = torch.mm(d_input, weight.transpose(0, 1))
+    d_w = torch.mm(input_feat.transpose(0, 1), d_input)
+    n_dst = int(d_input.size(0))
+    t_ptr, t_idx = block_transpose(edge_ptr, src_edges, n_dst, int(src_nodes))
+    d_x = aggregate(t_ptr, t_idx, d_tmp, mode="sum", zero_policy="zeros", n_rows=int(src_nodes))
+    return [d_x, d_w]
+
+
+def forward_gat(*args, **kwargs):
+    raise NotImplementedError("fastgl.forward_gat: attention-weighted aggregation is not part of this library")
+
+
+def backward_gat(*args, **kwargs):
+    raise NotImplementedError("fastgl.backward_gat: attention-weighted aggregation is not part of this library")
+
+
+# ---------------------------------------------------------------------------------------
+# extensions
+# ---------------------------------------------------------------------------------------
+_MODES = {"sum": L.AGG_SUM, "mean": L.AGG_MEAN, "gcn": L.AGG_GCN, "colmean": L.AGG_COLMEAN}
+_ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
+
+
+def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
+              out=None):
+    """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
+    accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean;
+    ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``."""
+    _check_input(indptr, "indptr", _I32)
+    _check_input(indices, "indices", _I32)
+    if not isinstance(feat, torch.Tensor) or not feat.is_cuda:
+        raise RuntimeError("feat must be a CUDA tensor")
+    if feat.dim() != 2 or feat.stride(1) != 1 or feat.dtype not in _FEAT:
+        raise RuntimeError("feat must be a 2-D fp32/bf16 tensor with unit column stride")
+    if row_norm is not None:
+        _check_input(row_norm, "row_norm", _I32)
+    if col_norm is not None:
+        _check_input(col_norm, "col_norm", _I32)
+    dev = _same_device(indptr, indices, feat, row_norm, col_norm)
+    n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
+    if n < 0 or n > indptr.numel() - 1:
+        raise RuntimeError("n_rows (%d) does not match indptr (%d entries)" % (n, indptr.numel()))
+    m = _MODES[mode]
+    z = _ZERO[zero_policy]
+    if z == L.ZERO_COPY_SELF and n > feat.size(0):
+        raise RuntimeError("zero_policy 'self' needs feat to have a row for every output row")
+    D = int(feat.size(1))
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty((n, D), dtype=feat.dtype, device=dev)
+        elif out.shape != (n, D) or out.dtype != feat.dtype or out.stride(1) != 1 or not out.is_cuda:
+            raise RuntimeError("out has the wrong shape, dtype or layout")
+        if n > 0:
+            L.check(L.lib().fgl_aggregate(L.ptr(indptr), L.ptr(indices), n, None, L.ptr(feat), int(feat.stride(0)), D,
+                                          L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
+                                          L.ptr(col_norm), L.ptr(out), int(out.stride(0)), L.stream_handle()))
+    return out
+
+
+def block_transpose(indptr, indices, n_rows, n_cols):
+    """Column-major companion ``(t_indptr[n_cols+1], t_indices[nnz])`` of a block CSR."""
+    _check_input(indptr, "indptr", _I32)
+    _check_input(indices, "indices", _I32)
+    dev = _same_device(indptr, indices)
+    n_rows, n_cols = int(n_rows), int(n_cols)
+    nnz = int(indices.numel())
+    lib = L.lib()
+    with torch.cuda.device(dev):
+        t_ptr = torch.empty(n_cols + 1, dtype=torch.int32, device=dev)
+        t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
+        ws = L.workspace(lib.fgl_block_transpose_workspace_bytes(n_cols, nnz), dev)
+        L.check(lib.fgl_block_transpose(L.ptr(indptr), L.ptr(indices), n_rows, None, n_cols, None, nnz, L.ptr(t_ptr),
+                                        L.ptr(t_idx), L.ptr(ws), ws.numel(), L.stream_handle()))
+    return t_ptr, t_idx
+
+
+def table_size(num: int, scale: int) -> int:
+    """The reference's TableSize (cuda_hashtable.cuh:27-30)."""
+    return int(L.lib().fgl_table_size(int(num), int(scale)))
+
+
+class BlocksPlan:
+    """Bounds and persistent scratch for sampling mini-batches of one shape."""
+
+    def __init__(self, n_nodes: int, n_seeds: int, hop_fanouts, device):
+        lib = L.lib()
+        self.n_nodes, self.n_seeds = int(n_nodes), int(n_seeds)
+        self.hop_fanouts = [int(f) for f in hop_fanouts]
+        self.n_hops = len(self.hop_fanouts)
+        self.device = torch.device(device)
+        self._fan = (C.c_int32 * self.n_hops)(*self.hop_fanouts)
+        cap_dst = (C.c_int64 * self.n_hops)()
+        cap_edges = (C.c_int64 * self.n_hops)()
+        cap_uniq, slots, ws_bytes = C.c_int64(), C.c_int64(), C.c_size_t()
+        L.check(lib.fgl_sample_blocks_plan(self.n_nodes, self.n_seeds, self._fan, self.n_hops, cap_dst, cap_edges,
+                                           C.byref(cap_uniq), C.byref(slots), C.byref(ws_bytes)))
+        self.cap_dst = list(cap_dst)
+        self.cap_edges = list(cap_edges)
+        self.cap_uniq, self.slots, self.ws_bytes = cap_uniq.value, slots.value, ws_bytes.value
+        self.table = torch.empty(self.slots, dtype=torch.int64, device=self.device)
+        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=self.device)
+
+
+def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
+                        keep_global=(0,)):
+    """All hops of one mini-batch in one enqueue (no host synchronisation inside).
+
+    Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
+    src_global[h] or None, counts)``; hop 0 expands the raw seeds.  ``counts`` (int32,
+    ``2*n_hops + 2``) holds the node count before each hop and after the last, then the
+    edge count of each hop, then the status word; the caller reads it once per batch.
+    ``keep_global`` lists the hops (negative = from the end) whose pre-relabel source ids are kept."""
+    _check_input(edge_ptr, "edge_ptr", _PTR)
+    _check_input(indices, "indices", _I32)
+    _check_input(seeds, "seeds", _I32)
+    dev = _same_device(edge_ptr, indices, seeds)
+    if int(seeds.numel()) != plan.n_seeds:
+        raise RuntimeError("plan was made for %d seeds, got %d" % (plan.n_seeds, seeds.numel()))
+    H = plan.n_hops
+    keep = {(h + H) % H for h in keep_global}
+    lib = L.lib()
+    with torch.cuda.device(dev):
+        uniq = torch.empty(max(plan.cap_uniq, 1), dtype=torch.int32, device=dev)
+        block_ptr = [torch.empty(plan.cap_dst[h] + 1, dtype=torch.int32, device=dev) for h in range(H)]
+        src_local = [torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev) for h in range(H)]
+        src_global = [torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev) if h in keep else None
+                      for h in range(H)]
+        counts = torch.empty(2 * H + 2, dtype=torch.int32, device=dev)
+        arr = lambda ts: (C.c_void_p * H)(*[L.ptr(t) for t in ts])
+        L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
+                                      int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H,
+                                      int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF,
+                                      L.ptr(plan.table), plan.slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
+                                      arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
+                                      L.stream_handle()))
+    return uniq, block_ptr, src_local, src_global, counts
+
+
+def rmat_keys(first_edge: int, n_edges: int, scale: int, n_nodes: int, seed: int, device) -> torch.Tensor:
+    """2*n_edges symmetrised int64 keys ``row<<32 | col`` of seeded R-MAT draws (INT64_MAX = dropped)."""
+    with torch.cuda.device(device):
+        keys = torch.empty(2 * int(n_edges), dtype=torch.int64, device=device)
+        L.check(L.lib().fgl_rmat_keys(int(first_edge), int(n_edges), int(scale), int(n_nodes),
+                                      int(seed) & 0xFFFFFFFFFFFFFFFF, L.ptr(keys), L.stream_handle()))
+    return keys

@@ -1,0 +1,173 @@
+"""Mini-batch block sampler with the interface of the reference's ``FusedMapSampler``
+(FusedMapSampler.py:27-109) -- same constructor arguments, same attributes the trainer
+fills in (``edge_src``, ``edge_dst``, ``edge_ptr``, ``nodes_num``; train_fastgl.py:240-244),
+same ``sample_blocks(g, seed_nodes) -> (input_nodes, output_nodes, blocks)`` -- without DGL:
+a block is the light ``Block`` below instead of a ``DGLBlock``.
+
+Two paths produce identical blocks:
+  * ``fused=True`` (default): all hops in one enqueue of the C ABI's ``fgl_sample_blocks``;
+    one host read-back per mini-batch;
+  * ``fused=False``: the reference's per-hop loop, call for call, through the drop-in
+    operators ``sample_node`` and ``transfer_edge_id``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+class Block:
+    """One hop of a sampled mini-batch: a bipartite graph from ``n_src`` source nodes to
+    ``n_dst`` destination nodes (the first ``n_dst`` source nodes *are* the destination
+    nodes), stored as a CSR over destination rows: ``edge_ptr`` int32[n_dst+1],
+    ``src_local`` int32[E].  ``src_global`` (optional) holds the same edges with graph ids."""
+
+    def __init__(self, edge_ptr, src_local, n_src, n_dst, src_global=None):
+        self.edge_ptr = edge_ptr
+        self.src_local = src_local
+        self._n_src = int(n_src)
+        self._n_dst = int(n_dst)
+        self.src_global = src_global
+        self._dst_local = None
+        self._transposed = None
+        self._src_deg = None
+
+    # -- the part of the DGLBlock interface that the reference's model code uses -------------
+    def num_src_nodes(self):
+        return self._n_src
+
+    def num_dst_nodes(self):
+        return self._n_dst
+
+    def num_edges(self):
+        return int(self.src_local.numel())
+
+    def edges(self):
+        """``(src_local, dst_local)`` as COO, grouped by destination in row order."""
+        if self._dst_local is None:
+            deg = (self.edge_ptr[1:] - self.edge_ptr[:-1]).long()
+            rows = torch.arange(self._n_dst, device=self.edge_ptr.device, dtype=torch.int32)
+            self._dst_local = torch.repeat_interleave(rows, deg, output_size=self.num_edges())
+        return self.src_local, self._dst_local
+
+    def int(self):
+        return self
+
+    def to(self, device):
+        if torch.device(device) != self.edge_ptr.device:
+            raise RuntimeError("Block.to: blocks live on the device they were sampled on")
+        return self
+
+    # -- what this library adds ---------------------------------------------------------
+    def in_degrees(self):
+        return self.edge_ptr[1:] - self.edge_ptr[:-1]
+
+    def out_degrees(self):
+        if self._src_deg is None:
+            self._src_deg = ops.cal_deg(self.src_local, self._n_src)
+        return self._src_deg
+
+    def transposed(self):
+        """``(t_ptr int32[n_src+1], t_dst int32[E])``: for each source node the destination
+        rows it feeds (built on first use, kept for the backward pass)."""
+        if self._transposed is None:
+            self._transposed = ops.block_transpose(self.edge_ptr, self.src_local, self._n_dst, self._n_src)
+        return self._transposed
+
+    def __repr__(self):
+        return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())
+
+
+class FusedMapSampler:
+    def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
+                 prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0):
+        if mask is not None and prob is not None:
+            raise ValueError('Mask and probability arguments are mutually exclusive. '
+                             'Consider multiplying the probability with the mask to achieve the same goal.')
+        if prob is not None or mask is not None:
+            raise NotImplementedError("weighted / masked sampling is not part of this library")
+        if edge_dir != 'in':
+            raise NotImplementedError("only in-neighbour sampling (edge_dir='in'), as in the reference")
+        if replace:
+            raise NotImplementedError("sampling is without replacement")
+        self.fanouts = list(fanouts)
+        self.edge_dir = edge_dir
+        self.replace = replace
+        self.output_device = output_device
+        self.fused = fused
+        self.rng_seed = int(rng_seed)
+        self.batches = 0
+        self.nodes_num = 0
+        self.edge_src = None  # CSR indices (source id of every edge, edges sorted by destination)
+        self.edge_dst = None  # unused by the kernels; kept because the reference's trainer sets it
+        self.edge_ptr = None  # CSR indptr (int32 or int64)
+        self.output_nodes = None
+        self._plans = {}
+
+    def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
+        self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
+        self.nodes_num = int(edge_ptr.numel()) - 1 if nodes_num is None else int(nodes_num)
+        return self
+
+    # -------------------------------------------------------------------------------------
+    def sample_blocks(self, g, seed_nodes, exclude_eids=None):
+        """``-> (input_nodes, output_nodes, blocks)``; ``blocks[0]`` is the outermost hop and
+        was sampled with ``fanouts[0]`` (seeds are expanded with ``fanouts[-1]`` first,
+        FusedMapSampler.py:72).  ``g`` is ignored, as in the reference (train_fastgl.py:245-246)."""
+        if self.edge_ptr is None or self.edge_src is None:
+            raise RuntimeError("FusedMapSampler: edge_ptr / edge_src are not set")
+        self.output_nodes = seed_nodes
+        seeds = seed_nodes.to(device=self.edge_src.device, dtype=torch.int32).contiguous()
+        stream_base = (self.batches * 64) & 0xFFFFFFFF
+        self.batches += 1
+        if self.fused:
+            return self._sample_fused(seeds, stream_base)
+        return self._sample_layerwise(seeds, stream_base)
+
+    def _sample_fused(self, seeds, stream_base):
+        hop_fanouts = list(reversed(self.fanouts))
+        H = len(hop_fanouts)
+        key = (int(seeds.numel()), tuple(hop_fanouts), self.nodes_num, seeds.device)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = ops.BlocksPlan(self.nodes_num, int(seeds.numel()), hop_fanouts, seeds.device)
+            self._plans = {key: plan}
+        uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
+                                                                   self.rng_seed, stream_base, keep_global=(H - 1,))
+        c = counts.tolist()  # the one host synchronisation of the mini-batch
+        if c[2 * H + 1]:
+            ops._raise_status(c[2 * H + 1], "sample_blocks")
+        blocks = []
+        for h in range(H):
+            n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]
+            blocks.insert(0, Block(bptr[h][:n_dst + 1], src_l[h][:n_e], n_src, n_dst,
+                                   None if src_g[h] is None else src_g[h][:n_e]))
+        return uniq[:c[H]], seeds, blocks
+
+    def _sample_layerwise(self, seeds, stream_base):
+        # the reference loop (FusedMapSampler.py:72-107), one drop-in call per step
+        raw_seed_nodes = seeds.clone()
+        seed_nodes_acc = seeds
+        blocks = []
+        dst_nodes = int(seeds.size(0))
+        saved = dict(ops._rng_state)
+        ops._rng_state["seed"] = self.rng_seed
+        try:
+            for block_index, fanout in enumerate(reversed(self.fanouts)):
+                ops._rng_state["calls"] = stream_base + block_index
+                src_out, dst_out, _ = ops.sample_node(self.edge_src, self.edge_dst if self.edge_dst is not None else self.edge_src,
+                                                      self.edge_ptr, seed_nodes_acc, dst_nodes, fanout)
+                block_ptr = ops.sample_node.last_block_ptr
+                edge_nums = int(src_out.size(0))
+                dst_unique = raw_seed_nodes if block_index == 0 else seed_nodes_acc
+                n_dst = int(dst_unique.size(0))
+                max_src_num = min(self.nodes_num, fanout * n_dst)
+                src_global = src_out.clone() if block_index == len(self.fanouts) - 1 else None
+                src_edges, _dst_edges, seed_nodes_acc = ops.transfer_edge_id(src_out, dst_out, dst_unique, dst_nodes,
+                                                                             dst_nodes + edge_nums, max_src_num, edge_nums)
+                blocks.insert(0, Block(block_ptr, src_edges, int(seed_nodes_acc.size(0)), n_dst, src_global))
+                dst_nodes = int(seed_nodes_acc.size(0))
+        finally:
+            ops._rng_state.update(saved)
+        return seed_nodes_acc, raw_seed_nodes, blocks

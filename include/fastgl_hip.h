@@ -1,0 +1,211 @@
+/*
+ * fastgl_hip.h -- C ABI of libfastgl_hip.so, the MI355X (gfx950) implementation of
+ * FastGL's hot path: CSR neighbour sampling, the fused id-map, block-CSR helpers and
+ * memory-aware aggregation (forward and backward).
+ *
+ * Conventions
+ *   - every pointer named d_* or documented "device" is a device pointer; everything
+ *     else is a host value.  The library never allocates or frees device memory and
+ *     never synchronises: all work is enqueued on `stream` (a hipStream_t passed as
+ *     void*, NULL = the null stream) and scratch comes from a caller workspace whose
+ *     size the matching *_workspace_bytes() function returns.
+ *   - "max/count pairs": a size that is only known on the device is passed as a host
+ *     upper bound (n_max) plus a device pointer to the actual int32 count (d_n, may be
+ *     NULL meaning "exactly n_max").  Grids are sized for the bound, kernels read the
+ *     count.  This is what lets a whole mini-batch be sampled without a host sync.
+ *   - return value: FGL_OK or an FGL_ERR_* code; fgl_last_error() gives the message of
+ *     the last failing call on the calling thread.  Argument errors are detected on the
+ *     host before anything is launched.  Conditions only a kernel can see (hash table
+ *     full, output capacity exceeded, id missing from the map) set bits in a device
+ *     status word (FGL_STATUS_*), never fault, and never spin.
+ *   - index arrays are int32; graph offsets (indptr of the full graph) int32 or int64.
+ *
+ * Each entry point names the reference interface (a1bc2def6g/fastgl-ae) it stands in for.
+ */
+#ifndef FASTGL_HIP_H
+#define FASTGL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGL_ABI_VERSION 1
+
+enum fgl_error {
+    FGL_OK = 0,
+    FGL_ERR_ARG = 1,         /* bad argument (null pointer, negative size, unsupported value) */
+    FGL_ERR_WORKSPACE = 2,   /* workspace too small or misaligned */
+    FGL_ERR_HIP = 3,         /* a HIP runtime call or kernel launch failed */
+    FGL_ERR_UNSUPPORTED = 4  /* valid request outside what the kernels implement */
+};
+
+enum fgl_dtype { FGL_F32 = 0, FGL_BF16 = 1 };
+
+/* per-edge weight of fgl_aggregate (row = output row, col = gathered row) */
+enum fgl_agg_mode {
+    FGL_AGG_SUM = 0,     /* w = 1                                             (GIN)  */
+    FGL_AGG_MEAN = 1,    /* w = 1 / deg(row)                                  (SAGE) */
+    FGL_AGG_GCN = 2,     /* w = (1/sqrt(row_norm[row])) * (1/sqrt(col_norm[col]))    */
+    FGL_AGG_COLMEAN = 3  /* w = 1 / max(col_norm[col], 1)   (backward of MEAN)        */
+};
+
+/* what an output row with no entries gets */
+enum fgl_zero_policy {
+    FGL_ZERO_COPY_SELF = 0, /* X[row]  (reference forward kernels)   */
+    FGL_ZERO_ZEROS = 1      /* zeros   (backward; DGL-style mean)    */
+};
+
+/* bits of the device status word */
+#define FGL_STATUS_TABLE_FULL 1u   /* an insert found no free slot          */
+#define FGL_STATUS_UNIQ_OVERFLOW 2u /* more unique ids than uniq_capacity   */
+#define FGL_STATUS_MISSING_KEY 4u  /* a looked-up id is not in the table    */
+#define FGL_STATUS_BAD_SEED 8u     /* a seed id outside [0, n_nodes)        */
+
+#define FGL_IDMAP_ORDERED 0 /* new ids numbered by first occurrence (deterministic) */
+#define FGL_MAX_FANOUT 192
+
+int fgl_abi_version(void);
+const char* fgl_last_error(void);
+
+/* ---------------------------------------------------------------------------------
+ * exclusive_sum  -- replaces fastgl.exclusive_sum (cuda_operators/aggregate_acc.cpp:514-520,
+ * utilis.cu:17-41): out[0..n] = exclusive prefix sums of in[0..n-1], out[n] = total.
+ * `out` may alias `in` if it has room for n+1 entries.
+ * ------------------------------------------------------------------------------- */
+size_t fgl_exclusive_sum_workspace_bytes(int64_t n_max);
+int fgl_exclusive_sum_i32(const int32_t* d_in, int64_t n_max, const int32_t* d_n, int32_t* d_out,
+                          void* d_ws, size_t ws_bytes, void* stream);
+
+/* cal_deg -- replaces fastgl.cal_deg (aggregate_acc.cpp:522-529, utilis.cu:43-79):
+ * d_deg[0..n_nodes) = histogram of d_ids[0..n_ids).  d_deg is cleared by the call. */
+int fgl_cal_deg(const int32_t* d_ids, int64_t n_ids_max, const int32_t* d_n_ids, int32_t* d_deg,
+                int64_t n_nodes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * sample_node -- replaces fastgl.sample_node (aggregate_acc.cpp:491-512, sample.cu:102-203).
+ * For seed position i (node s = d_seeds[i]): k_i = min(fanout, deg(s)); d_block_ptr =
+ * exclusive scan of k (n+1 entries; this IS the indptr of the sampled block's CSR);
+ * d_src_out[block_ptr[i] + j] = j-th chosen in-neighbour (global id);
+ * d_dst_out (optional, may be NULL) = s for each of those edges.
+ * deg <= fanout copies the row in CSR order; otherwise a uniform random k-subset WITHOUT
+ * replacement (Floyd) from Philox4x32-10 keyed by (rng_seed, stream_id, i).
+ * d_n_edges_out (optional) receives the edge count as int32.
+ * d_src_out / d_dst_out need room for n_seeds_max * fanout entries.
+ * ------------------------------------------------------------------------------- */
+size_t fgl_sample_workspace_bytes(int64_t n_seeds_max, int fanout);
+int fgl_sample_node(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                    const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                    uint64_t rng_seed, uint32_t stream_id,
+                    int32_t* d_src_out, int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out,
+                    uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream);
+
+/* TableSize -- the reference's sizing rule (cuda_hashtable.cuh:27-30), evaluated in 64 bits:
+ * (largest power of two <= num) << scale.  Kept for callers that size by it. */
+int64_t fgl_table_size(int64_t num, int scale);
+
+/* ---------------------------------------------------------------------------------
+ * id-map hash table -- replaces MutableDeviceOrderedHashTable and the free functions
+ * Hash/Insert/InsertSrc/Search (id_map.cu:26-59,179-255).  8-byte slots {key, local id},
+ * power-of-two slot count, multiplicative hash, linear probing bounded by the slot count.
+ * fgl_idmap_slots(n) = slot count for at most n distinct ids (load factor <= 1/2).
+ * ------------------------------------------------------------------------------- */
+int64_t fgl_idmap_slots(int64_t max_unique);
+size_t fgl_idmap_table_bytes(int64_t slots);
+int fgl_idmap_reset(void* d_table, int64_t slots, void* stream);
+
+/* insert the destination ids: local id of d_dst_ids[i] is i (id_map.cu:259-287); the ids
+ * are also copied to d_uniq[0..n) when d_uniq != d_dst_ids.  If an id repeats, lookups
+ * return its first position. */
+int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids, int64_t n_max,
+                         const int32_t* d_n, int32_t* d_uniq, uint32_t* d_status, void* stream);
+
+/* number the new source ids and relabel the edges (id_map.cu:290-383 for the src half).
+ * n_base ids are already numbered (host value n_base, or *d_n_base when non-NULL).
+ * New ids get n_base, n_base+1, ... in order of first occurrence in d_src_in and are
+ * appended to d_uniq; d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
+ * *d_n_total_out = n_base + number of new ids. */
+size_t fgl_idmap_map_src_workspace_bytes(int64_t n_edges_max);
+int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
+                      int64_t n_edges_max, const int32_t* d_n_edges,
+                      int64_t n_base, const int32_t* d_n_base, int32_t* d_n_total_out,
+                      int32_t* d_uniq, int64_t uniq_capacity, int flags,
+                      uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream);
+
+/* relabel ids that are already in the table, in place (the dst half of
+ * transfer_edge_id_kernel, id_map.cu:377-381).  A missing id becomes -1 and sets
+ * FGL_STATUS_MISSING_KEY (the reference's Search would loop forever, id_map.cu:242-255). */
+int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,
+                     uint32_t* d_status, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * sample_blocks -- all hops of FusedMapSampler.sample_blocks (FusedMapSampler.py:63-109)
+ * in one call with no host synchronisation: per hop sample_node -> id-map, the table and
+ * the numbering persisting across hops (hop h's unique list is hop h+1's seed list).
+ * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0].
+ * (The reference lists fanouts the other way round and iterates reversed(); the caller
+ * passes them already reversed.)
+ *
+ * fgl_sample_blocks_plan fills, for the given bounds, cap_dst[h] (max seeds of hop h),
+ * cap_edges[h] (max edges of hop h), *cap_uniq (max unique ids overall), *table_slots
+ * and *ws_bytes.
+ *
+ * Outputs (device): block_ptr[h] int32[cap_dst[h]+1], src_local[h] int32[cap_edges[h]],
+ * src_global[h] int32[cap_edges[h]] or NULL; d_uniq int32[cap_uniq];
+ * d_counts int32[2*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
+ * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word.
+ * ------------------------------------------------------------------------------- */
+int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
+                           int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,
+                           int64_t* table_slots, size_t* ws_bytes);
+int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                      const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
+                      uint64_t rng_seed, uint32_t stream_base,
+                      void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
+                      int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
+                      int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * block transpose -- the column-major companion of a block CSR, which turns the
+ * reference's atomic scatter in the backward kernels (aggregate_acc_kernel.cu:467-517,
+ * 554-596) into an atomic-free gather.  d_t_indptr int32[n_cols_max+1],
+ * d_t_indices int32[n_edges_max] (row ids, unordered within a column).
+ * ------------------------------------------------------------------------------- */
+size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max);
+int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
+                        int64_t n_rows_max, const int32_t* d_n_rows,
+                        int64_t n_cols_max, const int32_t* d_n_cols, int64_t n_edges_max,
+                        int32_t* d_t_indptr, int32_t* d_t_indices,
+                        void* d_ws, size_t ws_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * aggregate -- the memory-aware aggregation kernels: replaces the device part of
+ * fastgl.forward_gcn / forwaed_gin (aggregate_acc_kernel.cu:270-331, 375-427) and, on the
+ * transposed block, of backward_gcn / backward_gin (:467-517, :554-596); adds mean.
+ *   out[r, :] = sum over e in [indptr[r], indptr[r+1]) of w(r, indices[e]) * X[indices[e], :]
+ * X: [*, D] with row stride ldx elements; out: [n_rows, D] with row stride ldo; both of
+ * `dtype` (fp32, or bf16 with fp32 accumulation).  d_row_norm / d_col_norm: int32 degree
+ * arrays as required by `mode` (else NULL).
+ * ------------------------------------------------------------------------------- */
+int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
+                  int64_t n_rows_max, const int32_t* d_n_rows,
+                  const void* d_x, int64_t ldx, int D, int dtype, int mode, int zero_policy,
+                  const int32_t* d_row_norm, const int32_t* d_col_norm,
+                  void* d_out, int64_t ldo, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * Seeded R-MAT key generator for the synthetic graphs (a=.57 b=.19 c=.19 d=.05).
+ * For draw e in [first_edge, first_edge+n_edges): writes the two symmetrised keys
+ * (row<<32 | col) of the in-neighbour CSR, or INT64_MAX twice for a self loop / an
+ * endpoint >= n_nodes.  Has no counterpart in the reference (which downloads its datasets
+ * with shell scripts); it exists so benchmark graphs are reproducible on CPU and GPU.
+ * ------------------------------------------------------------------------------- */
+int fgl_rmat_keys(int64_t first_edge, int64_t n_edges, int scale, int64_t n_nodes, uint64_t seed,
+                  int64_t* d_keys, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTGL_HIP_H */

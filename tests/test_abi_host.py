@@ -1,0 +1,97 @@
+"""The C-ABI library loads, exports every symbol the header declares, and rejects bad
+arguments on the host (no kernel is launched here: runs without a GPU)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+
+import fastgl
+from fastgl import _lib as L
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "fastgl_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fgl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared()
+    assert len(names) >= 20
+    raw = C.CDLL(L.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), n
+    assert sorted(L.SIGNATURES) == names  # the python binding covers the header, nothing else
+
+
+def test_pure_host_entry_points():
+    lib = fastgl.lib()
+    assert lib.fgl_abi_version() == 1
+    assert fastgl.table_size(40960, 2) == 131072
+    assert fastgl.table_size(8110080, 2) == 16777216
+    assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25
+    assert lib.fgl_idmap_table_bytes(1 << 25) == 8 << 25
+    assert lib.fgl_exclusive_sum_workspace_bytes(10) > 0
+
+
+def test_plan_matches_the_worst_case_table():
+    # batch 8192, hops expanded with 5, 10, 15 on the 111M-node graph
+    fan = (C.c_int32 * 3)(5, 10, 15)
+    cd, ce = (C.c_int64 * 3)(), (C.c_int64 * 3)()
+    cu, sl, ws = C.c_int64(), C.c_int64(), C.c_size_t()
+    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 8192, fan, 3, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    assert list(cd) == [8192, 49152, 540672]
+    assert list(ce) == [40960, 491520, 8110080]
+    assert cu.value == 8650752 and sl.value == 1 << 25 and ws.value > 0
+    # a small graph caps the bounds
+    L.check(fastgl.lib().fgl_sample_blocks_plan(1000, 100, fan, 3, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    assert list(cd) == [100, 600, 1100] and cu.value == 1100
+
+
+def test_argument_errors_are_reported_not_launched():
+    lib = fastgl.lib()
+    fan = (C.c_int32 * 1)(0)
+    assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, None, None, None, None) == 1
+    assert b"fanout" in lib.fgl_last_error()
+    assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
+    assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table
+    assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 8, None) == 1
+    assert b"dtype" in lib.fgl_last_error()
+    assert lib.fgl_rmat_keys(0, 10, 40, 100, 0, None, None) == 1
+
+
+def test_operator_input_checks_raise_runtime_error():
+    cpu = torch.zeros(4, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        fastgl.cal_deg(cpu, 4)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        fastgl.sample_node(cpu, cpu, cpu, cpu, 4, 2)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        fastgl.transfer_edge_id(cpu, cpu, cpu, 4, 8, 4, 4)
+    with pytest.raises(NotImplementedError):
+        fastgl.forward_gat()
+
+
+def test_sampler_front_end_without_gpu():
+    with pytest.raises(ValueError):
+        fastgl.FusedMapSampler([5], prob="p", mask="m")
+    with pytest.raises(NotImplementedError):
+        fastgl.FusedMapSampler([5], replace=True)
+    s = fastgl.FusedMapSampler([15, 10, 5])
+    with pytest.raises(RuntimeError, match="not set"):
+        s.sample_blocks(None, torch.arange(4))
+    b = fastgl.Block(torch.tensor([0, 2, 2, 5], dtype=torch.int32), torch.tensor([3, 1, 0, 2, 4], dtype=torch.int32), 5, 3)
+    src, dst = b.edges()
+    assert dst.tolist() == [0, 0, 2, 2, 2] and b.num_src_nodes() == 5 and b.num_dst_nodes() == 3 and b.num_edges() == 5
+    assert b.in_degrees().tolist() == [2, 0, 3]
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libfastgl_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        L.lib()
