@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the FastGL hot path on one MI355X:  sample -> fused id-map -> aggregate.
+
+One step = one mini-batch of the workload through the hot path with everything resident in
+HBM: all hops of neighbour sampling + id-map (one enqueue, one count read-back), then the
+aggregation kernels of a GraphSAGE-mean model over the sampled blocks -- forward for every
+block (the outermost one gathers straight from the full feature table), and, for the blocks
+whose input needs a gradient, the block transpose and the backward gather.  The dense
+layers between aggregations are library GEMMs outside this path and are not run.
+
+Prints ONE JSON line.  `value` is sampled edges per second of the sampling + id-map stage;
+`roofline` describes the dominant kernel (the outermost block's forward aggregation) against
+the 8 TB/s HBM peak; `cpu_baseline` is the CPU oracle timed on a bounded sample of the same
+workload on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "fastgl-ae_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: nodes, R-MAT draws, feature dim, feature dtype, hidden, batch, training seeds, fanouts (reference order)
+    "c1": dict(nodes=100_000, draws=1_500_000, dim=128, dtype="f32", hidden=256, batch=1024, train=100_000, fanouts=[15, 10, 5]),
+    "c2": dict(nodes=2_400_000, draws=36_000_000, dim=100, dtype="f32", hidden=256, batch=8192, train=240_000, fanouts=[15, 10, 5]),
+    "c3": dict(nodes=111_000_000, draws=900_000_000, dim=128, dtype="f32", hidden=256, batch=8192, train=1_200_000, fanouts=[15, 10, 5]),
+}
+DESCRIPTIONS = {
+    "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
+    "c2": "R-MAT 2.4M nodes / ~62M edges, feat 100 fp32, hidden 256, batch 8192, fanout [15,10,5]",
+    "c3": "R-MAT 111M nodes / ~1.6B edges (int64 indptr, int32 indices), feat 111Mx128 fp32 resident, hidden 256, "
+          "batch 8192 of 1.2M training seeds, fanout [15,10,5]",
+}
+
+
+def log(*a):
+    print("[bench]", *a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-batches", type=int, default=2, help="mini-batches timed on the CPU oracle (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
+              "(mini-batches shard over GPUs by seed partition with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import fastgl
+
+    fastgl.lib()  # fail here, loudly, if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[args.workload]
+    N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
+    fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16
+    esz = 4 if fdtype == torch.float32 else 2
+
+    # ---- synthetic inputs, generated on the device ------------------------------------
+    t0 = time.time()
+    edge_ptr, edge_src = fastgl.graph.rmat_csr(N, w["draws"], seed=0, device=dev)
+    torch.cuda.synchronize()
+    n_graph_edges = int(edge_src.numel())
+    log("graph: %d nodes, %d directed edges, built in %.1fs" % (N, n_graph_edges, time.time() - t0))
+    torch.cuda.empty_cache()
+    t0 = time.time()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    feat = torch.empty((N, D), dtype=fdtype, device=dev)
+    for lo in range(0, N, 1 << 22):
+        hi = min(N, lo + (1 << 22))
+        feat[lo:hi] = torch.randn((hi - lo, D), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+    train = torch.randperm(N, generator=gen, device=dev)[:w["train"]].to(torch.int32)
+    n_batches = max(1, w["train"] // B)
+    torch.cuda.synchronize()
+    log("features %s x %d %s and %d training seeds in %.1fs" % (N, D, w["dtype"], w["train"], time.time() - t0))
+
+    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0).set_graph(edge_ptr, edge_src)
+    L = len(w["fanouts"])
+    # hidden activations / upstream gradients of the inner layers: synthetic, sized for the worst case
+    plan_caps = fastgl.BlocksPlan(N, B, list(reversed(w["fanouts"])), dev).cap_dst
+    cap_inner = plan_caps[-1]
+    hid = torch.randn((cap_inner, H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+    grad = torch.randn((cap_inner, H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def step(i, rec=None):
+        seeds = train[(i % n_batches) * B:(i % n_batches) * B + B]
+        e0, e1, e2, e3, e4 = ev(), ev(), ev(), ev(), ev()
+        e0.record()
+        input_nodes, _, blocks = sampler.sample_blocks(None, seeds)  # includes the one count read-back
+        e1.record()
+        b0 = blocks[0]
+        out0 = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
+        e2.record()
+        outs = [out0]
+        for b in blocks[1:]:
+            outs.append(fastgl.aggregate(b.edge_ptr, b.src_local, hid[:b.num_src_nodes()], mode="mean", zero_policy="zeros"))
+        e3.record()
+        for b in blocks[1:]:
+            t_ptr, t_idx = b.transposed()
+            outs.append(fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",
+                                         col_norm=b.in_degrees().contiguous()))
+        e4.record()
+        if rec is not None:
+            rec.append((blocks, (e0, e1, e2, e3, e4)))
+        return blocks
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    rec = []
+    t_start = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i, rec)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_start
+
+    # ---- reduce -------------------------------------------------------------------------
+    tot_edges = 0
+    t_sample = t_agg0 = t_fwd_in = t_bwd = 0.0
+    bytes_agg0 = 0
+    for blocks, (e0, e1, e2, e3, e4) in rec:
+        tot_edges += sum(b.num_edges() for b in blocks)
+        t_sample += e0.elapsed_time(e1)
+        t_agg0 += e1.elapsed_time(e2)
+        t_fwd_in += e2.elapsed_time(e3)
+        t_bwd += e3.elapsed_time(e4)
+        b0 = blocks[0]
+        e_, nd = b0.num_edges(), b0.num_dst_nodes()
+        bytes_agg0 += e_ * D * esz + nd * D * esz + 4 * e_ + 4 * (nd + 1)  # gathered rows + output + indices + offsets
+    K = args.steps
+    edges_per_s = tot_edges / (t_sample * 1e-3)
+    agg_gbps = bytes_agg0 / (t_agg0 * 1e-3) / 1e9
+    b_last = rec[-1][0]
+    log("last batch blocks:", b_last)
+    log("per step: sample+idmap %.3f ms, agg fwd outer %.3f ms, agg fwd inner %.3f ms, transpose+bwd %.3f ms, wall %.3f ms"
+        % (t_sample / K, t_agg0 / K, t_fwd_in / K, t_bwd / K, wall / K * 1e3))
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same workload ------------
+    cpu = None
+    if args.cpu_batches > 0:
+        from oracle import oracle as O
+        t0 = time.time()
+        h_ptr, h_src = edge_ptr.cpu().numpy(), edge_src.cpu().numpy()
+        log("graph copied to the host in %.1fs; oracle threads: %d" % (time.time() - t0, O.num_threads()))
+        cpu_edges, cpu_t, agg_t, agg_bytes = 0, 0.0, 0.0, 0
+        for i in range(args.cpu_batches):
+            seeds = train[i * B:(i + 1) * B].cpu().numpy()
+            t0 = time.perf_counter()
+            inp, oblocks = O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, i * 64)
+            cpu_t += time.perf_counter() - t0
+            cpu_edges += sum(int(b["src_local"].size) for b in oblocks)
+            ob = oblocks[0]
+            xb = feat.index_select(0, torch.from_numpy(inp).to(dev).long()).float().cpu().numpy()  # rows of the input nodes
+            t0 = time.perf_counter()
+            O.aggregate(ob["indptr"], ob["src_local"], xb, "mean", 1, out_dtype=np.float32)
+            agg_t += time.perf_counter() - t0
+            e_, nd = int(ob["src_local"].size), int(ob["n_dst"])
+            agg_bytes += e_ * D * 4 + nd * D * 4 + 4 * e_ + 4 * (nd + 1)
+        cpu = {"value": cpu_edges / cpu_t, "unit": "sampled edges/s", "cores": O.num_threads(), "kind": "port",
+               "sample": "%d mini-batches of %d seeds of the same workload through the CPU oracle "
+                         "(OpenMP sampling, sequential first-occurrence id-map); aggregation = fp32 OpenMP row gather "
+                         "of the outermost block" % (args.cpu_batches, B),
+               "aggregation_GBps": agg_bytes / agg_t / 1e9, "host_cpus": os.cpu_count()}
+        log("cpu baseline: %.3g edges/s (%d threads), aggregation %.1f GB/s" % (cpu["value"], cpu["cores"], cpu["aggregation_GBps"]))
+
+    out = {
+        "metric": "sampled edges/s (sample+id_map) + aggregation HBM GB/s (% peak), 1 MI355X",
+        "value": edges_per_s,
+        "unit": "sampled edges/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": wall / K * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w["dtype"],
+        "data": "synthetic",
+        "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
+                   "sampled_edges_per_step": tot_edges / K, "id_order": "first-occurrence (deterministic)",
+                   "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
+                           "feature table); block transpose + bwd gather on the inner blocks; no dense layers"},
+        "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
+                      "transpose_agg_bwd_inner": t_bwd / K},
+        "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS},
+        "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
+        "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": agg_gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "aggregate_kernel (outermost block, mean, forward)",
+                     "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_agg0 / K * 1e3},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

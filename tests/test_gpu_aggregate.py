@@ -1,0 +1,149 @@
+"""HIP aggregation (forward, and backward as a gather over the transposed block) against the
+fp64 oracle, through the C ABI.  Tolerances are the acceptance criterion's: 1e-5 relative
+for fp32 and 1e-2 for bf16, relative to the largest magnitude of the fp64 result row-block."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN_DIR
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+def dev_i32(a, cuda):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(cuda)
+
+
+def rel_err(got, want):
+    scale = max(np.abs(want).max(), 1e-30)
+    return np.abs(got.astype(np.float64) - want).max() / scale
+
+
+def make_block(rng, n_dst, n_src, max_deg, hubs=()):
+    deg = rng.integers(0, max_deg + 1, size=n_dst)
+    for r, d in hubs:
+        deg[r] = d
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    idx = rng.integers(0, n_src, size=ptr[-1]).astype(np.int32)
+    return ptr, idx, deg
+
+
+def run_modes(cuda, oracle, ptr, idx, deg, X_t, n_src, tol):
+    import fastgl
+    X_ref = X_t.float().cpu().numpy()  # the exact values the kernel reads (bf16 widened)
+    rn = np.maximum(deg, 1).astype(np.int32)
+    cn = np.maximum(np.bincount(idx, minlength=n_src), 1).astype(np.int32)
+    d_ptr, d_idx, d_rn, d_cn = dev_i32(ptr, cuda), dev_i32(idx, cuda), dev_i32(rn, cuda), dev_i32(cn, cuda)
+    for mode in ("sum", "mean", "gcn", "colmean"):
+        for pol_name, pol in (("self", 0), ("zeros", 1)):
+            got = fastgl.aggregate(d_ptr, d_idx, X_t, mode=mode, zero_policy=pol_name, row_norm=d_rn, col_norm=d_cn)
+            want = oracle.aggregate(ptr, idx, X_ref, mode, pol, rn, cn)
+            assert got.dtype == X_t.dtype and tuple(got.shape) == want.shape
+            err = rel_err(got.float().cpu().numpy(), want)
+            assert err < tol, (mode, pol_name, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [1, 7, 30, 64, 100, 128, 256, 602, 1030])
+def test_aggregate_vs_oracle(cuda, oracle, dtype, D):
+    print("aggregate D=%d %s" % (D, dtype), flush=True)
+    rng = np.random.default_rng(D)
+    n_dst, n_src = 517, 2000
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 12, hubs=[(3, 64), (4, 65), (100, 300)])
+    X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
+    run_modes(cuda, oracle, ptr, idx, deg, X, n_src, TOL[dtype])
+
+
+def test_aggregate_golden(cuda):
+    import fastgl
+    print("aggregate golden", flush=True)
+    g = np.load(os.path.join(GOLDEN_DIR, "aggregate_small.npz"))
+    d = lambda k: dev_i32(g[k], cuda)
+    X = torch.from_numpy(g["X"]).to(cuda)
+    for mode in ("sum", "mean", "gcn", "colmean"):
+        for pol_name, pol in (("self", 0), ("zeros", 1)):
+            got = fastgl.aggregate(d("ptr"), d("idx"), X, mode=mode, zero_policy=pol_name, row_norm=d("row_norm"), col_norm=d("col_norm"))
+            assert rel_err(got.cpu().numpy(), g["%s_%d" % (mode, pol)]) < 1e-5
+
+
+def test_strided_rows_and_narrow_vectors(cuda, oracle):
+    """a column slice of a wider table: row stride != row length, base not 16-byte aligned"""
+    import fastgl
+    print("aggregate strided", flush=True)
+    rng = np.random.default_rng(8)
+    n_dst, n_src = 200, 900
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 10)
+    wide = torch.from_numpy(rng.standard_normal((n_src, 70)).astype(np.float32)).to(cuda)
+    for lo, hi in ((0, 64), (1, 65), (2, 66), (3, 35)):
+        X = wide[:, lo:hi]
+        got = fastgl.aggregate(dev_i32(ptr, cuda), dev_i32(idx, cuda), X, mode="mean", zero_policy="zeros")
+        want = oracle.aggregate(ptr, idx, X.cpu().numpy(), "mean", 1)
+        assert rel_err(got.cpu().numpy(), want) < 1e-5
+
+
+def test_closed_forms_on_device(cuda):
+    import fastgl
+    print("aggregate closed forms", flush=True)
+    rng = np.random.default_rng(2)
+    ptr, idx, deg = make_block(rng, 300, 300, 20)
+    ones = torch.ones(300, 128, device=cuda)
+    s = fastgl.aggregate(dev_i32(ptr, cuda), dev_i32(idx, cuda), ones, mode="sum", zero_policy="zeros").cpu().numpy()
+    assert np.array_equal(s, np.repeat(deg[:, None], 128, 1).astype(np.float32))  # small integers: exact in fp32
+    m = fastgl.aggregate(dev_i32(ptr, cuda), dev_i32(idx, cuda), ones, mode="mean", zero_policy="zeros").cpu().numpy()
+    assert np.allclose(m[deg > 0], 1.0, rtol=1e-6) and (m[deg == 0] == 0).all()
+
+
+def test_block_transpose_and_backward(cuda, oracle):
+    """d_x = A^T d_out computed by gathering over the transposed block == oracle on the oracle's
+    (stable) transpose; the device transpose holds the same lists up to order within a column."""
+    import fastgl
+    print("transpose + backward", flush=True)
+    rng = np.random.default_rng(21)
+    n_dst, n_src, D = 3000, 9000, 128
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 15, hubs=[(0, 500)])
+    idx[: 2500] = 17  # a hub column
+    t_ptr, t_idx = fastgl.block_transpose(dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src)
+    w_ptr, w_idx = oracle.transpose(ptr, idx, n_src)
+    g_ptr, g_idx = t_ptr.cpu().numpy(), t_idx.cpu().numpy()
+    assert np.array_equal(g_ptr, w_ptr)
+    seg = np.repeat(np.arange(n_src), np.diff(w_ptr))
+    assert np.array_equal(g_idx[np.lexsort((g_idx, seg))], w_idx)             # same lists, sorted within columns
+    rn = np.maximum(deg, 1).astype(np.int32)
+    cn = np.maximum(np.bincount(idx, minlength=n_src), 1).astype(np.int32)
+    d_out = rng.standard_normal((n_dst, D)).astype(np.float32)
+    for mode, row_norm, col_norm in (("sum", None, None), ("colmean", None, rn), ("gcn", cn, rn)):
+        got = fastgl.aggregate(t_ptr, t_idx, torch.from_numpy(d_out).to(cuda), mode=mode, zero_policy="zeros",
+                               row_norm=None if row_norm is None else dev_i32(row_norm, cuda),
+                               col_norm=None if col_norm is None else dev_i32(col_norm, cuda))
+        want = oracle.aggregate(w_ptr, w_idx, d_out, mode, 1, row_norm, col_norm)
+        assert rel_err(got.cpu().numpy(), want) < 1e-5, mode
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128, 256, 602])
+def test_microbench_shape(cuda, oracle, dtype, D):
+    """8192 destination rows x exactly 25 neighbours out of 200K source rows, sum and mean,
+    forward and backward"""
+    import fastgl
+    print("microbench shape D=%d %s" % (D, dtype), flush=True)
+    g = torch.Generator().manual_seed(0)
+    n_dst, n_src, k = 8192, 200_000, 25
+    ptr = (torch.arange(n_dst + 1, dtype=torch.int32) * k)
+    idx = torch.randint(0, n_src, (n_dst * k,), generator=g, dtype=torch.int32)
+    X = torch.randn(n_src, D, generator=g).to(dtype)
+    dO = torch.randn(n_dst, D, generator=g).to(dtype)
+    d_ptr, d_idx, Xd, dOd = ptr.to(cuda), idx.to(cuda), X.to(cuda), dO.to(cuda)
+    t_ptr, t_idx = fastgl.block_transpose(d_ptr, d_idx, n_dst, n_src)
+    w_tptr, w_tidx = oracle.transpose(ptr.numpy(), idx.numpy(), n_src)
+    deg = np.full(n_dst, k, np.int32)
+    for mode, bmode in (("sum", "sum"), ("mean", "colmean")):
+        fwd = fastgl.aggregate(d_ptr, d_idx, Xd, mode=mode, zero_policy="zeros")
+        want = oracle.aggregate(ptr.numpy(), idx.numpy(), X.float().numpy(), mode, 1)
+        assert rel_err(fwd.float().cpu().numpy(), want) < TOL[dtype]
+        bwd = fastgl.aggregate(t_ptr, t_idx, dOd, mode=bmode, zero_policy="zeros", col_norm=dev_i32(deg, cuda))
+        wantb = oracle.aggregate(w_tptr, w_tidx, dO.float().numpy(), bmode, 1, None, deg)
+        assert rel_err(bwd.float().cpu().numpy(), wantb) < TOL[dtype]

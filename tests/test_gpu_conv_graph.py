@@ -1,0 +1,163 @@
+"""Layer-level parity (forward and autograd backward) against dense fp64 torch on the CPU,
+the drop-in operator signatures, and the device R-MAT generator against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_i32(a, cuda):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(cuda)
+
+
+def small_blocks(cuda, oracle, small_graph, fanouts=(4, 3), batch=200):
+    import fastgl
+    indptr, indices = small_graph
+    sampler = fastgl.FusedMapSampler(list(fanouts), rng_seed=3).set_graph(torch.from_numpy(indptr).to(cuda), dev_i32(indices, cuda))
+    seeds = np.random.default_rng(0).permutation(indptr.size - 1)[:batch].astype(np.int32)
+    return sampler.sample_blocks(None, dev_i32(seeds, cuda))
+
+
+def dense_adj(block, kind):
+    """fp64 dense operator of a block as the reference kernels define it"""
+    n_dst, n_src = block.num_dst_nodes(), block.num_src_nodes()
+    src, dst = (t.cpu().long() for t in block.edges())
+    A = torch.zeros(n_dst, n_src, dtype=torch.float64)
+    A.index_put_((dst, src), torch.ones(src.numel(), dtype=torch.float64), accumulate=True)
+    deg = A.sum(1)
+    if kind == "gcn":
+        dn = deg.clamp(min=1)
+        sn = torch.bincount(src, minlength=n_src).double().clamp(min=1)
+        A = dn.rsqrt()[:, None] * A * sn.rsqrt()[None, :]
+    if kind == "mean":
+        A = A / deg.clamp(min=1)[:, None]
+    passthrough = (deg == 0)
+    return A, passthrough
+
+
+@pytest.mark.parametrize("model_name", ["gcn", "gin"])
+def test_gcn_gin_forward_backward(cuda, oracle, small_graph, model_name):
+    import fastgl
+    print("conv %s" % model_name, flush=True)
+    input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
+    torch.manual_seed(0)
+    cls = fastgl.GCN if model_name == "gcn" else fastgl.GIN
+    model = cls(20, 16, 5, 2, None, True, 0.0).to(cuda)
+    x = torch.randn(input_nodes.numel(), 20, device=cuda, requires_grad=True)
+    out = model(blocks, x, neighbor_list=[4, 3])
+    gout = torch.randn_like(out)
+    out.backward(gout)
+
+    h = x.detach().cpu().double().requires_grad_(True)
+    ws = [l.weights.detach().cpu().double().requires_grad_(True) for l in model.layers]
+    cur = h
+    for block, w in zip(blocks, ws):
+        A, passthrough = dense_adj(block, "gcn" if model_name == "gcn" else "sum")
+        n_dst = block.num_dst_nodes()
+        if model_name == "gcn":
+            t = cur @ w
+            # rows without edges pass (X W)[d] through, and no gradient flows back through that copy
+            cur = A @ t + passthrough[:, None] * t[:n_dst].detach()
+        else:
+            cur = (A @ cur + passthrough[:, None] * cur[:n_dst].detach()) @ w
+    cur.backward(gout.cpu().double())
+    assert torch.allclose(out.detach().cpu().double(), cur.detach(), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
+    for l, w in zip(model.layers, ws):
+        assert torch.allclose(l.weights.grad.cpu().double(), w.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_sage_mean_with_fused_input_gather(cuda, oracle, small_graph):
+    import fastgl
+    print("conv sage", flush=True)
+    indptr, _ = small_graph
+    input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
+    torch.manual_seed(1)
+    feat = torch.randn(indptr.size - 1, 24, device=cuda)
+    model = fastgl.SAGE(24, 16, 5, 2, dropout=0.0).to(cuda)
+    out_fused = model(blocks, feat, input_nodes=input_nodes)          # first layer reads the full table
+    x = feat.index_select(0, input_nodes.long()).requires_grad_(True)  # the explicit gather the reference does
+    out = model(blocks, x)
+    assert torch.allclose(out, out_fused, rtol=1e-5, atol=1e-6)
+    gout = torch.randn_like(out)
+    out.backward(gout)
+
+    h = x.detach().cpu().double().requires_grad_(True)
+    cur = h
+    params = []
+    for i, (layer, block) in enumerate(zip(model.layers, blocks)):
+        A, _ = dense_adj(block, "mean")
+        ws = layer.fc_self.weight.detach().cpu().double().requires_grad_(True)
+        wn = layer.fc_neigh.weight.detach().cpu().double().requires_grad_(True)
+        b = layer.fc_neigh.bias.detach().cpu().double().requires_grad_(True)
+        params.append((layer, ws, wn, b))
+        cur = cur[:block.num_dst_nodes()] @ ws.T + (A @ cur) @ wn.T + b
+        if i == 0:
+            cur = torch.relu(cur)
+    cur.backward(gout.cpu().double())
+    assert torch.allclose(out.detach().cpu().double(), cur.detach(), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
+    for layer, ws, wn, b in params:
+        assert torch.allclose(layer.fc_self.weight.grad.cpu().double(), ws.grad, rtol=1e-4, atol=1e-5)
+        assert torch.allclose(layer.fc_neigh.weight.grad.cpu().double(), wn.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_drop_in_operator_flow(cuda, oracle, small_graph):
+    """The reference's own call sequence (GraphConv.py:91-98 on COO edges): cal_deg -> exclusive_sum ->
+    forward_gcn / backward_gcn and forwaed_gin / backward_gin, checked against the oracle."""
+    import fastgl
+    print("drop-in operator flow", flush=True)
+    _, _, blocks = small_blocks(cuda, oracle, small_graph)
+    block = blocks[0]
+    src, dst = block.edges()
+    n_dst, n_src = block.num_dst_nodes(), block.num_src_nodes()
+    raw = fastgl.cal_deg(dst, n_dst)
+    edge_ptr = fastgl.exclusive_sum(raw)
+    assert torch.equal(edge_ptr, block.edge_ptr)
+    src_norm = fastgl.cal_deg(src, n_src).clamp(min=1)
+    dst_norm = raw.clamp(min=1)
+    rng = np.random.default_rng(4)
+    X = torch.from_numpy(rng.standard_normal((n_src, 12)).astype(np.float32)).to(cuda)
+    W = torch.from_numpy(rng.standard_normal((12, 8)).astype(np.float32)).to(cuda)
+    ptr_h, src_h = edge_ptr.cpu().numpy(), src.cpu().numpy()
+    sn_h, dn_h = src_norm.cpu().numpy(), dst_norm.cpu().numpy()
+    T = (X.double() @ W.double()).float().cpu().numpy()
+
+    (out,) = fastgl.forward_gcn(edge_ptr, src, src_norm, dst_norm, X, W, 4, n_dst)
+    want = oracle.aggregate(ptr_h, src_h, T, "gcn", 0, dn_h, sn_h)
+    assert np.abs(out.cpu().numpy() - want).max() < 1e-4 * max(1, np.abs(want).max())
+
+    d_out = torch.from_numpy(rng.standard_normal((n_dst, 8)).astype(np.float32)).to(cuda)
+    d_x, d_w = fastgl.backward_gcn(edge_ptr, src, dst_norm, src_norm, d_out, W, X)  # (dst, src) order: GraphConv.py:37
+    t_ptr, t_idx = oracle.transpose(ptr_h, src_h, n_src)
+    G = oracle.aggregate(t_ptr, t_idx, d_out.cpu().numpy(), "gcn", 1, sn_h, dn_h)
+    assert np.abs(d_x.cpu().numpy() - G @ W.cpu().numpy().T.astype(np.float64)).max() < 1e-3
+    assert np.abs(d_w.cpu().numpy() - X.cpu().numpy().T.astype(np.float64) @ G).max() < 1e-3
+
+    out, tmp = fastgl.forwaed_gin(edge_ptr, src, X, W, 4, n_dst)
+    want_tmp = oracle.aggregate(ptr_h, src_h, X.cpu().numpy(), "sum", 0)
+    assert np.abs(tmp.cpu().numpy() - want_tmp).max() < 1e-4
+    assert np.abs(out.cpu().numpy() - want_tmp @ W.cpu().numpy().astype(np.float64)).max() < 1e-3
+    d_x, d_w = fastgl.backward_gin(edge_ptr, src, d_out, W, tmp, n_src)
+    d_tmp = d_out.cpu().numpy().astype(np.float64) @ W.cpu().numpy().T
+    want_dx = oracle.aggregate(t_ptr, t_idx, d_tmp.astype(np.float32), "sum", 1)
+    assert np.abs(d_x.cpu().numpy() - want_dx).max() < 1e-3
+    assert np.abs(d_w.cpu().numpy() - want_tmp.T @ d_out.cpu().numpy()).max() < 1e-3
+
+
+def test_rmat_keys_match_oracle(cuda, oracle):
+    import fastgl
+    print("rmat keys", flush=True)
+    for n_nodes, n, first, seed in ((1000, 5000, 0, 0), (100_000, 200_000, 12345, 7), (3, 100, 0, 1)):
+        scale = fastgl.graph.rmat_scale(n_nodes)
+        got = fastgl.rmat_keys(first, n, scale, n_nodes, seed, cuda).cpu().numpy()
+        assert np.array_equal(got, oracle.rmat_keys(first, n, scale, n_nodes, seed))
+
+
+def test_rmat_csr_matches_oracle(cuda, oracle, small_graph):
+    import fastgl
+    print("rmat csr", flush=True)
+    indptr, indices = small_graph
+    ptr, src = fastgl.graph.rmat_csr(100_000, 1_500_000, seed=0, device=cuda, chunk_draws=400_000)
+    assert np.array_equal(ptr.cpu().numpy(), indptr) and np.array_equal(src.cpu().numpy(), indices)

@@ -1,0 +1,73 @@
+"""Size-independent properties at a full benchmark shape: the 2.4M-node / ~62M-edge R-MAT
+graph, batch 8192, fanout [15,10,5] (the oracle is not run at this size)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_mid_shape_properties(cuda):
+    import fastgl
+    print("full-size: building 2.4M-node graph", flush=True)
+    n = 2_400_000
+    ptr, src = fastgl.graph.rmat_csr(n, 36_000_000, seed=0, device=cuda)
+    n_edges = int(src.numel())
+    print("edges:", n_edges, "max degree:", int((ptr[1:] - ptr[:-1]).max()), flush=True)
+    assert 50_000_000 < n_edges < 75_000_000
+    row_of_edge = torch.repeat_interleave(torch.arange(n, device=cuda), ptr[1:] - ptr[:-1])
+    graph_keys = (row_of_edge << 32) | src.long()
+    del row_of_edge
+
+    fanouts = [15, 10, 5]
+    sampler = fastgl.FusedMapSampler(fanouts, rng_seed=11).set_graph(ptr, src)
+    seeds = torch.randperm(n, device=cuda)[:8192].int()
+    input_nodes, out_nodes, blocks = sampler.sample_blocks(None, seeds)
+    print("blocks:", blocks, flush=True)
+    assert torch.equal(out_nodes, seeds)
+    assert input_nodes.unique().numel() == input_nodes.numel()           # unique ids
+    assert torch.equal(input_nodes[:8192], seeds)                        # seeds keep their positions
+    deg_all = (ptr[1:] - ptr[:-1])
+    cur_dst = seeds
+    for block, fanout in zip(reversed(blocks), reversed(fanouts)):
+        n_dst, n_src = block.num_dst_nodes(), block.num_src_nodes()
+        assert n_dst == cur_dst.numel()
+        src_l, dst_l = block.edges()
+        uniq = input_nodes[:n_src]
+        # exactly min(fanout, deg) edges per destination
+        want_k = torch.clamp(deg_all[cur_dst.long()], max=fanout).int()
+        assert torch.equal(block.in_degrees(), want_k)
+        # every sampled edge exists in the graph
+        g_src, g_dst = uniq[src_l.long()].long(), uniq[dst_l.long()].long()
+        keys = (g_dst << 32) | g_src
+        pos = torch.searchsorted(graph_keys, keys).clamp(max=n_edges - 1)
+        assert torch.equal(graph_keys[pos], keys)
+        # no neighbour twice for one destination
+        pair = (dst_l.long() << 32) | src_l.long()
+        assert pair.unique().numel() == pair.numel()
+        # the id-map: every local id in range, all source nodes referenced or inherited
+        assert int(src_l.max()) < n_src and int(src_l.min()) >= 0
+        if block.src_global is not None:
+            assert torch.equal(uniq[src_l.long()], block.src_global)
+        new_ids = torch.unique(src_l[src_l >= n_dst])
+        assert new_ids.numel() == n_src - n_dst                          # every new id is used by some edge
+        cur_dst = uniq
+    # aggregation at this shape: linearity and the all-ones closed form on the outermost block
+    b0 = blocks[0]
+    ones = torch.ones(b0.num_src_nodes(), 128, device=cuda)
+    deg0 = b0.in_degrees().float()
+    s = fastgl.aggregate(b0.edge_ptr, b0.src_local, ones, mode="sum", zero_policy="zeros")
+    assert torch.equal(s, deg0[:, None].expand(-1, 128))
+    x = torch.randn(b0.num_src_nodes(), 128, device=cuda)
+    y = torch.randn(b0.num_src_nodes(), 128, device=cuda)
+    lhs = fastgl.aggregate(b0.edge_ptr, b0.src_local, x + 2 * y, mode="mean", zero_policy="zeros")
+    rhs = fastgl.aggregate(b0.edge_ptr, b0.src_local, x, mode="mean", zero_policy="zeros") + \
+        2 * fastgl.aggregate(b0.edge_ptr, b0.src_local, y, mode="mean", zero_policy="zeros")
+    assert torch.allclose(lhs, rhs, rtol=1e-4, atol=1e-4)
+    # adjointness <A x, g> == <x, A^T g> ties the backward gather to the forward one
+    t_ptr, t_idx = b0.transposed()
+    g = torch.randn(b0.num_dst_nodes(), 128, device=cuda)
+    ax = fastgl.aggregate(b0.edge_ptr, b0.src_local, x, mode="sum", zero_policy="zeros")
+    atg = fastgl.aggregate(t_ptr, t_idx, g, mode="sum", zero_policy="zeros")
+    a, b = (ax.double() * g.double()).sum().item(), (x.double() * atg.double()).sum().item()
+    assert abs(a - b) <= 1e-6 * max(abs(a), abs(b), 1.0)

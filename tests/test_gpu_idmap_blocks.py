@@ -1,0 +1,133 @@
+"""HIP fused id-map and the all-hops sampler against the oracle, through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN_DIR
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_i32(a, cuda):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(cuda)
+
+
+def canonical(src_local, uniq, n_dst, block_ptr=None):
+    """Order-free form of an id-map result: new ids renumbered by ascending graph id, each
+    destination row's edge list sorted."""
+    tail = uniq[n_dst:]
+    order = np.argsort(tail, kind="stable")
+    remap = np.concatenate([np.arange(n_dst), n_dst + np.argsort(order, kind="stable")])
+    s = remap[src_local]
+    if block_ptr is not None:
+        s = np.concatenate([np.sort(s[block_ptr[i]:block_ptr[i + 1]]) for i in range(len(block_ptr) - 1)] or [s[:0]])
+    return s, np.concatenate([uniq[:n_dst], tail[order]])
+
+
+def run_transfer(cuda, src, dst, dst_unique, n_nodes):
+    import fastgl
+    s, d = dev_i32(src, cuda), dev_i32(dst, cuda)
+    n_dst, e = len(dst_unique), len(src)
+    out = fastgl.transfer_edge_id(s, d, dev_i32(dst_unique, cuda), n_dst, n_dst + e, min(n_nodes, max(e, 1)), e)
+    assert out[0].data_ptr() == s.data_ptr() and out[1].data_ptr() == d.data_ptr()  # in place, like the reference
+    return out[0].cpu().numpy(), out[1].cpu().numpy(), out[2].cpu().numpy()
+
+
+def test_hand_fixture(cuda):
+    print("idmap hand fixture", flush=True)
+    g = np.load(os.path.join(GOLDEN_DIR, "idmap_hand.npz"))
+    s, d, u = run_transfer(cuda, g["src"], g["dst"], g["dst_unique"], 10)
+    assert np.array_equal(s, g["src_local"]) and np.array_equal(d, g["dst_local"]) and np.array_equal(u, g["uniq"])
+
+
+@pytest.mark.parametrize("n_ids,n_dst,n_edges", [(50, 10, 4000), (100_000, 1000, 15_000), (2**31 - 1, 64, 50_000),
+                                                 (3_000_000, 8192, 1_000_000), (7, 7, 0), (1000, 1, 2049)])
+def test_transfer_edge_id_vs_oracle(cuda, oracle, n_ids, n_dst, n_edges):
+    print("idmap %d %d %d" % (n_ids, n_dst, n_edges), flush=True)
+    rng = np.random.default_rng(n_edges + n_dst)
+    dst_unique = rng.choice(min(n_ids, 10**7), size=n_dst, replace=False).astype(np.int32)
+    # power-law-ish sources so that hot ids collide heavily
+    src = (rng.pareto(1.2, size=n_edges) * 50).astype(np.int64) % n_ids
+    src[::7] = rng.integers(0, n_ids, size=src[::7].size)
+    src = src.astype(np.int32)
+    dst = np.sort(rng.integers(0, n_dst, size=n_edges))
+    dst_g = dst_unique[dst] if n_edges else np.zeros(0, np.int32)
+    s, d, u = run_transfer(cuda, src, dst_g, dst_unique, n_ids)
+    ws, wd, wu = oracle.idmap(src, dst_g, dst_unique)
+    # bit-exact, order included (first-occurrence numbering) ...
+    assert np.array_equal(u, wu) and np.array_equal(s, ws) and np.array_equal(d, wd)
+    # ... and after the canonical sort that the acceptance criterion names
+    bptr = np.concatenate([[0], np.cumsum(np.bincount(dst, minlength=n_dst))])
+    cs, cu = canonical(s, u, n_dst, bptr)
+    cws, cwu = canonical(ws, wu, n_dst, bptr)
+    assert np.array_equal(cs, cws) and np.array_equal(cu, cwu)
+
+
+def test_transfer_edge_id_reports_missing_dst(cuda):
+    print("idmap missing key", flush=True)
+    with pytest.raises(RuntimeError, match="not in the map"):
+        run_transfer(cuda, np.array([1, 2], np.int32), np.array([5, 77], np.int32), np.array([5], np.int32), 100)
+
+
+def load_graph(cuda, indptr, indices):
+    return torch.from_numpy(indptr).to(cuda), dev_i32(indices, cuda)
+
+
+def check_blocks(oracle, indptr, indices, seeds, fanouts, got, rng_seed, stream_base):
+    inp, out_nodes, blocks = got
+    w_inp, w_blocks = oracle.sample_blocks(indptr, indices, seeds, fanouts, rng_seed, stream_base)
+    assert np.array_equal(inp.cpu().numpy(), w_inp)
+    assert np.array_equal(out_nodes.cpu().numpy(), seeds)
+    assert len(blocks) == len(w_blocks)
+    for b, w in zip(blocks, w_blocks):
+        assert (b.num_src_nodes(), b.num_dst_nodes()) == (w["n_src"], w["n_dst"])
+        assert np.array_equal(b.edge_ptr.cpu().numpy(), w["indptr"])
+        assert np.array_equal(b.src_local.cpu().numpy(), w["src_local"])
+        if b.src_global is not None:
+            assert np.array_equal(b.src_global.cpu().numpy(), w["src_global"])
+        src, dst = b.edges()
+        assert np.array_equal(dst.cpu().numpy(), np.repeat(np.arange(w["n_dst"]), np.diff(w["indptr"])))
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_sample_blocks_golden(cuda, oracle, fused):
+    import fastgl
+    print("sample_blocks golden fused=%s" % fused, flush=True)
+    g = np.load(os.path.join(GOLDEN_DIR, "sample_blocks_small.npz"))
+    ptr, idx = load_graph(cuda, g["indptr"], g["indices"])
+    s = fastgl.FusedMapSampler(g["fanouts"].tolist(), fused=fused, rng_seed=int(g["rng_seed"])).set_graph(ptr, idx)
+    inp, out_nodes, blocks = s.sample_blocks(None, dev_i32(g["seeds"], cuda))
+    assert np.array_equal(inp.cpu().numpy(), g["input_nodes"])
+    for i, b in enumerate(blocks):
+        assert np.array_equal(b.edge_ptr.cpu().numpy(), g["b%d_ptr" % i])
+        assert np.array_equal(b.src_local.cpu().numpy(), g["b%d_src_local" % i])
+        assert [b.num_src_nodes(), b.num_dst_nodes()] == g["b%d_shape" % i].tolist()
+    assert np.array_equal(blocks[0].src_global.cpu().numpy(), g["b0_src_global"])
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64), ([3], 1), ([64, 2], 300)])
+def test_sample_blocks_vs_oracle(cuda, oracle, small_graph, fused, fanouts, batch):
+    import fastgl
+    print("sample_blocks %s batch=%d fused=%s" % (fanouts, batch, fused), flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    sampler = fastgl.FusedMapSampler(fanouts, fused=fused, rng_seed=5).set_graph(ptr, idx)
+    rng = np.random.default_rng(batch)
+    for it in range(2):  # the second mini-batch uses the next Philox streams and a reused table
+        seeds = rng.permutation(indptr.size - 1)[:batch].astype(np.int32)
+        got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        check_blocks(oracle, indptr, indices, seeds, fanouts, got, 5, it * 64)
+
+
+def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
+    import fastgl
+    print("sample_blocks int32 ptr", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr.astype(np.int32), indices)
+    sampler = fastgl.FusedMapSampler([4, 4], rng_seed=1).set_graph(ptr, idx)
+    seeds = np.arange(100, 612, dtype=np.int32)
+    got = sampler.sample_blocks(None, torch.from_numpy(seeds.astype(np.int64)).to(cuda))  # DataLoader seeds are int64
+    check_blocks(oracle, indptr, indices, seeds, [4, 4], got, 1, 0)
