@@ -113,7 +113,10 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     if (rc != FGL_OK) return rc;
     FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
     FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
-    FGL_REQUIRE(table_slots >= p.table_slots, "sample_blocks: table has %lld slots, plan needs %lld", (long long)table_slots, (long long)p.table_slots);
+    // A table smaller than the plan's worst case is accepted (batches are usually far below the
+    // bound and a small table stays cache-resident): the seeds must fit, and a batch that
+    // outgrows the table is reported through FGL_STATUS_TABLE_FULL, never by a fault.
+    FGL_REQUIRE(table_slots >= fgl_idmap_slots(n_seeds), "sample_blocks: table has %lld slots, the seeds alone need %lld", (long long)table_slots, (long long)fgl_idmap_slots(n_seeds));
     FGL_REQUIRE(uniq_capacity >= p.cap_uniq, "sample_blocks: unique list holds %lld, plan needs %lld", (long long)uniq_capacity, (long long)p.cap_uniq);
     if (d_ws == nullptr || ws_bytes < p.ws_bytes) {
         set_error("sample_blocks: workspace too small (%zu < %zu)", ws_bytes, p.ws_bytes);

@@ -15,6 +15,8 @@
 //   2. mark       per edge: "am I the first edge of a new id?" -> one flag bit per edge
 //                 (8 edges per lane, one byte) + per-tile counts
 //   3. prefix     single workgroup over the tile counts; publishes the new node total
+//                 (the edge-parallel launches are grid-stride loops over the actual count,
+//                 so a bound much larger than the batch costs nothing)
 //   4. assign     per tile: scan of the flags -> local ids for the first edges; writes the
 //                 slot's val and appends the id to the unique list
 //   5. relabel    per edge: src_out[e] = val of the remembered slot
@@ -52,19 +54,21 @@ static inline TableRef make_ref(void* d_table, int64_t slots)
     return t;
 }
 
-__device__ __forceinline__ uint32_t load_key(const uint32_t* p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// A probe sequence longer than this is reported as "table full" (at load <= 1/2 with this
+// hash, sequences stay far below it), which also bounds the time a mis-sized table can cost.
+constexpr uint32_t kMaxProbes = 4096;
 
 // Finds the slot of `id`, inserting the key if absent.  Returns kEmpty if the table is full.
+// Keys only ever change from empty to a key, so an ordinary (cacheable, possibly stale) load
+// is enough for the first look: a stale "empty" is settled by the CAS, and a stale key cannot
+// exist.
 __device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id)
 {
     uint32_t p = (id * kHashMul) >> t.shift;
-    for (uint32_t n = 0; n <= t.mask; ++n) {
-        uint32_t k = load_key(&t.words[2 * (size_t)p]);
+    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
+    for (uint32_t n = 0; n < limit; ++n) {
+        uint32_t k = t.words[2 * (size_t)p];
         if (k == kEmpty) {
-            // a stale or racing view of an empty slot is settled by the CAS
             const uint32_t seen = atomicCAS(&t.words[2 * (size_t)p], kEmpty, id);
             k = (seen == kEmpty) ? id : seen;
         }
@@ -78,7 +82,8 @@ __device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id
 __device__ __forceinline__ uint32_t find_only(const uint32_t* __restrict__ words, uint32_t mask, int shift, uint32_t id)
 {
     uint32_t p = (id * kHashMul) >> shift;
-    for (uint32_t n = 0; n <= mask; ++n) {
+    const uint32_t limit = mask < kMaxProbes ? mask + 1 : kMaxProbes;
+    for (uint32_t n = 0; n < limit; ++n) {
         const uint32_t k = words[2 * (size_t)p];
         if (k == id) return p;
         if (k == kEmpty) return kEmpty;
@@ -110,21 +115,25 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
                                                                   uint32_t* __restrict__ slot_of, uint32_t* __restrict__ d_status)
 {
     const int64_t n_e = actual_count(e_max, d_e);
-    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (e >= n_e) return;
     const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
-    const uint32_t id = (uint32_t)src[e];
-    const uint32_t p = find_or_insert(t, id);
-    slot_of[e] = p;
-    if (p == kEmpty) {
-        if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
-        return;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
+        const uint32_t id = (uint32_t)src[e];
+        const uint32_t p = find_or_insert(t, id);
+        slot_of[e] = p;
+        if (p == kEmpty) {
+            if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+            continue;
+        }
+        uint32_t* val = &t.words[2 * (size_t)p + 1];
+        const uint32_t mine = n_base + (uint32_t)e;
+        // ids numbered earlier (val < n_base) are final; otherwise keep the smallest edge index.
+        // val only decreases while this kernel runs, so a stale read can only cause a redundant atomic.
+        if (*val > mine) atomicMin(val, mine);
     }
-    uint32_t* val = &t.words[2 * (size_t)p + 1];
-    const uint32_t mine = n_base + (uint32_t)e;
-    // ids numbered earlier (val < n_base) are final; otherwise keep the smallest edge index
-    if (__hip_atomic_load(val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > mine) atomicMin(val, mine);
 }
+
+__device__ __forceinline__ int64_t tiles_of(int64_t n) { return (n + kTile - 1) / kTile; }
 
 // flags8[tile*256 + lane] bit j  <=>  edge (tile*2048 + lane*8 + j) is the first edge of a new id
 __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
@@ -135,35 +144,55 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
-    const int64_t first = (int64_t)blockIdx.x * kTile + (int64_t)threadIdx.x * kItems;
-    uint32_t bits = 0;
+    const int64_t n_tiles = tiles_of(n_e);
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t first = tile * kTile + (int64_t)threadIdx.x * kItems;
+        uint32_t p[kItems];
 #pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-        const int64_t e = first + j;
-        if (e < n_e) {
-            const uint32_t p = slot_of[e];
-            if (p != kEmpty && t.words[2 * (size_t)p + 1] == n_base + (uint32_t)e) bits |= 1u << j;
-        }
+        for (int j = 0; j < kItems; ++j) p[j] = (first + j < n_e) ? slot_of[first + j] : kEmpty;
+        uint32_t v[kItems];
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) v[j] = (p[j] != kEmpty) ? t.words[2 * (size_t)p[j] + 1] : 0u;
+        uint32_t bits = 0;
+#pragma unroll
+        for (int j = 0; j < kItems; ++j)
+            if (p[j] != kEmpty && v[j] == n_base + (uint32_t)(first + j)) bits |= 1u << j;
+        flags8[tile * kBlock + threadIdx.x] = (uint8_t)bits;
+        int total;
+        (void)block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
+        if (threadIdx.x == 0) tile_sums[tile] = total;
     }
-    flags8[(int64_t)blockIdx.x * kBlock + threadIdx.x] = (uint8_t)bits;
-    int total;
-    (void)block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
-    if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
-// n_total = n_base + (number of new ids), clamped to the capacity of the unique list
-__global__ void idmap_publish_total_kernel(const int32_t* __restrict__ new_count, int64_t n_base_h,
-                                           const int32_t* __restrict__ d_n_base, int64_t capacity,
-                                           int32_t* __restrict__ d_n_total_out, uint32_t* __restrict__ d_status)
+// One workgroup: exclusive scan of the per-tile counts of new ids, then
+// n_total = n_base + (number of new ids), clamped to the capacity of the unique list.
+__global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_t* __restrict__ tile_sums,
+                                                                    int32_t* __restrict__ tile_prefix, int64_t e_max,
+                                                                    const int32_t* __restrict__ d_e, int64_t n_base_h,
+                                                                    const int32_t* __restrict__ d_n_base, int64_t capacity,
+                                                                    int32_t* __restrict__ d_n_total_out,
+                                                                    uint32_t* __restrict__ d_status)
 {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-    int64_t total = n_base + (int64_t)(*new_count);
-    if (total > capacity) {
-        if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
-        total = capacity;
+    __shared__ int smem[1024 / kWave + 1];
+    const int n_tiles = (int)tiles_of(actual_count(e_max, d_e));
+    int carry = 0;
+    for (int start = 0; start < n_tiles; start += 1024) {
+        const int i = start + (int)threadIdx.x;
+        const int v = i < n_tiles ? tile_sums[i] : 0;
+        int total;
+        const int ex = block_exclusive_scan<1024>(v, smem, &total);
+        if (i < n_tiles) tile_prefix[i] = carry + ex;
+        carry += total;
     }
-    if (d_n_total_out) *d_n_total_out = (int32_t)total;
+    if (threadIdx.x == 0) {
+        const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
+        int64_t total = n_base + (int64_t)carry;
+        if (total > capacity) {
+            if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
+            total = capacity;
+        }
+        if (d_n_total_out) *d_n_total_out = (int32_t)total;
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void idmap_assign_kernel(TableRef t, const int32_t* __restrict__ src, int64_t e_max,
@@ -177,19 +206,22 @@ __global__ __launch_bounds__(kBlock) void idmap_assign_kernel(TableRef t, const 
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-    const int64_t first = (int64_t)blockIdx.x * kTile + (int64_t)threadIdx.x * kItems;
-    const uint32_t bits = first < n_e ? flags8[(int64_t)blockIdx.x * kBlock + threadIdx.x] : 0u;
-    int total;
-    int64_t local = n_base + tile_prefix[blockIdx.x] + block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
+    const int64_t n_tiles = tiles_of(n_e);
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t first = tile * kTile + (int64_t)threadIdx.x * kItems;
+        const uint32_t bits = first < n_e ? flags8[tile * kBlock + threadIdx.x] : 0u;
+        int total;
+        int64_t local = n_base + tile_prefix[tile] + block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
 #pragma unroll
-    for (int j = 0; j < kItems; ++j) {
-        if (bits & (1u << j)) {
-            const int64_t e = first + j;
-            if (local < capacity) {
-                t.words[2 * (size_t)slot_of[e] + 1] = (uint32_t)local;
-                uniq[local] = src[e];
+        for (int j = 0; j < kItems; ++j) {
+            if (bits & (1u << j)) {
+                const int64_t e = first + j;
+                if (local < capacity) {
+                    t.words[2 * (size_t)slot_of[e] + 1] = (uint32_t)local;
+                    uniq[local] = src[e];
+                }
+                ++local;
             }
-            ++local;
         }
     }
 }
@@ -199,25 +231,36 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_kernel(TableRef t, int64
                                                                int32_t* __restrict__ out)
 {
     const int64_t n_e = actual_count(e_max, d_e);
-    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (e >= n_e) return;
-    const uint32_t p = slot_of[e];
-    out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
+        const uint32_t p = slot_of[e];
+        out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void idmap_lookup_kernel(TableRef t, int32_t* __restrict__ ids, int64_t n_max,
                                                               const int32_t* __restrict__ d_n, uint32_t* __restrict__ d_status)
 {
     const int64_t n = actual_count(n_max, d_n);
-    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    const uint32_t p = find_only(t.words, t.mask, t.shift, (uint32_t)ids[i]);
-    if (p == kEmpty) {
-        if (d_status) atomicOr(d_status, FGL_STATUS_MISSING_KEY);
-        ids[i] = -1;
-    } else {
-        ids[i] = (int32_t)t.words[2 * (size_t)p + 1];
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        const uint32_t p = find_only(t.words, t.mask, t.shift, (uint32_t)ids[i]);
+        if (p == kEmpty) {
+            if (d_status) atomicOr(d_status, FGL_STATUS_MISSING_KEY);
+            ids[i] = -1;
+        } else {
+            ids[i] = (int32_t)t.words[2 * (size_t)p + 1];
+        }
     }
+}
+
+// Workgroups for a grid-stride pass over n items: enough to fill every CU several times
+// over, never more than the work needs.
+static inline unsigned stride_grid(int64_t n_items, int items_per_block)
+{
+    int64_t blocks = ceil_div(n_items > 0 ? n_items : 1, items_per_block);
+    if (blocks > 8192) blocks = 8192;
+    return (unsigned)blocks;
 }
 
 // ---- launchers ------------------------------------------------------------------
@@ -232,6 +275,7 @@ int launch_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_i
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE(n_max >= 0 && n_max <= slots / 2, "idmap_insert_dst: %lld ids do not fit %lld slots at load 1/2", (long long)n_max, (long long)slots);
+    FGL_REQUIRE(n_max <= 0x7FFFFFFF, "idmap_insert_dst: too many ids");
     if (n_max == 0) return FGL_OK;
     FGL_REQUIRE(d_dst_ids != nullptr, "idmap_insert_dst: null ids");
     const int64_t blocks = ceil_div(n_max, kBlock);
@@ -249,7 +293,6 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
     c.take<uint8_t>((size_t)tiles * kBlock);    // flags8
     c.take<int32_t>((size_t)tiles);             // tile sums
     c.take<int32_t>((size_t)tiles);             // tile prefix
-    c.take<int32_t>(1);                         // new id count
     return c.used();
 }
 
@@ -262,7 +305,6 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     FGL_REQUIRE(flags == FGL_IDMAP_ORDERED, "idmap_map_src: unknown flags %d", flags);
     FGL_REQUIRE(n_edges_max >= 0 && n_base >= 0 && uniq_capacity >= 0, "idmap_map_src: negative size");
     FGL_REQUIRE(n_base + n_edges_max <= 0xFFFFFFFEll, "idmap_map_src: n_base + n_edges exceeds 32 bits");
-    FGL_REQUIRE(uniq_capacity <= slots / 2, "idmap_map_src: %lld unique ids do not fit %lld slots at load 1/2", (long long)uniq_capacity, (long long)slots);
     FGL_REQUIRE(n_edges_max == 0 || (d_src_in && d_src_out && d_uniq), "idmap_map_src: null pointer");
     FGL_REQUIRE(d_n_total_out == nullptr || d_n_total_out != d_n_base, "idmap_map_src: n_total_out must not alias n_base");
     if (d_ws == nullptr || ws_bytes < idmap_map_src_workspace_bytes(n_edges_max)) {
@@ -275,25 +317,23 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     uint8_t* flags8 = c.take<uint8_t>((size_t)tiles * kBlock);
     int32_t* sums = c.take<int32_t>((size_t)tiles);
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
-    int32_t* new_count = c.take<int32_t>(1);
     const TableRef t = make_ref(d_table, slots);
-    const int64_t edge_blocks = ceil_div(n_edges_max > 0 ? n_edges_max : 1, kBlock);
+    const unsigned edge_blocks = stride_grid(n_edges_max, kBlock);
+    const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
 
-    hipLaunchKernelGGL(idmap_insert_src_kernel, dim3((unsigned)edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+    hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, d_status);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
-    hipLaunchKernelGGL(idmap_mark_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges, n_base,
+    hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges, n_base,
                        d_n_base, slot_of, flags8, sums);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
-    int rc = launch_tile_prefix(sums, (int)tiles, prefix, new_count, nullptr, nullptr, 0, nullptr, stream);
-    if (rc != FGL_OK) return rc;
-    hipLaunchKernelGGL(idmap_publish_total_kernel, dim3(1), dim3(64), 0, stream, new_count, n_base, d_n_base, uniq_capacity,
-                       d_n_total_out, d_status);
-    FGL_CHECK_LAUNCH("idmap_publish_total_kernel");
-    hipLaunchKernelGGL(idmap_assign_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
+    hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max, d_n_edges,
+                       n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
+    FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
+    hipLaunchKernelGGL(idmap_assign_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
                        d_n_edges, n_base, d_n_base, slot_of, flags8, prefix, d_uniq, uniq_capacity);
     FGL_CHECK_LAUNCH("idmap_assign_kernel");
-    hipLaunchKernelGGL(idmap_relabel_kernel, dim3((unsigned)edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max,
+    hipLaunchKernelGGL(idmap_relabel_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max,
                        d_n_edges, slot_of, d_src_out);
     FGL_CHECK_LAUNCH("idmap_relabel_kernel");
     return FGL_OK;
@@ -351,8 +391,7 @@ FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_i
     FGL_REQUIRE(n_max >= 0, "idmap_lookup: negative size");
     if (n_max == 0) return FGL_OK;
     FGL_REQUIRE(d_ids != nullptr, "idmap_lookup: null ids");
-    const int64_t blocks = ceil_div(n_max, kBlock);
-    hipLaunchKernelGGL(idmap_lookup_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream),
+    hipLaunchKernelGGL(idmap_lookup_kernel, dim3(stride_grid(n_max, kBlock)), dim3(kBlock), 0, as_stream(stream),
                        make_ref(const_cast<void*>(d_table), slots), d_ids, n_max, d_n, d_status);
     FGL_CHECK_LAUNCH("idmap_lookup_kernel");
     return FGL_OK;

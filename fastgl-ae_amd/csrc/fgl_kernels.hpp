@@ -9,9 +9,10 @@ size_t scan_workspace_bytes(int64_t n_max);
 int launch_exclusive_sum(const int32_t* d_in, int64_t n_max, const int32_t* d_n, int32_t* d_out,
                          int32_t* d_total_extra, void* d_ws, size_t ws_bytes, hipStream_t stream);
 // single-workgroup scan of per-tile sums; the total is written to *total_a, *total_b and
-// at_count_base[actual count of (n_max, d_n)] (each optional)
+// at_count_base[actual count of (n_max, d_n)] (each optional); tile_items > 0 restricts the
+// scan to the tiles the actual count occupies
 int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_prefix, int32_t* total_a,
-                       int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n,
+                       int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n, int tile_items,
                        hipStream_t stream);
 int launch_fill_u32(uint32_t* p, int64_t n, uint32_t value, hipStream_t stream);
 

@@ -11,6 +11,8 @@
 //                             then a flat pass over the tile's output edges so that the
 //                             src/dst writes are fully coalesced and the copy-all rows read
 //                             `indices` contiguously.
+// Launches 1 and 3 are grid-stride loops over the tiles the actual seed count occupies, so
+// a host-side bound far above the actual count costs nothing.
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
@@ -25,33 +27,36 @@ __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restric
 {
     __shared__ int smem[TS / kWave + 1];
     const int64_t n = actual_count(n_max, d_n);
-    const int64_t i = (int64_t)blockIdx.x * TS + threadIdx.x;
-    int k = 0;
-    if (i < n) {
-        const int64_t s = seeds[i];
-        int64_t a = 0, deg = 0;
-        if (s >= 0 && s < n_nodes) {
-            if (is64) {
-                const int64_t* p = static_cast<const int64_t*>(indptr);
-                a = p[s];
-                deg = p[s + 1] - a;
-            } else {
-                const int32_t* p = static_cast<const int32_t*>(indptr);
-                a = p[s];
-                deg = (int64_t)p[s + 1] - a;
+    const int64_t n_tiles = (n + TS - 1) / TS;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i = tile * TS + threadIdx.x;
+        int k = 0;
+        if (i < n) {
+            const int64_t s = seeds[i];
+            int64_t a = 0, deg = 0;
+            if (s >= 0 && s < n_nodes) {
+                if (is64) {
+                    const int64_t* p = static_cast<const int64_t*>(indptr);
+                    a = p[s];
+                    deg = p[s + 1] - a;
+                } else {
+                    const int32_t* p = static_cast<const int32_t*>(indptr);
+                    a = p[s];
+                    deg = (int64_t)p[s + 1] - a;
+                }
+                if (deg < 0) deg = 0;
+                if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
+            } else if (d_status) {
+                atomicOr(d_status, FGL_STATUS_BAD_SEED);
             }
-            if (deg < 0) deg = 0;
-            if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
-        } else if (d_status) {
-            atomicOr(d_status, FGL_STATUS_BAD_SEED);
+            row_start[i] = a;
+            deg_out[i] = (int32_t)deg;
+            k = deg < fanout ? (int)deg : fanout;
         }
-        row_start[i] = a;
-        deg_out[i] = (int32_t)deg;
-        k = deg < fanout ? (int)deg : fanout;
+        int total;
+        (void)block_exclusive_scan<TS>(k, smem, &total);
+        if (threadIdx.x == 0) tile_sums[tile] = total;
     }
-    int total;
-    (void)block_exclusive_scan<TS>(k, smem, &total);
-    if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
 template <int TS>
@@ -74,50 +79,73 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
 
     const int tid = (int)threadIdx.x;
     const int64_t n = actual_count(n_max, d_n);
-    const int64_t i = (int64_t)blockIdx.x * TS + tid;
-    int deg = 0, seed = 0;
-    int64_t row = 0;
-    if (i < n) {
-        deg = deg_arr[i];
-        row = row_start[i];
-        seed = seeds[i];
-    }
-    const int k = deg < fanout ? deg : fanout;
-    int total;
-    const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-    const int base = tile_prefix[blockIdx.x];
-    s_off[tid] = ex;
-    if (tid == 0) s_off[TS] = total;
-    s_row[tid] = row;
-    s_deg[tid] = deg;
-    s_seed[tid] = seed;
-    if (i < n) block_ptr[i] = base + ex;
-
-    if (deg > fanout) {
-        // Floyd: for j = deg-k .. deg-1 draw t in [0, j]; take t unless already taken, else j.
-        uint32_t o[4];
-        for (int m = 0; m < fanout; ++m) {
-            if ((m & 1) == 0) philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32), stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
-            const uint64_t r = (m & 1) ? ((uint64_t)o[2] | ((uint64_t)o[3] << 32)) : ((uint64_t)o[0] | ((uint64_t)o[1] << 32));
-            const uint32_t j = (uint32_t)(deg - fanout + m);
-            const uint32_t t = (uint32_t)__umul64hi(r, (uint64_t)j + 1u);
-            bool dup = false;
-            for (int q = 0; q < m; ++q) dup |= (s_sel[q * TS + tid] == t);
-            s_sel[m * TS + tid] = dup ? j : t;
+    const int64_t n_tiles = (n + TS - 1) / TS;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i = tile * TS + tid;
+        int deg = 0, seed = 0;
+        int64_t row = 0;
+        if (i < n) {
+            deg = deg_arr[i];
+            row = row_start[i];
+            seed = seeds[i];
         }
-    }
-    __syncthreads();
+        const int k = deg < fanout ? deg : fanout;
+        int total;
+        const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
+        const int base = tile_prefix[tile];
+        s_off[tid] = ex;
+        if (tid == 0) s_off[TS] = total;
+        s_row[tid] = row;
+        s_deg[tid] = deg;
+        s_seed[tid] = seed;
+        if (i < n) block_ptr[i] = base + ex;
 
-    for (int x = tid; x < total; x += TS) {
-        int lo = 0, hi = TS;  // s_off[lo] <= x < s_off[hi]
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (s_off[mid] <= x) lo = mid; else hi = mid;
+        if (deg > fanout) {
+            // Floyd: for j = deg-k .. deg-1 draw t in [0, j]; take t unless already taken, else j.
+            uint32_t o[4];
+            for (int m = 0; m < fanout; ++m) {
+                if ((m & 1) == 0) philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32), stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
+                const uint64_t r = (m & 1) ? ((uint64_t)o[2] | ((uint64_t)o[3] << 32)) : ((uint64_t)o[0] | ((uint64_t)o[1] << 32));
+                const uint32_t j = (uint32_t)(deg - fanout + m);
+                const uint32_t t = (uint32_t)__umul64hi(r, (uint64_t)j + 1u);
+                bool dup = false;
+                for (int q = 0; q < m; ++q) dup |= (s_sel[q * TS + tid] == t);
+                s_sel[m * TS + tid] = dup ? j : t;
+            }
         }
-        const int j = x - s_off[lo];
-        const int64_t pos = s_deg[lo] <= fanout ? (int64_t)j : (int64_t)s_sel[j * TS + lo];
-        src_out[(int64_t)base + x] = indices[s_row[lo] + pos];
-        if (dst_out) dst_out[(int64_t)base + x] = s_seed[lo];
+        __syncthreads();
+
+        // flat pass over the tile's output edges, four independent gathers in flight per lane
+        for (int x0 = tid; x0 < total; x0 += 4 * TS) {
+            int seed_of[4];
+            int32_t got[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int x = x0 + u * TS;
+                got[u] = 0;
+                seed_of[u] = 0;
+                if (x < total) {
+                    int lo = 0, hi = TS;  // s_off[lo] <= x < s_off[hi]
+                    while (hi - lo > 1) {
+                        const int mid = (lo + hi) >> 1;
+                        if (s_off[mid] <= x) lo = mid; else hi = mid;
+                    }
+                    const int j = x - s_off[lo];
+                    const int64_t pos = s_deg[lo] <= fanout ? (int64_t)j : (int64_t)s_sel[j * TS + lo];
+                    got[u] = indices[s_row[lo] + pos];
+                    seed_of[u] = s_seed[lo];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int x = x0 + u * TS;
+                if (x < total) {
+                    src_out[(int64_t)base + x] = got[u];
+                    if (dst_out) dst_out[(int64_t)base + x] = seed_of[u];
+                }
+            }
+        }
+        __syncthreads();  // the tile's LDS is reused by the next iteration
     }
 }
 
@@ -149,14 +177,15 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     int32_t* sums = c.take<int32_t>((size_t)tiles);
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
 
-    hipLaunchKernelGGL(sample_degree_kernel<TS>, dim3((unsigned)tiles), dim3(TS), 0, stream, d_indptr, indptr_is64,
+    const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    hipLaunchKernelGGL(sample_degree_kernel<TS>, dim3(grid), dim3(TS), 0, stream, d_indptr, indptr_is64,
                        n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
     FGL_CHECK_LAUNCH("sample_degree_kernel");
-    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds,
+    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds, TS,
                                 stream);
     if (rc != FGL_OK) return rc;
     const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
-    hipLaunchKernelGGL(sample_edges_kernel<TS>, dim3((unsigned)tiles), dim3(TS), lds, stream, d_indices, d_seeds,
+    hipLaunchKernelGGL(sample_edges_kernel<TS>, dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,
                        (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr);
     FGL_CHECK_LAUNCH("sample_edges_kernel");

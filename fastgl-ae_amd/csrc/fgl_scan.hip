@@ -40,15 +40,20 @@ __global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(const int32_t* _
 }
 
 // One workgroup: tile_prefix[t] = sum of tile_sums[0..t).  The grand total goes to
-// *total_a and *total_b and to at_count_base[actual count] (each optional).
+// *total_a and *total_b and to at_count_base[actual count] (each optional).  With
+// tile_items > 0 only the tiles that the actual count occupies are read.
 __global__ __launch_bounds__(1024) void scan_tile_prefix_kernel(const int32_t* __restrict__ tile_sums, int n_tiles,
                                                                 int32_t* __restrict__ tile_prefix,
                                                                 int32_t* __restrict__ total_a,
                                                                 int32_t* __restrict__ total_b,
                                                                 int32_t* __restrict__ at_count_base, int64_t n_max,
-                                                                const int32_t* __restrict__ d_n)
+                                                                const int32_t* __restrict__ d_n, int tile_items)
 {
     __shared__ int smem[1024 / kWave + 1];
+    if (tile_items > 0) {
+        const int64_t used = (actual_count(n_max, d_n) + tile_items - 1) / tile_items;
+        if (used < n_tiles) n_tiles = (int)used;
+    }
     int carry = 0;
     for (int start = 0; start < n_tiles; start += 1024) {
         const int t = start + (int)threadIdx.x;
@@ -66,11 +71,11 @@ __global__ __launch_bounds__(1024) void scan_tile_prefix_kernel(const int32_t* _
 }
 
 int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_prefix, int32_t* total_a,
-                       int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n,
+                       int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n, int tile_items,
                        hipStream_t stream)
 {
     hipLaunchKernelGGL(scan_tile_prefix_kernel, dim3(1), dim3(1024), 0, stream, tile_sums, n_tiles, tile_prefix,
-                       total_a, total_b, at_count_base, n_max, d_n);
+                       total_a, total_b, at_count_base, n_max, d_n, tile_items);
     FGL_CHECK_LAUNCH("scan_tile_prefix_kernel");
     return FGL_OK;
 }
@@ -127,7 +132,7 @@ int launch_exclusive_sum(const int32_t* d_in, int64_t n_max, const int32_t* d_n,
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
     hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, sums);
     FGL_CHECK_LAUNCH("scan_tile_sums_kernel");
-    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_total_extra, nullptr, nullptr, 0, nullptr, stream);
+    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_total_extra, nullptr, nullptr, 0, nullptr, 0, stream);
     if (rc != FGL_OK) return rc;
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, prefix,
                        d_out);

@@ -338,14 +338,16 @@ class BlocksPlan:
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
-                        keep_global=(0,)):
+                        keep_global=(0,), table_slots=None):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
     src_global[h] or None, counts)``; hop 0 expands the raw seeds.  ``counts`` (int32,
     ``2*n_hops + 2``) holds the node count before each hop and after the last, then the
     edge count of each hop, then the status word; the caller reads it once per batch.
-    ``keep_global`` lists the hops (negative = from the end) whose pre-relabel source ids are kept."""
+    ``keep_global`` lists the hops (negative = from the end) whose pre-relabel source ids are kept.
+    ``table_slots`` (a power of two, default the plan's worst case) uses only that much of the
+    hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
     _check_input(indices, "indices", _I32)
     _check_input(seeds, "seeds", _I32)
@@ -354,6 +356,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         raise RuntimeError("plan was made for %d seeds, got %d" % (plan.n_seeds, seeds.numel()))
     H = plan.n_hops
     keep = {(h + H) % H for h in keep_global}
+    slots = plan.slots if table_slots is None else min(int(table_slots), plan.slots)
     lib = L.lib()
     with torch.cuda.device(dev):
         uniq = torch.empty(max(plan.cap_uniq, 1), dtype=torch.int32, device=dev)
@@ -366,7 +369,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF,
-                                      L.ptr(plan.table), plan.slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
+                                      L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
                                       L.stream_handle()))
     return uniq, block_ptr, src_local, src_global, counts

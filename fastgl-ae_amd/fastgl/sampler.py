@@ -104,6 +104,7 @@ class FusedMapSampler:
         self.edge_ptr = None  # CSR indptr (int32 or int64)
         self.output_nodes = None
         self._plans = {}
+        self._uniq_seen = 0  # largest number of unique nodes any mini-batch has produced
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
         self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
@@ -133,11 +134,26 @@ class FusedMapSampler:
         if plan is None:
             plan = ops.BlocksPlan(self.nodes_num, int(seeds.numel()), hop_fanouts, seeds.device)
             self._plans = {key: plan}
-        uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
-                                                                   self.rng_seed, stream_base, keep_global=(H - 1,))
-        c = counts.tolist()  # the one host synchronisation of the mini-batch
-        if c[2 * H + 1]:
-            ops._raise_status(c[2 * H + 1], "sample_blocks")
+        # The plan's table can never overflow but is sized for batches without any repeated
+        # neighbour.  Real batches are far smaller, and a table that fits the caches is much
+        # faster, so after the first batch the table is sized from the largest batch seen (load
+        # <= 1/4); a batch that still outgrows it is detected by the kernels and simply redone
+        # with the full table.  Results do not depend on the table size.
+        slots_for = ops.L.lib().fgl_idmap_slots
+        slots = plan.slots if self._uniq_seen == 0 else min(plan.slots, max(slots_for(2 * self._uniq_seen), slots_for(plan.n_seeds)))
+        while True:
+            uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
+                                                                       self.rng_seed, stream_base, keep_global=(H - 1,),
+                                                                       table_slots=slots)
+            c = counts.tolist()  # the one host synchronisation of the mini-batch
+            status = c[2 * H + 1]
+            if status & ops.L.STATUS_TABLE_FULL and slots < plan.slots:
+                slots = plan.slots
+                continue
+            break
+        if status:
+            ops._raise_status(status, "sample_blocks")
+        self._uniq_seen = max(self._uniq_seen, c[H])
         blocks = []
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]

@@ -150,7 +150,10 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  *
  * fgl_sample_blocks_plan fills, for the given bounds, cap_dst[h] (max seeds of hop h),
  * cap_edges[h] (max edges of hop h), *cap_uniq (max unique ids overall), *table_slots
- * and *ws_bytes.
+ * (the slot count that can never overflow) and *ws_bytes.  fgl_sample_blocks also accepts a
+ * smaller power-of-two table (at least fgl_idmap_slots(n_seeds)), which stays cache-resident
+ * when batches are far below the bound; a batch that outgrows it sets FGL_STATUS_TABLE_FULL
+ * in the status word, its outputs are then invalid and the caller repeats it with more slots.
  *
  * Outputs (device): block_ptr[h] int32[cap_dst[h]+1], src_local[h] int32[cap_edges[h]],
  * src_global[h] int32[cap_edges[h]] or NULL; d_uniq int32[cap_uniq];

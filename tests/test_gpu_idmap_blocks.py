@@ -131,3 +131,22 @@ def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     seeds = np.arange(100, 612, dtype=np.int32)
     got = sampler.sample_blocks(None, torch.from_numpy(seeds.astype(np.int64)).to(cuda))  # DataLoader seeds are int64
     check_blocks(oracle, indptr, indices, seeds, [4, 4], got, 1, 0)
+
+
+def test_undersized_table_is_detected_and_redone(cuda, oracle, small_graph):
+    """The sampler sizes its hash table from earlier batches; a batch that outgrows it must be
+    caught by the kernels (status word) and repeated with the worst-case table, with the same result."""
+    import fastgl
+    print("sample_blocks undersized table", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=9).set_graph(ptr, idx)
+    sampler._uniq_seen = 1  # pretend earlier batches were tiny: the table only fits the seeds
+    seeds = np.random.default_rng(3).permutation(indptr.size - 1)[:512].astype(np.int32)
+    got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+    check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], got, 9, 0)
+    assert sampler._uniq_seen == got[0].numel() > 2 * 512
+    # the raw entry point reports the overflow instead of faulting or spinning
+    plan = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda)
+    out = fastgl.sample_blocks_fused(plan, ptr, idx, dev_i32(seeds, cuda), 9, 0, table_slots=1024)
+    assert out[4].tolist()[-1] & 1  # FGL_STATUS_TABLE_FULL
