@@ -17,8 +17,6 @@
 
 namespace fgl {
 
-template <int N>
-struct VecF32 { float v[N]; };
 
 // ---- vector load / store of VEC elements as fp32 -----------------------------------
 template <typename T, int VEC>
@@ -157,6 +155,9 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
             my_col = indices[base + gl];
             my_w = edge_weight<MODE>(my_col, row_factor, col_norm);
         }
+        // four row loads are issued before the first FMA; the tail of the list goes one by one
+        // (measured: longer or predicated unrolls gain nothing on long lists and lose up to 2x
+        // on the one- and two-entry lists of a transposed block)
         int t = 0;
         for (; t + 4 <= cnt; t += 4) {
             const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
