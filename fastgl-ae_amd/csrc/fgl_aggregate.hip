@@ -19,32 +19,42 @@ namespace fgl {
 
 
 // ---- vector load / store of VEC elements as fp32 -----------------------------------
+// Rows are moved with one 16-byte access per lane.  The vector types are declared with
+// 4-byte alignment: rows whose length is not a multiple of the vector (602 floats = 2408
+// bytes) start on 8- or 4-byte boundaries, and gfx950 global loads/stores of any width only
+// need dword alignment.  The last lane of a row whose length is not a multiple of VEC uses
+// the element-wise partial forms.
 template <typename T, int VEC>
 struct RowIO;
 
-template <int VEC>
-struct RowIO<float, VEC> {
-    using Raw = float __attribute__((ext_vector_type(VEC)));
+template <>
+struct RowIO<float, 4> {
+    typedef float Raw __attribute__((ext_vector_type(4), aligned(4)));
     static __device__ __forceinline__ Raw load(const float* p) { return *reinterpret_cast<const Raw*>(p); }
-    static __device__ __forceinline__ void fma(float (&acc)[VEC], float w, Raw r)
+    static __device__ __forceinline__ Raw load_partial(const float* p, int n)
     {
+        Raw r = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] += w * r[i];
+        for (int i = 0; i < 3; ++i)
+            if (i < n) r[i] = p[i];
+        return r;
     }
-    static __device__ __forceinline__ void store(float* p, const float (&acc)[VEC])
+    static __device__ __forceinline__ void fma(float (&acc)[4], float w, Raw r)
     {
-        Raw r;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) r[i] = acc[i];
+        for (int i = 0; i < 4; ++i) acc[i] += w * r[i];
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&acc)[4])
+    {
+        Raw r = {acc[0], acc[1], acc[2], acc[3]};
         *reinterpret_cast<Raw*>(p) = r;
     }
-};
-template <>
-struct RowIO<float, 1> {
-    using Raw = float;
-    static __device__ __forceinline__ Raw load(const float* p) { return *p; }
-    static __device__ __forceinline__ void fma(float (&acc)[1], float w, Raw r) { acc[0] += w * r; }
-    static __device__ __forceinline__ void store(float* p, const float (&acc)[1]) { *p = acc[0]; }
+    static __device__ __forceinline__ void store_partial(float* p, const float (&acc)[4], int n)
+    {
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+            if (i < n) p[i] = acc[i];
+    }
 };
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
@@ -56,48 +66,50 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
     return u >> 16;
 }
 
-// bf16 rows are moved as 32-bit words holding two elements (VEC is even) or as single halfwords.
-template <int VEC>
-struct RowIO<uint16_t, VEC> {
-    static_assert(VEC % 2 == 0, "bf16 vectors hold an even number of elements");
-    using Raw = uint32_t __attribute__((ext_vector_type(VEC / 2)));
+// bf16: eight elements per lane as four 32-bit words (rows must start on 4-byte boundaries)
+template <>
+struct RowIO<uint16_t, 8> {
+    typedef uint32_t Raw __attribute__((ext_vector_type(4), aligned(4)));
     static __device__ __forceinline__ Raw load(const uint16_t* p) { return *reinterpret_cast<const Raw*>(p); }
-    static __device__ __forceinline__ void fma(float (&acc)[VEC], float w, Raw r)
+    static __device__ __forceinline__ Raw load_partial(const uint16_t* p, int n)
+    {
+        Raw r = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 7; ++i)
+            if (i < n) r[i >> 1] |= (uint32_t)p[i] << ((i & 1) * 16);
+        return r;
+    }
+    static __device__ __forceinline__ void fma(float (&acc)[8], float w, Raw r)
     {
 #pragma unroll
-        for (int i = 0; i < VEC / 2; ++i) {
+        for (int i = 0; i < 4; ++i) {
             acc[2 * i] += w * bf16_bits_to_f32(r[i] & 0xFFFFu);
             acc[2 * i + 1] += w * bf16_bits_to_f32(r[i] >> 16);
         }
     }
-    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[VEC])
+    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[8])
     {
         Raw r;
 #pragma unroll
-        for (int i = 0; i < VEC / 2; ++i) r[i] = f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) r[i] = f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16);
         *reinterpret_cast<Raw*>(p) = r;
     }
-};
-template <>
-struct RowIO<uint16_t, 2> {
-    using Raw = uint32_t;
-    static __device__ __forceinline__ Raw load(const uint16_t* p) { return *reinterpret_cast<const uint32_t*>(p); }
-    static __device__ __forceinline__ void fma(float (&acc)[2], float w, Raw r)
+    static __device__ __forceinline__ void store_partial(uint16_t* p, const float (&acc)[8], int n)
     {
-        acc[0] += w * bf16_bits_to_f32(r & 0xFFFFu);
-        acc[1] += w * bf16_bits_to_f32(r >> 16);
-    }
-    static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[2])
-    {
-        *reinterpret_cast<uint32_t*>(p) = f32_to_bf16_bits(acc[0]) | (f32_to_bf16_bits(acc[1]) << 16);
+#pragma unroll
+        for (int i = 0; i < 7; ++i)
+            if (i < n) p[i] = (uint16_t)f32_to_bf16_bits(acc[i]);
     }
 };
+// bf16 rows that start on odd element boundaries: one element per lane
 template <>
 struct RowIO<uint16_t, 1> {
     using Raw = uint16_t;
     static __device__ __forceinline__ Raw load(const uint16_t* p) { return *p; }
+    static __device__ __forceinline__ Raw load_partial(const uint16_t* p, int) { return *p; }
     static __device__ __forceinline__ void fma(float (&acc)[1], float w, Raw r) { acc[0] += w * bf16_bits_to_f32(r); }
     static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[1]) { *p = (uint16_t)f32_to_bf16_bits(acc[0]); }
+    static __device__ __forceinline__ void store_partial(uint16_t* p, const float (&acc)[1], int) { store(p, acc); }
 };
 
 // per-edge weight, evaluated by the lane that loaded the neighbour id
@@ -128,7 +140,14 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
     const int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
     if (row >= n_rows) return;  // uniform per group: the cross-lane reads below stay inside the group
     const int col0 = ((int)blockIdx.y * LPR + gl) * VEC;
-    const bool live = col0 < D;
+    const int nvalid = D - col0;       // elements of this lane's vector that exist in the row
+    const bool live = nvalid > 0;
+    const bool full = nvalid >= VEC;   // false only for the last lane of a row with D % VEC != 0
+    auto load_row = [&](const T* p) { return full ? IO::load(p) : IO::load_partial(p, nvalid); };
+    auto store_row = [&](T* p, const float (&a)[VEC]) {
+        if (full) IO::store(p, a);
+        else IO::store_partial(p, a, nvalid);
+    };
 
     const int a = indptr[row], b = indptr[row + 1];
     float acc[VEC];
@@ -137,8 +156,8 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
 
     if (a == b) {
         if (live) {
-            if (zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, IO::load(X + row * ldx + col0));
-            IO::store(out + row * ldo + col0, acc);
+            if (zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, load_row(X + row * ldx + col0));
+            store_row(out + row * ldo + col0, acc);
         }
         return;
     }
@@ -165,10 +184,10 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
             const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
             const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
             if (live) {
-                const typename IO::Raw r0 = IO::load(X + (int64_t)c0 * ldx + col0);
-                const typename IO::Raw r1 = IO::load(X + (int64_t)c1 * ldx + col0);
-                const typename IO::Raw r2 = IO::load(X + (int64_t)c2 * ldx + col0);
-                const typename IO::Raw r3 = IO::load(X + (int64_t)c3 * ldx + col0);
+                const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r1 = load_row(X + (int64_t)c1 * ldx + col0);
+                const typename IO::Raw r2 = load_row(X + (int64_t)c2 * ldx + col0);
+                const typename IO::Raw r3 = load_row(X + (int64_t)c3 * ldx + col0);
                 IO::fma(acc, w0, r0);
                 IO::fma(acc, w1, r1);
                 IO::fma(acc, w2, r2);
@@ -178,10 +197,10 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
         for (; t < cnt; ++t) {
             const int c0 = __shfl(my_col, t, LPR);
             const float w0 = __shfl(my_w, t, LPR);
-            if (live) IO::fma(acc, w0, IO::load(X + (int64_t)c0 * ldx + col0));
+            if (live) IO::fma(acc, w0, load_row(X + (int64_t)c0 * ldx + col0));
         }
     }
-    if (live) IO::store(out + row * ldo + col0, acc);
+    if (live) store_row(out + row * ldo + col0, acc);
 }
 
 // ---- block transpose ---------------------------------------------------------------
@@ -271,16 +290,10 @@ static int launch_agg_vec(int mode, hipStream_t stream, const int32_t* indptr, c
     }
 }
 
-// widest vector (in elements) that the row length, both strides and both base addresses allow
-static int pick_vec(int D, int64_t ldx, int64_t ldo, const void* x, const void* out, int elem_bytes)
+// bf16 rows can be moved eight elements at a time when every row starts on a 4-byte boundary
+static bool bf16_rows_dword_aligned(int64_t ldx, int64_t ldo, const void* x, const void* out)
 {
-    int vec = 16 / elem_bytes;
-    while (vec > 1) {
-        const uintptr_t bytes = (uintptr_t)vec * elem_bytes;
-        if (D % vec == 0 && ldx % vec == 0 && ldo % vec == 0 && ((uintptr_t)x % bytes) == 0 && ((uintptr_t)out % bytes) == 0) break;
-        vec >>= 1;
-    }
-    return vec;
+    return ldx % 2 == 0 && ldo % 2 == 0 && ((uintptr_t)x % 4) == 0 && ((uintptr_t)out % 4) == 0;
 }
 
 }  // namespace fgl
@@ -304,23 +317,14 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     FGL_REQUIRE(d_indptr && d_indices && d_x && d_out, "aggregate: null pointer");
     FGL_REQUIRE(d_x != d_out, "aggregate: output aliases the input");
     hipStream_t s = as_stream(stream);
-    if (dtype == FGL_F32) {
-        const float* X = static_cast<const float*>(d_x);
-        float* O = static_cast<float*>(d_out);
-        switch (pick_vec(D, ldx, ldo, d_x, d_out, 4)) {
-            case 4: return launch_agg_vec<float, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-            case 2: return launch_agg_vec<float, 2>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-            default: return launch_agg_vec<float, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-        }
-    }
+    if (dtype == FGL_F32)
+        return launch_agg_vec<float, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, static_cast<const float*>(d_x), ldx, D,
+                                        zero_policy, d_row_norm, d_col_norm, static_cast<float*>(d_out), ldo);
     const uint16_t* X = static_cast<const uint16_t*>(d_x);
     uint16_t* O = static_cast<uint16_t*>(d_out);
-    switch (pick_vec(D, ldx, ldo, d_x, d_out, 2)) {
-        case 8: return launch_agg_vec<uint16_t, 8>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-        case 4: return launch_agg_vec<uint16_t, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-        case 2: return launch_agg_vec<uint16_t, 2>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-        default: return launch_agg_vec<uint16_t, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-    }
+    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out))
+        return launch_agg_vec<uint16_t, 8>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+    return launch_agg_vec<uint16_t, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
 }
 
 FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
