@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-batches", type=int, default=2, help="mini-batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
@@ -148,6 +151,14 @@ def main():
     rb.record()
     torch.cuda.synchronize()
     t_kernel0 = ra.elapsed_time(rb)
+
+    if args.pmc_copy_mib > 0:
+        a = torch.zeros(args.pmc_copy_mib << 20, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        b.copy_(a)  # __amd_rocclr_copyBuffer: reads and writes exactly pmc_copy_mib MiB
+        torch.cuda.synchronize()
+        del a, b
 
     # ---- reduce -------------------------------------------------------------------------
     tot_edges = 0

@@ -103,7 +103,8 @@ FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const in
 
 FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                                  const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                                 uint64_t rng_seed, uint32_t stream_base, void* d_table, int64_t table_slots,
+                                 uint64_t rng_seed, uint32_t stream_base, int idmap_flags, void* d_table,
+                                 int64_t table_slots,
                                  int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
                                  int32_t* const* src_local, int32_t* const* src_global, int32_t* d_counts, void* d_ws,
                                  size_t ws_bytes, void* stream)
@@ -145,7 +146,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
                            stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s);
         if (rc != FGL_OK) return rc;
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
-                                  d_counts + h + 1, d_uniq, uniq_capacity, FGL_IDMAP_ORDERED, d_status, ws + ws_sample,
+                                  d_counts + h + 1, d_uniq, uniq_capacity, idmap_flags, d_status, ws + ws_sample,
                                   ws_bytes - ws_sample, s);
         if (rc != FGL_OK) return rc;
     }

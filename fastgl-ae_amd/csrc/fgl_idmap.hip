@@ -254,6 +254,84 @@ __global__ __launch_bounds__(kBlock) void idmap_lookup_kernel(TableRef t, int32_
     }
 }
 
+// ---- arrival-order numbering (FGL_IDMAP_ARRIVAL) ---------------------------------------
+// The lane whose CAS installs a key numbers it at once from a global counter, as the
+// reference does (id_map.cu:314-321) -- but with one counter update per workgroup instead
+// of one per new id.  Two launches instead of five and about half the table traffic; the
+// numbering of new ids then depends on scheduling (any run is a valid map, and equal to
+// every other after sorting the new ids).
+__global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t, const int32_t* __restrict__ src,
+                                                                      int64_t e_max, const int32_t* __restrict__ d_e,
+                                                                      int64_t n_base_h, const int32_t* __restrict__ d_n_base,
+                                                                      uint32_t* __restrict__ slot_of, int32_t* __restrict__ counter,
+                                                                      int32_t* __restrict__ uniq, int64_t capacity,
+                                                                      uint32_t* __restrict__ d_status)
+{
+    __shared__ int smem[kBlock / kWave + 1];
+    __shared__ int s_base;
+    const int64_t n_e = actual_count(e_max, d_e);
+    const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t rounds = (n_e + stride - 1) / stride;  // same trip count for every lane: the loop holds barriers
+    for (int64_t r = 0; r < rounds; ++r) {
+        const int64_t e = r * stride + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+        uint32_t p = kEmpty, id = 0;
+        int won = 0;
+        if (e < n_e) {
+            id = (uint32_t)src[e];
+            uint32_t q = (id * kHashMul) >> t.shift;
+            const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
+            for (uint32_t n = 0; n < limit; ++n) {
+                uint32_t k = t.words[2 * (size_t)q];
+                if (k == kEmpty) {
+                    const uint32_t seen = atomicCAS(&t.words[2 * (size_t)q], kEmpty, id);
+                    if (seen == kEmpty) { won = 1; k = id; } else k = seen;
+                }
+                if (k == id) { p = q; break; }
+                q = (q + 1) & t.mask;
+            }
+            slot_of[e] = p;
+            if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+        }
+        int total;
+        const int rank = block_exclusive_scan<kBlock>(won, smem, &total);
+        if (threadIdx.x == 0) s_base = total ? atomicAdd(counter, total) : 0;
+        __syncthreads();
+        if (won) {
+            const int64_t local = n_base + s_base + rank;
+            if (local < capacity) {
+                t.words[2 * (size_t)p + 1] = (uint32_t)local;
+                uniq[local] = (int32_t)id;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
+                                                                       const uint32_t* __restrict__ slot_of,
+                                                                       int32_t* __restrict__ out, const int32_t* __restrict__ counter,
+                                                                       int64_t n_base_h, const int32_t* __restrict__ d_n_base,
+                                                                       int64_t capacity, int32_t* __restrict__ d_n_total_out,
+                                                                       uint32_t* __restrict__ d_status)
+{
+    const int64_t n_e = actual_count(e_max, d_e);
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
+        const uint32_t p = slot_of[e];
+        out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
+        int64_t total = n_base + (int64_t)(*counter);
+        if (total > capacity) {
+            if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
+            total = capacity;
+        }
+        if (d_n_total_out) *d_n_total_out = (int32_t)total;
+    }
+}
+
 // Workgroups for a grid-stride pass over n items: enough to fill every CU several times
 // over, never more than the work needs.
 static inline unsigned stride_grid(int64_t n_items, int items_per_block)
@@ -302,7 +380,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          size_t ws_bytes, hipStream_t stream)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
-    FGL_REQUIRE(flags == FGL_IDMAP_ORDERED, "idmap_map_src: unknown flags %d", flags);
+    FGL_REQUIRE(flags == FGL_IDMAP_ORDERED || flags == FGL_IDMAP_ARRIVAL, "idmap_map_src: unknown flags %d", flags);
     FGL_REQUIRE(n_edges_max >= 0 && n_base >= 0 && uniq_capacity >= 0, "idmap_map_src: negative size");
     FGL_REQUIRE(n_base + n_edges_max <= 0xFFFFFFFEll, "idmap_map_src: n_base + n_edges exceeds 32 bits");
     FGL_REQUIRE(n_edges_max == 0 || (d_src_in && d_src_out && d_uniq), "idmap_map_src: null pointer");
@@ -320,6 +398,19 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     const TableRef t = make_ref(d_table, slots);
     const unsigned edge_blocks = stride_grid(n_edges_max, kBlock);
     const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
+
+    if (flags == FGL_IDMAP_ARRIVAL) {
+        int32_t* counter = sums;  // one int of the (otherwise unused) tile-sum array
+        int rc0 = launch_fill_u32(reinterpret_cast<uint32_t*>(counter), 1, 0u, stream);
+        if (rc0 != FGL_OK) return rc0;
+        hipLaunchKernelGGL(idmap_insert_arrival_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
+                           d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_status);
+        FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
+        hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
+                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
+        FGL_CHECK_LAUNCH("idmap_relabel_publish_kernel");
+        return FGL_OK;
+    }
 
     hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, d_status);

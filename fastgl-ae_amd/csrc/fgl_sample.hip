@@ -7,7 +7,8 @@
 //   2. tile prefix            single workgroup; also writes block_ptr[n] and the edge count
 //   3. sample_edges_kernel    per tile of TS seeds: wave64 scan of k -> output offsets,
 //                             Floyd subset selection for rows longer than the fanout (one lane
-//                             per seed, picks kept in LDS, conflict-free [pick][seed] layout),
+//                             per seed, Philox stream keyed by the node id, picks kept in LDS in a
+//                             conflict-free [pick][seed] layout),
 //                             then a flat pass over the tile's output edges so that the
 //                             src/dst writes are fully coalesced and the copy-all rows read
 //                             `indices` contiguously.
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restric
     }
 }
 
-template <int TS>
+template <int TS, int U>
 __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restrict__ indices,
                                                           const int32_t* __restrict__ seeds, int64_t n_max,
                                                           const int32_t* __restrict__ d_n, int fanout,
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
             // Floyd: for j = deg-k .. deg-1 draw t in [0, j]; take t unless already taken, else j.
             uint32_t o[4];
             for (int m = 0; m < fanout; ++m) {
-                if ((m & 1) == 0) philox4x32_10((uint32_t)i, (uint32_t)((uint64_t)i >> 32), stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
+                if ((m & 1) == 0) philox4x32_10((uint32_t)seed, 0u, stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
                 const uint64_t r = (m & 1) ? ((uint64_t)o[2] | ((uint64_t)o[3] << 32)) : ((uint64_t)o[0] | ((uint64_t)o[1] << 32));
                 const uint32_t j = (uint32_t)(deg - fanout + m);
                 const uint32_t t = (uint32_t)__umul64hi(r, (uint64_t)j + 1u);
@@ -115,12 +116,13 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
         }
         __syncthreads();
 
-        // flat pass over the tile's output edges, four independent gathers in flight per lane
-        for (int x0 = tid; x0 < total; x0 += 4 * TS) {
-            int seed_of[4];
-            int32_t got[4];
+        // flat pass over the tile's output edges, U independent gathers in flight per lane
+        // (U * TS covers a whole tile for the common fanouts, so the pass is one round trip)
+        for (int x0 = tid; x0 < total; x0 += U * TS) {
+            int seed_of[U];
+            int32_t got[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int x = x0 + u * TS;
                 got[u] = 0;
                 seed_of[u] = 0;
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                 }
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int x = x0 + u * TS;
                 if (x < total) {
                     src_out[(int64_t)base + x] = got[u];
@@ -185,9 +187,14 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
                                 stream);
     if (rc != FGL_OK) return rc;
     const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
-    hipLaunchKernelGGL(sample_edges_kernel<TS>, dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,
-                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,
-                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr);
+#define FGL_LAUNCH_EDGES(U)                                                                                        \
+    hipLaunchKernelGGL((sample_edges_kernel<TS, U>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,          \
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
+                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr)
+    if (fanout <= 4) FGL_LAUNCH_EDGES(4);
+    else if (fanout <= 8) FGL_LAUNCH_EDGES(8);
+    else FGL_LAUNCH_EDGES(16);
+#undef FGL_LAUNCH_EDGES
     FGL_CHECK_LAUNCH("sample_edges_kernel");
     return FGL_OK;
 }

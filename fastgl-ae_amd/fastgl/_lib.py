@@ -20,7 +20,7 @@ F32, BF16 = 0, 1
 AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN = 0, 1, 2, 3
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED = 1, 2, 4, 8
-IDMAP_ORDERED = 0
+IDMAP_ORDERED, IDMAP_ARRIVAL = 0, 1
 MAX_FANOUT = 192
 
 _i64, _i32, _u64, _u32, _vp, _sz = C.c_int64, C.c_int, C.c_uint64, C.c_uint32, C.c_void_p, C.c_size_t
@@ -43,7 +43,7 @@ SIGNATURES = {
     "fgl_idmap_map_src": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _sz, _vp]),
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp]),
-    "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64]),
     "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _sz, _vp]),
     "fgl_aggregate": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),

@@ -338,7 +338,7 @@ class BlocksPlan:
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
-                        keep_global=(0,), table_slots=None):
+                        keep_global=(0,), table_slots=None, id_order="first"):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
@@ -347,7 +347,9 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     edge count of each hop, then the status word; the caller reads it once per batch.
     ``keep_global`` lists the hops (negative = from the end) whose pre-relabel source ids are kept.
     ``table_slots`` (a power of two, default the plan's worst case) uses only that much of the
-    hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL)."""
+    hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL).
+    ``id_order``: ``"first"`` numbers new ids by first occurrence (deterministic), ``"arrival"`` as
+    their inserts land (faster; any run is a valid map, equal to every other after sorting the new ids)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
     _check_input(indices, "indices", _I32)
     _check_input(seeds, "seeds", _I32)
@@ -369,7 +371,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF,
-                                      L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
+                                      {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order], L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
                                       L.stream_handle()))
     return uniq, block_ptr, src_local, src_global, counts

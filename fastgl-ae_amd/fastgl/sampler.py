@@ -81,7 +81,8 @@ class Block:
 
 class FusedMapSampler:
     def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
-                 prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0):
+                 prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0,
+                 id_order="first"):
         if mask is not None and prob is not None:
             raise ValueError('Mask and probability arguments are mutually exclusive. '
                              'Consider multiplying the probability with the mask to achieve the same goal.')
@@ -96,6 +97,9 @@ class FusedMapSampler:
         self.replace = replace
         self.output_device = output_device
         self.fused = fused
+        if id_order not in ("first", "arrival"):
+            raise ValueError("id_order must be 'first' or 'arrival'")
+        self.id_order = id_order  # numbering of new node ids (fused path): see ops.sample_blocks_fused
         self.rng_seed = int(rng_seed)
         self.batches = 0
         self.nodes_num = 0
@@ -144,7 +148,7 @@ class FusedMapSampler:
         while True:
             uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
                                                                        self.rng_seed, stream_base, keep_global=(H - 1,),
-                                                                       table_slots=slots)
+                                                                       table_slots=slots, id_order=self.id_order)
             c = counts.tolist()  # the one host synchronisation of the mini-batch
             status = c[2 * H + 1]
             if status & ops.L.STATUS_TABLE_FULL and slots < plan.slots:

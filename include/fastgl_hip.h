@@ -65,6 +65,8 @@ enum fgl_zero_policy {
 #define FGL_STATUS_BAD_SEED 8u     /* a seed id outside [0, n_nodes)        */
 
 #define FGL_IDMAP_ORDERED 0 /* new ids numbered by first occurrence (deterministic) */
+#define FGL_IDMAP_ARRIVAL 1 /* new ids numbered as their inserts land (the reference's rule,
+                               id_map.cu:314-321): fewer passes, order depends on scheduling */
 #define FGL_MAX_FANOUT 192
 
 int fgl_abi_version(void);
@@ -91,7 +93,8 @@ int fgl_cal_deg(const int32_t* d_ids, int64_t n_ids_max, const int32_t* d_n_ids,
  * d_src_out[block_ptr[i] + j] = j-th chosen in-neighbour (global id);
  * d_dst_out (optional, may be NULL) = s for each of those edges.
  * deg <= fanout copies the row in CSR order; otherwise a uniform random k-subset WITHOUT
- * replacement (Floyd) from Philox4x32-10 keyed by (rng_seed, stream_id, i).
+ * replacement (Floyd) from Philox4x32-10 keyed by (rng_seed, stream_id, s): what a node
+ * draws does not depend on its position in the seed list.
  * d_n_edges_out (optional) receives the edge count as int32.
  * d_src_out / d_dst_out need room for n_seeds_max * fanout entries.
  * ------------------------------------------------------------------------------- */
@@ -124,9 +127,10 @@ int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids,
 
 /* number the new source ids and relabel the edges (id_map.cu:290-383 for the src half).
  * n_base ids are already numbered (host value n_base, or *d_n_base when non-NULL).
- * New ids get n_base, n_base+1, ... in order of first occurrence in d_src_in and are
- * appended to d_uniq; d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
- * *d_n_total_out = n_base + number of new ids. */
+ * New ids get n_base, n_base+1, ... and are appended to d_uniq -- in order of first
+ * occurrence in d_src_in (flags = FGL_IDMAP_ORDERED) or of arrival (FGL_IDMAP_ARRIVAL);
+ * d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
+ * *d_n_total_out = n_base + number of new ids (must not alias d_n_base). */
 size_t fgl_idmap_map_src_workspace_bytes(int64_t n_edges_max);
 int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
                       int64_t n_edges_max, const int32_t* d_n_edges,
@@ -144,7 +148,8 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * sample_blocks -- all hops of FusedMapSampler.sample_blocks (FusedMapSampler.py:63-109)
  * in one call with no host synchronisation: per hop sample_node -> id-map, the table and
  * the numbering persisting across hops (hop h's unique list is hop h+1's seed list).
- * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0].
+ * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0];
+ * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL.
  * (The reference lists fanouts the other way round and iterates reversed(); the caller
  * passes them already reversed.)
  *
@@ -165,7 +170,7 @@ int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fano
                            int64_t* table_slots, size_t* ws_bytes);
 int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                       const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                      uint64_t rng_seed, uint32_t stream_base,
+                      uint64_t rng_seed, uint32_t stream_base, int idmap_flags,
                       void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
                       int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
                       int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);

@@ -16,7 +16,7 @@
  *
  * Deliberate departures from the reference (each one is also what the HIP library does):
  *   - random picks are WITHOUT replacement (Floyd's subset algorithm) from a
- *     Philox4x32-10 stream keyed by (rng_seed, stream_id, seed position); the reference
+ *     Philox4x32-10 stream keyed by (rng_seed, stream_id, node id); the reference
  *     draws curand()%deg with replacement from a per-launch-constant stream
  *     (sample.cu:70,91), which its own caller labels replace=False;
  *   - new source ids get local ids in first-occurrence order (one legal outcome of the
@@ -74,8 +74,9 @@ static inline uint64_t mulhi64(uint64_t a, uint64_t b)
     return (uint64_t)(((unsigned __int128)a * b) >> 64);
 }
 
-/* The m-th 64-bit draw of seed position `pos` in sampling stream `stream_id`.
- * Counter = {pos_lo, pos_hi, stream_id, m/2}, key = {seed_lo, seed_hi}; even m takes words
+/* The m-th 64-bit draw for node `pos` in sampling stream `stream_id` (the picks of a node
+ * depend on the node, the stream and the seed only -- not on where it sits in the seed list).
+ * Counter = {node_lo, node_hi, stream_id, m/2}, key = {seed_lo, seed_hi}; even m takes words
  * 0..1 of the block, odd m words 2..3. */
 static inline uint64_t sample_draw(uint64_t rng_seed, uint32_t stream_id, uint64_t pos, uint32_t m)
 {
@@ -139,7 +140,7 @@ ORC_API int64_t orc_sample_node(const void* indptr, int indptr_is64, const int32
                     if (dst_out) dst_out[off + j] = (int32_t)s;
                 }
             } else {
-                orc_floyd_subset(deg, fanout, rng_seed, stream_id, (uint64_t)i, sel);
+                orc_floyd_subset(deg, fanout, rng_seed, stream_id, (uint64_t)s, sel);
                 for (int j = 0; j < fanout; ++j) {
                     src_out[off + j] = indices[a + sel[j]];
                     if (dst_out) dst_out[off + j] = (int32_t)s;

@@ -150,3 +150,34 @@ def test_undersized_table_is_detected_and_redone(cuda, oracle, small_graph):
     plan = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda)
     out = fastgl.sample_blocks_fused(plan, ptr, idx, dev_i32(seeds, cuda), 9, 0, table_slots=1024)
     assert out[4].tolist()[-1] & 1  # FGL_STATUS_TABLE_FULL
+
+
+@pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64)])
+def test_arrival_order_equals_oracle_after_canonical_sort(cuda, oracle, small_graph, fanouts, batch):
+    """id_order="arrival" numbers new ids in scheduling order (the reference's rule), so local ids
+    differ from run to run; in graph ids -- the canonical form -- every hop must hold exactly the
+    oracle's edges, because what a node draws depends only on (seed, stream, node id)."""
+    import fastgl
+    print("sample_blocks arrival order %s" % fanouts, flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    sampler = fastgl.FusedMapSampler(fanouts, rng_seed=17, id_order="arrival").set_graph(ptr, idx)
+    seeds = np.random.default_rng(batch + 1).permutation(indptr.size - 1)[:batch].astype(np.int32)
+    for it in range(2):
+        inp, _, blocks = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        w_inp, w_blocks = oracle.sample_blocks(indptr, indices, seeds, fanouts, 17, it * 64)
+        uniq = inp.cpu().numpy()
+        assert np.array_equal(uniq[:batch], seeds)
+        assert np.unique(uniq).size == uniq.size
+        assert np.array_equal(np.sort(uniq), np.sort(w_inp))
+        for b, w in zip(blocks, w_blocks):
+            assert (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()) == (w["n_src"], w["n_dst"], w["src_local"].size)
+            src_l, dst_l = (t.cpu().numpy() for t in b.edges())
+            got = np.stack([uniq[dst_l], uniq[src_l]], 1)
+            w_dst = np.repeat(np.arange(w["n_dst"]), np.diff(w["indptr"]))
+            want = np.stack([w_inp[w_dst], w_inp[w["src_local"]]], 1)
+            assert np.array_equal(got[np.lexsort((got[:, 1], got[:, 0]))], want[np.lexsort((want[:, 1], want[:, 0]))])
+            # the block's node numbering is a prefix of the batch's: dst nodes first, in place
+            assert set(uniq[:b.num_src_nodes()].tolist()) == set(w_inp[:w["n_src"]].tolist())
+            if b.src_global is not None:
+                assert np.array_equal(uniq[src_l], b.src_global.cpu().numpy())

@@ -77,7 +77,7 @@ def test_uniform_inclusion_chi_square(oracle, deg, fanout):
     without replacement sum((O-E)^2/E) * (deg-1)/(deg-fanout) ~ chi2(deg-1)."""
     n = 20000
     indptr, indices = _ring_graph(n, deg)
-    seeds = np.arange(n, dtype=np.int32)
+    seeds = np.random.default_rng(deg).permutation(n).astype(np.int32)
     src, dst, ptr = oracle.sample_node(indptr, indices, seeds, fanout, rng_seed=123, stream_id=9)
     offs = (src.astype(np.int64) - dst - 1) % n          # position of the pick inside the row
     counts = np.bincount(offs, minlength=deg)
