@@ -51,6 +51,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-batches", type=int, default=2, help="mini-batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
+                    help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -94,7 +96,7 @@ def main():
     torch.cuda.synchronize()
     log("features %s x %d %s and %d training seeds in %.1fs" % (N, D, w["dtype"], w["train"], time.time() - t0))
 
-    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0).set_graph(edge_ptr, edge_src)
+    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
     L = len(w["fanouts"])
     # hidden activations / upstream gradients of the inner layers: synthetic, sized for the worst case
     plan_caps = fastgl.BlocksPlan(N, B, list(reversed(w["fanouts"])), dev).cap_dst
@@ -158,7 +160,9 @@ def main():
         torch.cuda.synchronize()
         b.copy_(a)  # __amd_rocclr_copyBuffer: reads and writes exactly pmc_copy_mib MiB
         torch.cuda.synchronize()
-        del a, b
+        c = a.view(torch.float32) * 1.0  # an ordinary elementwise kernel: reads and writes the same amount
+        torch.cuda.synchronize()
+        del a, b, c
 
     # ---- reduce -------------------------------------------------------------------------
     tot_edges = 0
@@ -223,7 +227,7 @@ def main():
         "dtype": w["dtype"],
         "data": "synthetic",
         "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
-                   "sampled_edges_per_step": tot_edges / K, "id_order": "first-occurrence (deterministic)",
+                   "sampled_edges_per_step": tot_edges / K, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
                    "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
                            "feature table); block transpose + bwd gather on the inner blocks; no dense layers"},
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,

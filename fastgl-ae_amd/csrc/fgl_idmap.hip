@@ -10,8 +10,8 @@
 // to_block gives -- instead of the reference's race on one global counter (id_map.cu:317-320).
 //
 // map_src = five launches:
-//   1. insert     per edge: probe, CAS the key in if new, atomicMin the first-edge index,
-//                 remember the slot
+//   1. insert     per edge: probe (one 8-byte load per slot), install {key, first-edge index}
+//                 with one 64-bit CAS if new, else atomicMin the first-edge index; remember the slot
 //   2. mark       per edge: "am I the first edge of a new id?" -> one flag bit per edge
 //                 (8 edges per lane, one byte) + per-tile counts
 //   3. prefix     single workgroup over the tile counts; publishes the new node total
@@ -58,21 +58,31 @@ static inline TableRef make_ref(void* d_table, int64_t slots)
 // hash, sequences stay far below it), which also bounds the time a mis-sized table can cost.
 constexpr uint32_t kMaxProbes = 4096;
 
-// Finds the slot of `id`, inserting the key if absent.  Returns kEmpty if the table is full.
-// Keys only ever change from empty to a key, so an ordinary (cacheable, possibly stale) load
-// is enough for the first look: a stale "empty" is settled by the CAS, and a stale key cannot
-// exist.
-__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id)
+// Finds the slot of `id`, inserting {id, val_if_new} if absent; if the key is already there,
+// lowers its val to `val_if_new` when that is smaller (val_if_new = 0xFFFFFFFF: leave it).
+// Returns kEmpty if the table is full.
+//
+// One 8-byte load per probe reads key and val together.  Keys only ever change from empty to a
+// key and vals only ever decrease while inserts run, so an ordinary (cacheable, possibly stale)
+// load is enough for the first look: a stale "empty" is settled by the 64-bit CAS, which
+// installs key and val in one atomic, and a stale val can only cause a redundant atomicMin.
+__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new)
 {
+    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
+    const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)val_if_new << 32);
     uint32_t p = (id * kHashMul) >> t.shift;
     const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
     for (uint32_t n = 0; n < limit; ++n) {
-        uint32_t k = t.words[2 * (size_t)p];
-        if (k == kEmpty) {
-            const uint32_t seen = atomicCAS(&t.words[2 * (size_t)p], kEmpty, id);
-            k = (seen == kEmpty) ? id : seen;
+        unsigned long long s = slots[p];
+        if ((uint32_t)s == kEmpty) {
+            const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
+            if (seen == ~0ull) return p;
+            s = seen;
         }
-        if (k == id) return p;
+        if ((uint32_t)s == id) {
+            if ((uint32_t)(s >> 32) > val_if_new) atomicMin(&t.words[2 * (size_t)p + 1], val_if_new);
+            return p;
+        }
         p = (p + 1) & t.mask;
     }
     return kEmpty;
@@ -101,12 +111,8 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, co
     if (i >= n) return;
     const int32_t id = ids[i];
     if (uniq != nullptr && uniq != ids) uniq[i] = id;
-    const uint32_t p = find_or_insert(t, (uint32_t)id);
-    if (p == kEmpty) {
-        if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
-        return;
-    }
-    atomicMin(&t.words[2 * (size_t)p + 1], (uint32_t)i);
+    const uint32_t p = find_or_insert(t, (uint32_t)id, (uint32_t)i);  // a repeated id keeps its first position
+    if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
 }
 
 __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* __restrict__ src,
@@ -118,18 +124,11 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
     const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
-        const uint32_t id = (uint32_t)src[e];
-        const uint32_t p = find_or_insert(t, id);
+        // ids numbered earlier hold val < n_base and stay as they are; a new id keeps the smallest
+        // n_base + (edge index) among the edges that mention it
+        const uint32_t p = find_or_insert(t, (uint32_t)src[e], n_base + (uint32_t)e);
         slot_of[e] = p;
-        if (p == kEmpty) {
-            if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
-            continue;
-        }
-        uint32_t* val = &t.words[2 * (size_t)p + 1];
-        const uint32_t mine = n_base + (uint32_t)e;
-        // ids numbered earlier (val < n_base) are final; otherwise keep the smallest edge index.
-        // val only decreases while this kernel runs, so a stale read can only cause a redundant atomic.
-        if (*val > mine) atomicMin(val, mine);
+        if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
     }
 }
 

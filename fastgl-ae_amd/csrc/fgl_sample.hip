@@ -5,7 +5,8 @@
 //   1. sample_degree_kernel   one lane per seed: two offsets of the row, k = min(fanout, deg),
 //                             staged row start / degree, per-tile sum of k
 //   2. tile prefix            single workgroup; also writes block_ptr[n] and the edge count
-//   3. sample_edges_kernel    per tile of TS seeds: wave64 scan of k -> output offsets,
+//   3. sample_edges_reg_kernel (fanout <= 32) / sample_edges_kernel (larger fanouts)
+//                             per tile of TS seeds: wave64 scan of k -> output offsets,
 //                             Floyd subset selection for rows longer than the fanout (one lane
 //                             per seed, Philox stream keyed by the node id, picks kept in LDS in a
 //                             conflict-free [pick][seed] layout),
@@ -151,6 +152,82 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
     }
 }
 
+// Variant for fanout <= F (F = 8, 16, 32): the picks live in registers (both Floyd loops are
+// fully unrolled, so the membership test costs no LDS traffic), every lane issues all of its
+// row reads at once (one memory round trip per tile), and the values are staged through LDS at
+// their output offsets so that the global writes are one coalesced pass.
+template <int TS, int F>
+__global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __restrict__ indices,
+                                                              const int32_t* __restrict__ seeds, int64_t n_max,
+                                                              const int32_t* __restrict__ d_n, int fanout,
+                                                              const int64_t* __restrict__ row_start,
+                                                              const int32_t* __restrict__ deg_arr,
+                                                              const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
+                                                              uint32_t seed_hi, uint32_t stream_id,
+                                                              int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
+                                                              int32_t* __restrict__ block_ptr)
+{
+    extern __shared__ int32_t s_stage[];  // [TS*fanout] sampled ids (+ [TS*fanout] seed ids when dst_out is wanted)
+    __shared__ int s_scan[TS / kWave + 1];
+    int32_t* s_val = s_stage;
+    int32_t* s_dst = s_stage + TS * fanout;
+
+    const int tid = (int)threadIdx.x;
+    const int64_t n = actual_count(n_max, d_n);
+    const int64_t n_tiles = (n + TS - 1) / TS;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i = tile * TS + tid;
+        int deg = 0, seed = 0;
+        int64_t row = 0;
+        if (i < n) {
+            deg = deg_arr[i];
+            row = row_start[i];
+            seed = seeds[i];
+        }
+        const int k = deg < fanout ? deg : fanout;
+        int total;
+        const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
+        const int base = tile_prefix[tile];
+        if (i < n) block_ptr[i] = base + ex;
+
+        uint32_t sel[F];
+#pragma unroll
+        for (int m = 0; m < F; ++m) sel[m] = (uint32_t)m;  // deg <= fanout: the whole row, in CSR order
+        if (deg > fanout) {
+            // Floyd: for j = deg-k .. deg-1 draw t in [0, j]; take t unless already taken, else j.
+            uint32_t o[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int m = 0; m < F; ++m) {
+                if (m < fanout) {
+                    if ((m & 1) == 0) philox4x32_10((uint32_t)seed, 0u, stream_id, (uint32_t)(m >> 1), seed_lo, seed_hi, o);
+                    const uint64_t r = (m & 1) ? ((uint64_t)o[2] | ((uint64_t)o[3] << 32)) : ((uint64_t)o[0] | ((uint64_t)o[1] << 32));
+                    const uint32_t j = (uint32_t)(deg - fanout + m);
+                    const uint32_t t = (uint32_t)__umul64hi(r, (uint64_t)j + 1u);
+                    bool dup = false;
+#pragma unroll
+                    for (int q = 0; q < m; ++q) dup |= (sel[q] == t);
+                    sel[m] = dup ? j : t;
+                }
+            }
+        }
+        int32_t v[F];
+#pragma unroll
+        for (int m = 0; m < F; ++m) v[m] = (m < k) ? indices[row + (int64_t)sel[m]] : 0;
+#pragma unroll
+        for (int m = 0; m < F; ++m)
+            if (m < k) {
+                s_val[ex + m] = v[m];
+                if (dst_out) s_dst[ex + m] = seed;
+            }
+        __syncthreads();
+        for (int x = tid; x < total; x += TS) {
+            src_out[(int64_t)base + x] = s_val[x];
+            if (dst_out) dst_out[(int64_t)base + x] = s_dst[x];
+        }
+        __syncthreads();  // the staging area is reused by the next tile
+    }
+}
+
 static inline int tile_seeds_for(int fanout) { return fanout <= 48 ? 256 : 64; }
 
 size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
@@ -186,14 +263,25 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds, TS,
                                 stream);
     if (rc != FGL_OK) return rc;
+    if constexpr (TS == 256) if (fanout <= 32) {
+        const size_t lds_reg = (size_t)fanout * TS * sizeof(int32_t) * (d_dst_out ? 2 : 1);
+#define FGL_LAUNCH_REG(F)                                                                                           \
+    hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
+                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr)
+        if (fanout <= 8) FGL_LAUNCH_REG(8);
+        else if (fanout <= 16) FGL_LAUNCH_REG(16);
+        else FGL_LAUNCH_REG(32);
+#undef FGL_LAUNCH_REG
+        FGL_CHECK_LAUNCH("sample_edges_reg_kernel");
+        return FGL_OK;
+    }
     const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
 #define FGL_LAUNCH_EDGES(U)                                                                                        \
     hipLaunchKernelGGL((sample_edges_kernel<TS, U>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,          \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
                        (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr)
-    if (fanout <= 4) FGL_LAUNCH_EDGES(4);
-    else if (fanout <= 8) FGL_LAUNCH_EDGES(8);
-    else FGL_LAUNCH_EDGES(16);
+    FGL_LAUNCH_EDGES(16);
 #undef FGL_LAUNCH_EDGES
     FGL_CHECK_LAUNCH("sample_edges_kernel");
     return FGL_OK;
