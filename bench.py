@@ -31,13 +31,81 @@ WORKLOADS = {
     "c1": dict(nodes=100_000, draws=1_500_000, dim=128, dtype="f32", hidden=256, batch=1024, train=100_000, fanouts=[15, 10, 5]),
     "c2": dict(nodes=2_400_000, draws=36_000_000, dim=100, dtype="f32", hidden=256, batch=8192, train=240_000, fanouts=[15, 10, 5]),
     "c3": dict(nodes=111_000_000, draws=900_000_000, dim=128, dtype="f32", hidden=256, batch=8192, train=1_200_000, fanouts=[15, 10, 5]),
+    "c5": dict(nodes=269_000_000, draws=3_320_000_000, dim=128, dtype="bf16", hidden=256, batch=8192, train=1_200_000, fanouts=[15, 10, 5]),
+    "c5deep": dict(nodes=269_000_000, draws=3_320_000_000, dim=128, dtype="bf16", hidden=256, batch=8192, train=1_200_000,
+                   fanouts=[10, 10, 10, 10, 10]),
+    "c4": None,  # aggregation-only microbench, see run_c4
 }
 DESCRIPTIONS = {
     "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
     "c2": "R-MAT 2.4M nodes / ~62M edges, feat 100 fp32, hidden 256, batch 8192, fanout [15,10,5]",
     "c3": "R-MAT 111M nodes / ~1.6B edges (int64 indptr, int32 indices), feat 111Mx128 fp32 resident, hidden 256, "
           "batch 8192 of 1.2M training seeds, fanout [15,10,5]",
+    "c5": "R-MAT 269M nodes / ~4.0B edges (int64 indptr, int32 indices), feat 269Mx128 bf16 resident, hidden 256, "
+          "batch 8192, fanout [15,10,5]",
+    "c5deep": "R-MAT 269M nodes / ~4.0B edges (int64 indptr, int32 indices), feat 269Mx128 bf16 resident, hidden 256, "
+              "batch 8192, fanout [10,10,10,10,10]",
+    "c4": "aggregation microbench: 8192 dst x exactly 25 src out of 200K rows (int32 CSR), D in {64,128,256,602}, fp32 and bf16, "
+          "sum and mean, forward and backward",
 }
+
+
+def run_c4(args):
+    """Aggregation-only microbench.  Forward = gather over the block, backward = gather over the
+    transposed block; every case is 50 back-to-back launches between two HIP events."""
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    n_dst, n_src, k = 8192, 200_000, 25
+    ptr = (torch.arange(n_dst + 1, dtype=torch.int32) * k).to(dev)
+    idx = torch.randint(0, n_src, (n_dst * k,), generator=g, dtype=torch.int32).to(dev)
+    t_ptr, t_idx = fastgl.block_transpose(ptr, idx, n_dst, n_src)
+    deg = torch.full((n_dst,), k, dtype=torch.int32, device=dev)
+    E = n_dst * k
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def timed(fn, reps=50):
+        for _ in range(5):
+            fn()
+        a, b = ev(), ev()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3  # us
+
+    rows = []
+    for dt, name, esz in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
+        for D in (64, 128, 256, 602):
+            X = torch.randn(n_src, D, generator=g).to(dt).to(dev)
+            dO = torch.randn(n_dst, D, generator=g).to(dt).to(dev)
+            of = torch.empty((n_dst, D), dtype=dt, device=dev)
+            ob = torch.empty((n_src, D), dtype=dt, device=dev)
+            bf = E * D * esz + n_dst * D * esz + 4 * E + 4 * (n_dst + 1)
+            bb = E * D * esz + n_src * D * esz + 4 * E + 4 * (n_src + 1)
+            for mode, bmode in (("sum", "sum"), ("mean", "colmean")):
+                uf = timed(lambda: fastgl.aggregate(ptr, idx, X, mode=mode, zero_policy="zeros", out=of))
+                ub = timed(lambda: fastgl.aggregate(t_ptr, t_idx, dO, mode=bmode, zero_policy="zeros", col_norm=deg, out=ob))
+                rows.append({"dtype": name, "D": D, "mode": mode, "fwd_us": uf, "fwd_GBps": bf / uf / 1e3,
+                             "fwd_frac_peak": bf / uf / 1e3 / HBM_PEAK_GBPS, "bwd_us": ub, "bwd_GBps": bb / ub / 1e3,
+                             "bwd_frac_peak": bb / ub / 1e3 / HBM_PEAK_GBPS})
+                log("%-4s D=%-3d %-4s fwd %6.1f us %5.0f GB/s (%4.1f%%) | bwd %6.1f us %5.0f GB/s (%4.1f%%)"
+                    % (name, D, mode, uf, bf / uf / 1e3, bf / uf / 1e3 / HBM_PEAK_GBPS * 100, ub, bb / ub / 1e3,
+                       bb / ub / 1e3 / HBM_PEAK_GBPS * 100))
+    head = [r for r in rows if r["dtype"] == "f32" and r["D"] == 128 and r["mode"] == "mean"][0]
+    print(json.dumps({
+        "metric": "aggregation HBM GB/s (% peak), 1 MI355X", "value": head["fwd_GBps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": 50, "warmup": 5, "ms_per_step": head["fwd_us"] / 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": DESCRIPTIONS["c4"]},
+        "roofline": {"bound": "hbm", "achieved": head["fwd_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": head["fwd_frac_peak"], "traffic": None, "kernel": "aggregate_kernel (D=128 fp32 mean forward)"},
+        "cpu_baseline": None, "cases": rows}), flush=True)
+
 
 
 def log(*a):
@@ -73,6 +141,8 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "c4":
+        return run_c4(args)
     w = WORKLOADS[args.workload]
     N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
     fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16

@@ -31,14 +31,39 @@ def rmat_csr(n_nodes: int, n_draws: int, seed: int = 0, device="cuda", ptr_dtype
         if k.numel() and int(k[-1]) == _I64_MAX:
             k = k[:-1]
         parts.append(k)
-    if not parts:
-        keys = torch.empty(0, dtype=torch.int64, device=device)
-    elif len(parts) == 1:
-        keys = parts[0]
-    else:
-        keys = torch.unique(torch.cat(parts))
+    keys = _merge_sorted_unique(parts, device)
     del parts
     return csr_from_keys(keys, n_nodes, ptr_dtype)
+
+
+def _merge_sorted_unique(parts, device, max_items=1 << 30):
+    """Union of sorted duplicate-free int64 lists, sorted.  torch's sort/unique take fewer than
+    2^31 items per call, so a large union is assembled from disjoint key ranges (each range is a
+    contiguous slice of every sorted part)."""
+    if not parts:
+        return torch.empty(0, dtype=torch.int64, device=device)
+    if len(parts) == 1:
+        return parts[0]
+    total = sum(int(p.numel()) for p in parts)
+    if total <= max_items:
+        return torch.unique(torch.cat(parts))
+    n_ranges = 2 * ((total + max_items - 1) // max_items)
+    ref = max(parts, key=lambda p: p.numel())
+    cuts = ref[torch.linspace(0, ref.numel() - 1, n_ranges + 1, device=device).long()[1:-1]]  # quantiles of one part
+    cut_pos = [torch.searchsorted(p, cuts).tolist() for p in parts]
+    out = []
+    for r in range(n_ranges):
+        segs = []
+        for p, pos in zip(parts, cut_pos):
+            lo = 0 if r == 0 else pos[r - 1]
+            hi = p.numel() if r == n_ranges - 1 else pos[r]
+            segs.append(p[lo:hi])
+        seg = torch.cat(segs)
+        if seg.numel() >= (1 << 31) - 1:
+            raise RuntimeError("rmat_csr: a key range holds %d items; use smaller chunks" % seg.numel())
+        out.append(torch.unique(seg))
+        del segs, seg
+    return torch.cat(out)
 
 
 def csr_from_keys(keys, n_nodes: int, ptr_dtype=torch.int64, chunk=1 << 26):

@@ -161,3 +161,14 @@ def test_rmat_csr_matches_oracle(cuda, oracle, small_graph):
     indptr, indices = small_graph
     ptr, src = fastgl.graph.rmat_csr(100_000, 1_500_000, seed=0, device=cuda, chunk_draws=400_000)
     assert np.array_equal(ptr.cpu().numpy(), indptr) and np.array_equal(src.cpu().numpy(), indices)
+
+
+def test_merge_of_sorted_parts_by_key_range(cuda):
+    """the large-graph path of the CSR builder (union assembled per key range) equals a plain unique"""
+    import fastgl
+    print("graph merge by range", flush=True)
+    g = torch.Generator(device=cuda).manual_seed(0)
+    parts = [torch.unique(torch.randint(0, 1 << 40, (n,), generator=g, device=cuda)) for n in (50_000, 1, 120_000, 70_000)]
+    want = torch.unique(torch.cat(parts))
+    got = fastgl.graph._merge_sorted_unique(parts, cuda, max_items=40_000)
+    assert torch.equal(got, want)

@@ -71,3 +71,30 @@ def test_mid_shape_properties(cuda):
     atg = fastgl.aggregate(t_ptr, t_idx, g, mode="sum", zero_policy="zeros")
     a, b = (ax.double() * g.double()).sum().item(), (x.double() * atg.double()).sum().item()
     assert abs(a - b) <= 1e-6 * max(abs(a), abs(b), 1.0)
+
+
+def test_offsets_beyond_int32(cuda):
+    """A CSR with more than 2^31 edges (int64 row offsets): rows at the far end are sampled from the
+    right place.  Closed form: indices[e] = e mod 2^20, so a full-neighbourhood row is a known range."""
+    import fastgl
+    print("full-size: >2^31-edge CSR", flush=True)
+    n_nodes, deg = 1 << 22, 520                      # 2.18e9 edges
+    n_edges = n_nodes * deg
+    assert n_edges > (1 << 31)
+    ptr = torch.arange(n_nodes + 1, dtype=torch.int64, device=cuda) * deg
+    idx = torch.empty(n_edges, dtype=torch.int32, device=cuda)
+    step = 1 << 28
+    for lo in range(0, n_edges, step):
+        hi = min(n_edges, lo + step)
+        idx[lo:hi] = (torch.arange(lo, hi, dtype=torch.int64, device=cuda) & ((1 << 20) - 1)).int()
+    seeds = torch.tensor([n_nodes - 1, n_nodes - 2, (1 << 22) - 4096, 5, 0], dtype=torch.int32, device=cuda)
+    # fanout >= degree is impossible here (520 > 192), so check picks against the row's value range instead:
+    # row v holds the consecutive values (v*deg + j) mod 2^20, j < deg; every pick must be one of them, without repeats
+    src, dst, num = fastgl.sample_node(idx, idx, ptr, seeds, seeds.numel(), 192)
+    assert int(num.item()) == 192 * seeds.numel()
+    src = src.view(seeds.numel(), 192).long()
+    assert torch.equal(dst.view(seeds.numel(), 192), seeds[:, None].expand(-1, 192))
+    first = (seeds.long() * deg) & ((1 << 20) - 1)
+    off = (src - first[:, None]) & ((1 << 20) - 1)
+    assert int(off.max()) < deg and int(off.min()) >= 0
+    assert all(off[i].unique().numel() == 192 for i in range(seeds.numel()))
