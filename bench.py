@@ -168,11 +168,20 @@ def main():
 
     sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
     L = len(w["fanouts"])
-    # hidden activations / upstream gradients of the inner layers: synthetic, sized for the worst case
-    plan_caps = fastgl.BlocksPlan(N, B, list(reversed(w["fanouts"])), dev).cap_dst
-    cap_inner = plan_caps[-1]
-    hid = torch.randn((cap_inner, H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
-    grad = torch.randn((cap_inner, H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+    # hidden activations / upstream gradients of the inner layers: synthetic; sized from a probe
+    # batch with head-room (the worst-case bound would be tens of GB for deep fanouts) and grown on demand
+    _, _, probe = sampler.sample_blocks(None, train[:B])
+    inner = {"rows": 0}
+
+    def inner_buffers(rows):
+        if rows > inner["rows"]:
+            inner["rows"] = int(rows * 1.5) + 1
+            inner["hid"] = torch.randn((inner["rows"], H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+            inner["grad"] = torch.randn((inner["rows"], H), generator=gen, device=dev, dtype=torch.float32).to(fdtype)
+        return inner["hid"], inner["grad"]
+
+    inner_buffers(max(b.num_src_nodes() for b in probe[1:]) if L > 1 else 1)
+    del probe
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
 
@@ -186,6 +195,7 @@ def main():
         out0 = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
         e2.record()
         outs = [out0]
+        hid, grad = inner_buffers(max([b.num_src_nodes() for b in blocks[1:]] + [1]))
         for b in blocks[1:]:
             outs.append(fastgl.aggregate(b.edge_ptr, b.src_local, hid[:b.num_src_nodes()], mode="mean", zero_policy="zeros"))
         e3.record()
@@ -195,16 +205,19 @@ def main():
                                          col_norm=b.in_degrees().contiguous()))
         e4.record()
         if rec is not None:
-            rec.append((blocks, (e0, e1, e2, e3, e4)))
+            rec.append(((sum(b.num_edges() for b in blocks), b0.num_edges(), b0.num_dst_nodes()), (e0, e1, e2, e3, e4)))
+            keep.append(b0)
+            del keep[:-4]  # a few outermost blocks are kept for the kernel-time replay below
         return blocks
 
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    rec = []
+    rec, keep = [], []
     t_start = time.perf_counter()
+    last_blocks = None
     for i in range(args.steps):
-        step(args.warmup + i, rec)
+        last_blocks = step(args.warmup + i, rec)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
 
@@ -213,13 +226,15 @@ def main():
     # is empty, so it contains the host's launch latency.  For the roofline the same launches
     # (same kernel, same blocks as the timed steps) are replayed back to back between two HIP
     # events on the stream they run on: the queue stays full and the interval is kernel time.
-    out_buf = torch.empty((max(b[0][0].num_dst_nodes() for b in rec), D), dtype=fdtype, device=dev)
+    out_buf = torch.empty((max(b.num_dst_nodes() for b in keep), D), dtype=fdtype, device=dev)
     ra, rb = ev(), ev()
     torch.cuda.synchronize()
     ra.record()
-    for blocks, _ in rec:
-        b0 = blocks[0]
+    replay_bytes = 0
+    for r in range(args.steps):
+        b0 = keep[r % len(keep)]
         fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros", out=out_buf[:b0.num_dst_nodes()])
+        replay_bytes += b0.num_edges() * D * esz + b0.num_dst_nodes() * D * esz + 4 * b0.num_edges() + 4 * (b0.num_dst_nodes() + 1)
     rb.record()
     torch.cuda.synchronize()
     t_kernel0 = ra.elapsed_time(rb)
@@ -238,20 +253,18 @@ def main():
     tot_edges = 0
     t_sample = t_agg0 = t_fwd_in = t_bwd = 0.0
     bytes_agg0 = 0
-    for blocks, (e0, e1, e2, e3, e4) in rec:
-        tot_edges += sum(b.num_edges() for b in blocks)
+    for (n_e_all, e_, nd), (e0, e1, e2, e3, e4) in rec:
+        tot_edges += n_e_all
         t_sample += e0.elapsed_time(e1)
         t_agg0 += e1.elapsed_time(e2)
         t_fwd_in += e2.elapsed_time(e3)
         t_bwd += e3.elapsed_time(e4)
-        b0 = blocks[0]
-        e_, nd = b0.num_edges(), b0.num_dst_nodes()
         bytes_agg0 += e_ * D * esz + nd * D * esz + 4 * e_ + 4 * (nd + 1)  # gathered rows + output + indices + offsets
     K = args.steps
     edges_per_s = tot_edges / (t_sample * 1e-3)
-    agg_gbps = bytes_agg0 / (t_kernel0 * 1e-3) / 1e9
-    b_last = rec[-1][0]
-    log("last batch blocks:", b_last)
+    agg_gbps = replay_bytes / (t_kernel0 * 1e-3) / 1e9
+    bytes_agg0 = replay_bytes
+    log("last batch blocks:", last_blocks)
     log("per step: sample+idmap %.3f ms, agg fwd outer %.3f ms, agg fwd inner %.3f ms, transpose+bwd %.3f ms, wall %.3f ms"
         % (t_sample / K, t_agg0 / K, t_fwd_in / K, t_bwd / K, wall / K * 1e3))
 

@@ -25,7 +25,10 @@ struct BlocksPlan {
     size_t ws_bytes;
 };
 
-static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops, BlocksPlan* p)
+// node_capacity (optional, n_hops+1 entries): the caller's own limit on the number of nodes before
+// hop h (entry n_hops: after the last hop).  The plan is the worst case clipped to it.
+static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops, const int64_t* node_capacity,
+                     BlocksPlan* p)
 {
     FGL_REQUIRE(n_hops >= 1 && n_hops <= 32, "sample_blocks: %d hops outside [1, 32]", n_hops);
     FGL_REQUIRE(n_nodes >= 0 && n_seeds >= 0 && fanouts != nullptr, "sample_blocks: bad sizes");
@@ -33,6 +36,10 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
     size_t ws = 0;
     for (int h = 0; h < n_hops; ++h) {
         FGL_REQUIRE(fanouts[h] >= 1 && fanouts[h] <= FGL_MAX_FANOUT, "sample_blocks: fanout %d outside [1, %d]", fanouts[h], FGL_MAX_FANOUT);
+        if (node_capacity) {
+            FGL_REQUIRE(node_capacity[h] >= n_seeds, "sample_blocks: node_capacity[%d] = %lld is below the seed count", h, (long long)node_capacity[h]);
+            if (cur > node_capacity[h]) cur = node_capacity[h];
+        }
         p->cap_dst[h] = cur;
         p->cap_edges[h] = cur * fanouts[h];
         FGL_REQUIRE(p->cap_edges[h] <= 0x7FFFFFFF, "sample_blocks: hop %d may produce %lld edges, beyond int32 offsets", h, (long long)p->cap_edges[h]);
@@ -42,6 +49,10 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
         int64_t next = cur + p->cap_edges[h];
         if (next > n_nodes + n_seeds) next = n_nodes + n_seeds;
         cur = next;
+    }
+    if (node_capacity) {
+        FGL_REQUIRE(node_capacity[n_hops] >= p->cap_dst[n_hops - 1], "sample_blocks: node_capacity[%d] is below an earlier entry", n_hops);
+        if (cur > node_capacity[n_hops]) cur = node_capacity[n_hops];
     }
     p->cap_uniq = cur;
     p->table_slots = fgl_idmap_slots(cur);
@@ -85,11 +96,11 @@ __global__ __launch_bounds__(kBlock) void rmat_keys_kernel(int64_t first_edge, i
 using namespace fgl;
 
 FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                                      int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq, int64_t* table_slots,
-                                      size_t* ws_bytes)
+                                      const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges,
+                                      int64_t* cap_uniq, int64_t* table_slots, size_t* ws_bytes)
 {
     BlocksPlan p;
-    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, &p);
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
     if (rc != FGL_OK) return rc;
     for (int h = 0; h < n_hops; ++h) {
         if (cap_dst) cap_dst[h] = p.cap_dst[h];
@@ -103,14 +114,14 @@ FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const in
 
 FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                                  const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                                 uint64_t rng_seed, uint32_t stream_base, int idmap_flags, void* d_table,
+                                 const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base, int idmap_flags, void* d_table,
                                  int64_t table_slots,
                                  int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
                                  int32_t* const* src_local, int32_t* const* src_global, int32_t* d_counts, void* d_ws,
                                  size_t ws_bytes, void* stream)
 {
     BlocksPlan p;
-    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, &p);
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
     if (rc != FGL_OK) return rc;
     FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
     FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
@@ -145,8 +156,11 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         rc = launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], rng_seed,
                            stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s);
         if (rc != FGL_OK) return rc;
+        // the node count this hop may grow to: what the next hop's buffers (or the unique list) hold;
+        // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped
+        const int64_t grow_to = (h + 1 < n_hops && p.cap_dst[h + 1] < p.cap_uniq) ? p.cap_dst[h + 1] : p.cap_uniq;
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
-                                  d_counts + h + 1, d_uniq, uniq_capacity, idmap_flags, d_status, ws + ws_sample,
+                                  d_counts + h + 1, d_uniq, grow_to, idmap_flags, d_status, ws + ws_sample,
                                   ws_bytes - ws_sample, s);
         if (rc != FGL_OK) return rc;
     }

@@ -42,8 +42,8 @@ SIGNATURES = {
     "fgl_idmap_map_src_workspace_bytes": (_sz, [_i64]),
     "fgl_idmap_map_src": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _sz, _vp]),
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
-    "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp]),
-    "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64]),
     "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _sz, _vp]),
     "fgl_aggregate": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),

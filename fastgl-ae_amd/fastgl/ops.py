@@ -318,17 +318,20 @@ def table_size(num: int, scale: int) -> int:
 class BlocksPlan:
     """Bounds and persistent scratch for sampling mini-batches of one shape."""
 
-    def __init__(self, n_nodes: int, n_seeds: int, hop_fanouts, device):
+    def __init__(self, n_nodes: int, n_seeds: int, hop_fanouts, device, node_capacity=None):
+        """``node_capacity`` (optional, ``n_hops + 1`` ints): the caller's own limit on the node count
+        before each hop / after the last; the worst-case bounds are clipped to it."""
         lib = L.lib()
         self.n_nodes, self.n_seeds = int(n_nodes), int(n_seeds)
         self.hop_fanouts = [int(f) for f in hop_fanouts]
         self.n_hops = len(self.hop_fanouts)
         self.device = torch.device(device)
         self._fan = (C.c_int32 * self.n_hops)(*self.hop_fanouts)
+        self._node_cap = None if node_capacity is None else (C.c_int64 * (self.n_hops + 1))(*[int(c) for c in node_capacity])
         cap_dst = (C.c_int64 * self.n_hops)()
         cap_edges = (C.c_int64 * self.n_hops)()
         cap_uniq, slots, ws_bytes = C.c_int64(), C.c_int64(), C.c_size_t()
-        L.check(lib.fgl_sample_blocks_plan(self.n_nodes, self.n_seeds, self._fan, self.n_hops, cap_dst, cap_edges,
+        L.check(lib.fgl_sample_blocks_plan(self.n_nodes, self.n_seeds, self._fan, self.n_hops, self._node_cap, cap_dst, cap_edges,
                                            C.byref(cap_uniq), C.byref(slots), C.byref(ws_bytes)))
         self.cap_dst = list(cap_dst)
         self.cap_edges = list(cap_edges)
@@ -369,7 +372,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         counts = torch.empty(2 * H + 2, dtype=torch.int32, device=dev)
         arr = lambda ts: (C.c_void_p * H)(*[L.ptr(t) for t in ts])
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
-                                      int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H,
+                                      int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF,
                                       {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order], L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),

@@ -107,8 +107,9 @@ class FusedMapSampler:
         self.edge_dst = None  # unused by the kernels; kept because the reference's trainer sets it
         self.edge_ptr = None  # CSR indptr (int32 or int64)
         self.output_nodes = None
-        self._plans = {}
-        self._uniq_seen = 0  # largest number of unique nodes any mini-batch has produced
+        self._shape = None
+        self._plans = {}        # node-capacity tuple (None = worst case) -> BlocksPlan
+        self._nodes_seen = None  # per hop: the largest node count any mini-batch has reached
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
         self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
@@ -133,31 +134,43 @@ class FusedMapSampler:
     def _sample_fused(self, seeds, stream_base):
         hop_fanouts = list(reversed(self.fanouts))
         H = len(hop_fanouts)
-        key = (int(seeds.numel()), tuple(hop_fanouts), self.nodes_num, seeds.device)
-        plan = self._plans.get(key)
-        if plan is None:
-            plan = ops.BlocksPlan(self.nodes_num, int(seeds.numel()), hop_fanouts, seeds.device)
-            self._plans = {key: plan}
-        # The plan's table can never overflow but is sized for batches without any repeated
-        # neighbour.  Real batches are far smaller, and a table that fits the caches is much
-        # faster, so after the first batch the table is sized from the largest batch seen (load
-        # <= 1/4); a batch that still outgrows it is detected by the kernels and simply redone
-        # with the full table.  Results do not depend on the table size.
-        slots_for = ops.L.lib().fgl_idmap_slots
-        slots = plan.slots if self._uniq_seen == 0 else min(plan.slots, max(slots_for(2 * self._uniq_seen), slots_for(plan.n_seeds)))
+        lib = ops.L.lib()
+        n_seeds = int(seeds.numel())
+        shape = (n_seeds, tuple(hop_fanouts), self.nodes_num, seeds.device)
+        if self._shape != shape:
+            self._shape, self._plans, self._nodes_seen = shape, {}, None
+        # Worst-case bounds assume that no neighbour ever repeats: 8.6 M nodes for 8192 seeds and
+        # fanouts 5/10/15 where real batches hold ~1 M, and the whole graph for deep fanouts.  A hash
+        # table that fits the caches is much faster and output buffers sized by the bound cost GBs,
+        # so after the first batch both are sized from the largest batch seen (x1.5, table load <=
+        # 1/4).  A batch that outgrows them is detected by the kernels (status word) and simply
+        # redone with the worst-case plan; results do not depend on the sizes.
+        caps = None
+        if self._nodes_seen is not None:
+            caps = tuple(max(n_seeds, -(-int(1.5 * n) // 4096) * 4096) for n in self._nodes_seen)
         while True:
+            plan = self._plans.get(caps)
+            if plan is None:
+                plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
+                self._plans = {k: v for k, v in self._plans.items() if k is None}  # keep the worst-case plan only
+                self._plans[caps] = plan
+            slots = plan.slots
+            if caps is not None:
+                slots = min(slots, max(lib.fgl_idmap_slots(2 * self._nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
             uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
                                                                        self.rng_seed, stream_base, keep_global=(H - 1,),
                                                                        table_slots=slots, id_order=self.id_order)
             c = counts.tolist()  # the one host synchronisation of the mini-batch
             status = c[2 * H + 1]
-            if status & ops.L.STATUS_TABLE_FULL and slots < plan.slots:
-                slots = plan.slots
+            if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and caps is not None:
+                caps = None
+                self._nodes_seen = None
                 continue
             break
         if status:
             ops._raise_status(status, "sample_blocks")
-        self._uniq_seen = max(self._uniq_seen, c[H])
+        seen = c[:H + 1]
+        self._nodes_seen = seen if self._nodes_seen is None else [max(a, b) for a, b in zip(seen, self._nodes_seen)]
         blocks = []
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]

@@ -153,6 +153,13 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * (The reference lists fanouts the other way round and iterates reversed(); the caller
  * passes them already reversed.)
  *
+ * node_capacity (optional, n_hops+1 host entries, NULL = none): the caller's own limit on the
+ * number of nodes before hop h (last entry: after the last hop).  Worst-case bounds assume
+ * that no neighbour ever repeats; for deep fanouts they reach the size of the graph, so a
+ * caller that knows its batches may size its buffers by experience instead.  A batch that
+ * grows past a limit sets FGL_STATUS_UNIQ_OVERFLOW (its outputs are then invalid, nothing is
+ * written out of bounds) and is repeated with larger limits.
+ *
  * fgl_sample_blocks_plan fills, for the given bounds, cap_dst[h] (max seeds of hop h),
  * cap_edges[h] (max edges of hop h), *cap_uniq (max unique ids overall), *table_slots
  * (the slot count that can never overflow) and *ws_bytes.  fgl_sample_blocks also accepts a
@@ -166,11 +173,11 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word.
  * ------------------------------------------------------------------------------- */
 int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                           int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,
+                           const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,
                            int64_t* table_slots, size_t* ws_bytes);
 int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                       const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                      uint64_t rng_seed, uint32_t stream_base, int idmap_flags,
+                      const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base, int idmap_flags,
                       void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
                       int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
                       int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);

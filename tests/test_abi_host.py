@@ -43,19 +43,25 @@ def test_plan_matches_the_worst_case_table():
     fan = (C.c_int32 * 3)(5, 10, 15)
     cd, ce = (C.c_int64 * 3)(), (C.c_int64 * 3)()
     cu, sl, ws = C.c_int64(), C.c_int64(), C.c_size_t()
-    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 8192, fan, 3, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 8192, fan, 3, None, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
     assert list(cd) == [8192, 49152, 540672]
     assert list(ce) == [40960, 491520, 8110080]
     assert cu.value == 8650752 and sl.value == 1 << 25 and ws.value > 0
     # a small graph caps the bounds
-    L.check(fastgl.lib().fgl_sample_blocks_plan(1000, 100, fan, 3, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    L.check(fastgl.lib().fgl_sample_blocks_plan(1000, 100, fan, 3, None, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
     assert list(cd) == [100, 600, 1100] and cu.value == 1100
+    # the caller's own limits clip the plan
+    lim = (C.c_int64 * 4)(100, 300, 400, 500)
+    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, lim, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    assert list(cd) == [100, 300, 400] and list(ce) == [500, 3000, 6000] and cu.value == 500
+    bad = (C.c_int64 * 4)(50, 300, 400, 500)
+    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, bad, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
 
 
 def test_argument_errors_are_reported_not_launched():
     lib = fastgl.lib()
     fan = (C.c_int32 * 1)(0)
-    assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, None, None, None, None) == 1
+    assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, None, None, None, None, None) == 1
     assert b"fanout" in lib.fgl_last_error()
     assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
     assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table

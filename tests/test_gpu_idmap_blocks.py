@@ -133,23 +133,34 @@ def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     check_blocks(oracle, indptr, indices, seeds, [4, 4], got, 1, 0)
 
 
-def test_undersized_table_is_detected_and_redone(cuda, oracle, small_graph):
-    """The sampler sizes its hash table from earlier batches; a batch that outgrows it must be
-    caught by the kernels (status word) and repeated with the worst-case table, with the same result."""
+def test_undersized_buffers_are_detected_and_redone(cuda, oracle, small_graph):
+    """The sampler sizes its hash table and output buffers from earlier batches; a batch that outgrows
+    them must be caught by the kernels (status word) and repeated with the worst-case plan, same result."""
     import fastgl
-    print("sample_blocks undersized table", flush=True)
+    print("sample_blocks undersized buffers", flush=True)
     indptr, indices = small_graph
     ptr, idx = load_graph(cuda, indptr, indices)
     sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=9).set_graph(ptr, idx)
-    sampler._uniq_seen = 1  # pretend earlier batches were tiny: the table only fits the seeds
-    seeds = np.random.default_rng(3).permutation(indptr.size - 1)[:512].astype(np.int32)
-    got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
-    check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], got, 9, 0)
-    assert sampler._uniq_seen == got[0].numel() > 2 * 512
-    # the raw entry point reports the overflow instead of faulting or spinning
+    low = np.flatnonzero(np.diff(indptr) <= 1)[:512].astype(np.int32)       # a batch that hardly grows ...
+    got = sampler.sample_blocks(None, dev_i32(low, cuda))
+    check_blocks(oracle, indptr, indices, low, [15, 10, 5], got, 9, 0)
+    sampler._nodes_seen = [512, 600, 700, 800]                              # (pretend it stayed tiny)
+    hubs = np.argsort(-np.diff(indptr))[:512].astype(np.int32)              # ... followed by one that explodes
+    got = sampler.sample_blocks(None, dev_i32(hubs, cuda))
+    check_blocks(oracle, indptr, indices, hubs, [15, 10, 5], got, 9, 64)
+    assert sampler._nodes_seen[-1] == got[0].numel() > 4096                 # outgrew the 4096-node buffers, was redone
+    got = sampler.sample_blocks(None, dev_i32(low, cuda))                   # and sized-by-experience again
+    check_blocks(oracle, indptr, indices, low, [15, 10, 5], got, 9, 128)
+    # the raw entry point reports both kinds of overflow instead of faulting or spinning
+    seeds = dev_i32(hubs, cuda)
     plan = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda)
-    out = fastgl.sample_blocks_fused(plan, ptr, idx, dev_i32(seeds, cuda), 9, 0, table_slots=1024)
+    out = fastgl.sample_blocks_fused(plan, ptr, idx, seeds, 9, 0, table_slots=1024)
     assert out[4].tolist()[-1] & 1  # FGL_STATUS_TABLE_FULL
+    tight = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda, node_capacity=[512, 600, 700, 800])
+    assert tight.cap_dst == [512, 600, 700] and tight.cap_uniq == 800
+    out = fastgl.sample_blocks_fused(tight, ptr, idx, seeds, 9, 0)
+    c = out[4].tolist()
+    assert c[-1] & 2 and c[1] <= 600 and c[2] <= 700 and c[3] <= 800  # FGL_STATUS_UNIQ_OVERFLOW, counts clamped
 
 
 @pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64)])
