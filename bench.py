@@ -25,6 +25,10 @@ for _p in (ROOT, os.path.join(ROOT, "fastgl-ae_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM traffic per launch of the dominant kernel on workload c3, from two `rocprofv3 --pmc` runs
+# (FETCH_SIZE 369898 KiB x 1.898 + WRITE_SIZE 55671 KiB x 1.000, the factors being what the same
+# counters read for this kernel run as a plain copy of known size; profiles/aggregate_kernel_c3_pmc.md)
+TRAFFIC_BYTES_C3 = 369898 * 1024 * 1.898 + 55671 * 1024 * 1.0
 
 WORKLOADS = {
     # name: nodes, R-MAT draws, feature dim, feature dtype, hidden, batch, training seeds, fanouts (reference order)
@@ -247,7 +251,15 @@ def main():
         torch.cuda.synchronize()
         c = a.view(torch.float32) * 1.0  # an ordinary elementwise kernel: reads and writes the same amount
         torch.cuda.synchronize()
-        del a, b, c
+        # the aggregation kernel itself as a plain copy: every row has exactly one neighbour, itself
+        # (sum mode, D=128 fp32): reads and writes pmc_copy_mib MiB of rows with the same instructions
+        rows = (args.pmc_copy_mib << 20) // (128 * 4)
+        x = a.view(torch.float32)[:rows * 128].view(rows, 128)
+        ident_ptr = torch.arange(rows + 1, dtype=torch.int32, device=dev)
+        ident_idx = torch.arange(rows, dtype=torch.int32, device=dev)
+        y = fastgl.aggregate(ident_ptr, ident_idx, x, mode="sum", zero_policy="zeros")
+        torch.cuda.synchronize()
+        del a, b, c, x, y
 
     # ---- reduce -------------------------------------------------------------------------
     tot_edges = 0
@@ -318,8 +330,9 @@ def main():
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS},
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": agg_gbps / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "aggregate_kernel (outermost block, mean, forward)",
+                     "frac": agg_gbps / HBM_PEAK_GBPS,
+                     "traffic": TRAFFIC_BYTES_C3 if args.workload == "c3" and args.id_order == "first" else None,
+                     "kernel": "aggregate_kernel<float,4,32,MEAN> (outermost block, forward)",
                      "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_kernel0 / K * 1e3},
         "cpu_baseline": cpu,
     }
