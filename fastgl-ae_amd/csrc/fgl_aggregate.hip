@@ -112,6 +112,28 @@ struct RowIO<uint16_t, 1> {
     static __device__ __forceinline__ void store_partial(uint16_t* p, const float (&acc)[1], int) { store(p, acc); }
 };
 
+// Everything one launch needs.  T-typed pointers are kept as void* so that one struct serves
+// both element types.
+struct AggArgs {
+    const int32_t* indptr;
+    const int32_t* indices;
+    int64_t n_rows_max;
+    const int32_t* d_n_rows;
+    const void* x;
+    int64_t ldx;
+    int D;
+    int zero_policy;
+    const int32_t* row_norm;
+    const int32_t* col_norm;
+    void* out;
+    int64_t ldo;
+    // FGL_AGG_EDGE only: per-entry, per-head weights w[entry_id * n_heads + head(column)]
+    const float* edge_w;
+    const int32_t* edge_index;  // entry -> entry_id (NULL: the entry's own position)
+    int n_heads;
+    int unit_dim;               // D / n_heads
+};
+
 // per-edge weight, evaluated by the lane that loaded the neighbour id
 template <int MODE>
 __device__ __forceinline__ float edge_weight(int col, float row_factor, const int32_t* __restrict__ col_norm)
@@ -125,17 +147,18 @@ __device__ __forceinline__ float edge_weight(int col, float row_factor, const in
 }
 
 template <typename T, int VEC, int LPR, int MODE>
-__global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __restrict__ indptr,
-                                                           const int32_t* __restrict__ indices, int64_t n_rows_max,
-                                                           const int32_t* __restrict__ d_n_rows,
-                                                           const T* __restrict__ X, int64_t ldx, int D, int zero_policy,
-                                                           const int32_t* __restrict__ row_norm,
-                                                           const int32_t* __restrict__ col_norm, T* __restrict__ out,
-                                                           int64_t ldo)
+__global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
 {
     using IO = RowIO<T, VEC>;
     constexpr int kGroups = kBlock / LPR;
-    const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx, ldo = g.ldo;
+    const int D = g.D;
+
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
     const int gl = (int)threadIdx.x % LPR;  // lane within the group
     const int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
     if (row >= n_rows) return;  // uniform per group: the cross-lane reads below stay inside the group
@@ -156,15 +179,61 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
 
     if (a == b) {
         if (live) {
-            if (zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, load_row(X + row * ldx + col0));
+            if (g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, load_row(X + row * ldx + col0));
             store_row(out + row * ldo + col0, acc);
         }
         return;
     }
 
+    if constexpr (MODE == FGL_AGG_EDGE) {
+        // attention-style weights: one float per (entry, head); a lane's VEC columns lie in one
+        // head when unit_dim is a multiple of VEC, else each column looks its head up
+        const float* __restrict__ ew = g.edge_w;
+        const int H = g.n_heads, unit = g.unit_dim;
+        const bool one_head = (unit % VEC) == 0;
+        int head[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int c = col0 + i < D ? col0 + i : D - 1;
+            head[i] = c / unit;
+        }
+        for (int base = a; base < b; base += LPR) {
+            const int cnt = (b - base) < LPR ? (b - base) : LPR;
+            int my_col = 0, my_eid = 0;
+            if (gl < cnt) {
+                my_col = indices[base + gl];
+                my_eid = g.edge_index ? g.edge_index[base + gl] : base + gl;
+            }
+            float part[VEC];  // this chunk's sum (see the note on two-level summation below)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
+            for (int t = 0; t < cnt; ++t) {
+                const int c0 = __shfl(my_col, t, LPR);
+                const int64_t e0 = __shfl(my_eid, t, LPR);
+                if (live) {
+                    const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
+                    if (one_head) {
+                        IO::fma(part, ew[e0 * H + head[0]], r0);
+                    } else {
+                        float x[VEC];
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) x[i] = 0.0f;
+                        IO::fma(x, 1.0f, r0);
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) part[i] += ew[e0 * H + head[i]] * x[i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += part[i];
+        }
+        if (live) store_row(out + row * ldo + col0, acc);
+        return;
+    }
+
     float row_factor = 1.0f;
     if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
-    if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)row_norm[row]);
+    if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
 
     for (int base = a; base < b; base += LPR) {
         const int cnt = (b - base) < LPR ? (b - base) : LPR;
@@ -172,11 +241,18 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
         float my_w = 0.0f;
         if (gl < cnt) {
             my_col = indices[base + gl];
-            my_w = edge_weight<MODE>(my_col, row_factor, col_norm);
+            my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
         }
         // four row loads are issued before the first FMA; the tail of the list goes one by one
         // (measured: longer or predicated unrolls gain nothing on long lists and lose up to 2x
-        // on the one- and two-entry lists of a transposed block)
+        // on the one- and two-entry lists of a transposed block).
+        // Two-level summation: each chunk of LPR entries is summed on its own and then added to
+        // the row total, so the rounding error of a row with thousands of entries (a hub in a
+        // transposed block) grows like LPR + n/LPR instead of n.  Rows of at most LPR entries --
+        // every sampled block -- are summed in plain CSR order.
+        float part[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
         int t = 0;
         for (; t + 4 <= cnt; t += 4) {
             const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
@@ -188,17 +264,19 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const int32_t* __rest
                 const typename IO::Raw r1 = load_row(X + (int64_t)c1 * ldx + col0);
                 const typename IO::Raw r2 = load_row(X + (int64_t)c2 * ldx + col0);
                 const typename IO::Raw r3 = load_row(X + (int64_t)c3 * ldx + col0);
-                IO::fma(acc, w0, r0);
-                IO::fma(acc, w1, r1);
-                IO::fma(acc, w2, r2);
-                IO::fma(acc, w3, r3);
+                IO::fma(part, w0, r0);
+                IO::fma(part, w1, r1);
+                IO::fma(part, w2, r2);
+                IO::fma(part, w3, r3);
             }
         }
         for (; t < cnt; ++t) {
             const int c0 = __shfl(my_col, t, LPR);
             const float w0 = __shfl(my_w, t, LPR);
-            if (live) IO::fma(acc, w0, load_row(X + (int64_t)c0 * ldx + col0));
+            if (live) IO::fma(part, w0, load_row(X + (int64_t)c0 * ldx + col0));
         }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += part[i];
     }
     if (live) store_row(out + row * ldo + col0, acc);
 }
@@ -225,7 +303,8 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
                                                                 const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
                                                                 const int32_t* __restrict__ t_indptr,
                                                                 const int32_t* __restrict__ rank,
-                                                                int32_t* __restrict__ t_indices)
+                                                                int32_t* __restrict__ t_indices,
+                                                                int32_t* __restrict__ t_edge)
 {
     const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
     const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -234,7 +313,11 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
     if (b > n_edges_max) b = n_edges_max;
     for (int64_t e = a; e < b; ++e) {
         const int32_t k = rank[e];
-        if (k >= 0) t_indices[(int64_t)t_indptr[indices[e]] + k] = (int32_t)r;
+        if (k >= 0) {
+            const int64_t pos = (int64_t)t_indptr[indices[e]] + k;
+            t_indices[pos] = (int32_t)r;
+            if (t_edge) t_edge[pos] = (int32_t)e;
+        }
     }
 }
 
@@ -248,18 +331,15 @@ size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
 
 // ---- dispatch ----------------------------------------------------------------------
 template <typename T, int VEC, int LPR>
-static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const int32_t* indptr, const int32_t* indices,
-                           int64_t n_rows_max, const int32_t* d_n_rows, const T* X, int64_t ldx, int D, int zero_policy,
-                           const int32_t* row_norm, const int32_t* col_norm, T* out, int64_t ldo)
+static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const AggArgs& g)
 {
-#define FGL_LAUNCH_MODE(M)                                                                                            \
-    hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, indptr, indices, n_rows_max, \
-                       d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo)
+#define FGL_LAUNCH_MODE(M) hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, g)
     switch (mode) {
         case FGL_AGG_SUM: FGL_LAUNCH_MODE(FGL_AGG_SUM); break;
         case FGL_AGG_MEAN: FGL_LAUNCH_MODE(FGL_AGG_MEAN); break;
         case FGL_AGG_GCN: FGL_LAUNCH_MODE(FGL_AGG_GCN); break;
-        default: FGL_LAUNCH_MODE(FGL_AGG_COLMEAN); break;
+        case FGL_AGG_COLMEAN: FGL_LAUNCH_MODE(FGL_AGG_COLMEAN); break;
+        default: FGL_LAUNCH_MODE(FGL_AGG_EDGE); break;
     }
 #undef FGL_LAUNCH_MODE
     FGL_CHECK_LAUNCH("aggregate_kernel");
@@ -267,15 +347,13 @@ static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const int32_
 }
 
 template <typename T, int VEC>
-static int launch_agg_vec(int mode, hipStream_t stream, const int32_t* indptr, const int32_t* indices, int64_t n_rows_max,
-                          const int32_t* d_n_rows, const T* X, int64_t ldx, int D, int zero_policy,
-                          const int32_t* row_norm, const int32_t* col_norm, T* out, int64_t ldo)
+static int launch_agg_vec(int mode, hipStream_t stream, const AggArgs& g)
 {
-    const int lanes_needed = (D + VEC - 1) / VEC;
+    const int lanes_needed = (g.D + VEC - 1) / VEC;
     int lpr = 8;
     while (lpr < 64 && lpr < lanes_needed) lpr <<= 1;
     const int64_t groups = kBlock / lpr;
-    const int64_t gx = ceil_div(n_rows_max, groups);
+    const int64_t gx = ceil_div(g.n_rows_max, groups);
     const int64_t gy = ceil_div(lanes_needed, lpr);
     if (gx > 0x7FFFFFFF || gy > 65535) {
         set_error("aggregate: grid too large (%lld x %lld)", (long long)gx, (long long)gy);
@@ -283,10 +361,10 @@ static int launch_agg_vec(int mode, hipStream_t stream, const int32_t* indptr, c
     }
     const dim3 grid((unsigned)gx, (unsigned)gy);
     switch (lpr) {
-        case 8: return launch_agg_mode<T, VEC, 8>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
-        case 16: return launch_agg_mode<T, VEC, 16>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
-        case 32: return launch_agg_mode<T, VEC, 32>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
-        default: return launch_agg_mode<T, VEC, 64>(mode, grid, stream, indptr, indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, row_norm, col_norm, out, ldo);
+        case 8: return launch_agg_mode<T, VEC, 8>(mode, grid, stream, g);
+        case 16: return launch_agg_mode<T, VEC, 16>(mode, grid, stream, g);
+        case 32: return launch_agg_mode<T, VEC, 32>(mode, grid, stream, g);
+        default: return launch_agg_mode<T, VEC, 64>(mode, grid, stream, g);
     }
 }
 
@@ -302,29 +380,32 @@ using namespace fgl;
 
 FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
                              const int32_t* d_n_rows, const void* d_x, int64_t ldx, int D, int dtype, int mode,
-                             int zero_policy, const int32_t* d_row_norm, const int32_t* d_col_norm, void* d_out,
+                             int zero_policy, const int32_t* d_row_norm, const int32_t* d_col_norm,
+                             const float* d_edge_w, int n_heads, const int32_t* d_edge_index, void* d_out,
                              int64_t ldo, void* stream)
 {
     FGL_REQUIRE(n_rows_max >= 0, "aggregate: negative row count");
     FGL_REQUIRE(D >= 1, "aggregate: feature length %d < 1", D);
     FGL_REQUIRE(ldx >= D && ldo >= D, "aggregate: row stride smaller than the row length");
     FGL_REQUIRE(dtype == FGL_F32 || dtype == FGL_BF16, "aggregate: unknown dtype %d", dtype);
-    FGL_REQUIRE(mode >= FGL_AGG_SUM && mode <= FGL_AGG_COLMEAN, "aggregate: unknown mode %d", mode);
+    FGL_REQUIRE(mode >= FGL_AGG_SUM && mode <= FGL_AGG_EDGE, "aggregate: unknown mode %d", mode);
     FGL_REQUIRE(zero_policy == FGL_ZERO_COPY_SELF || zero_policy == FGL_ZERO_ZEROS, "aggregate: unknown zero policy %d", zero_policy);
     FGL_REQUIRE(mode != FGL_AGG_GCN || (d_row_norm && d_col_norm), "aggregate: gcn mode needs row_norm and col_norm");
     FGL_REQUIRE(mode != FGL_AGG_COLMEAN || d_col_norm, "aggregate: colmean mode needs col_norm");
+    FGL_REQUIRE(mode != FGL_AGG_EDGE || (d_edge_w && n_heads >= 1 && D % n_heads == 0),
+                "aggregate: edge mode needs edge weights and a head count that divides the row length");
     if (n_rows_max == 0) return FGL_OK;
     FGL_REQUIRE(d_indptr && d_indices && d_x && d_out, "aggregate: null pointer");
     FGL_REQUIRE(d_x != d_out, "aggregate: output aliases the input");
+    AggArgs g;
+    g.indptr = d_indptr; g.indices = d_indices; g.n_rows_max = n_rows_max; g.d_n_rows = d_n_rows;
+    g.x = d_x; g.ldx = ldx; g.D = D; g.zero_policy = zero_policy; g.row_norm = d_row_norm; g.col_norm = d_col_norm;
+    g.out = d_out; g.ldo = ldo; g.edge_w = d_edge_w; g.edge_index = d_edge_index;
+    g.n_heads = n_heads > 0 ? n_heads : 1; g.unit_dim = D / g.n_heads;
     hipStream_t s = as_stream(stream);
-    if (dtype == FGL_F32)
-        return launch_agg_vec<float, 4>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, static_cast<const float*>(d_x), ldx, D,
-                                        zero_policy, d_row_norm, d_col_norm, static_cast<float*>(d_out), ldo);
-    const uint16_t* X = static_cast<const uint16_t*>(d_x);
-    uint16_t* O = static_cast<uint16_t*>(d_out);
-    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out))
-        return launch_agg_vec<uint16_t, 8>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
-    return launch_agg_vec<uint16_t, 1>(mode, s, d_indptr, d_indices, n_rows_max, d_n_rows, X, ldx, D, zero_policy, d_row_norm, d_col_norm, O, ldo);
+    if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, s, g);
+    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, s, g);
+    return launch_agg_vec<uint16_t, 1>(mode, s, g);
 }
 
 FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
@@ -335,8 +416,8 @@ FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_
 
 FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
                                    const int32_t* d_n_rows, int64_t n_cols_max, const int32_t* d_n_cols,
-                                   int64_t n_edges_max, int32_t* d_t_indptr, int32_t* d_t_indices, void* d_ws,
-                                   size_t ws_bytes, void* stream)
+                                   int64_t n_edges_max, int32_t* d_t_indptr, int32_t* d_t_indices,
+                                   int32_t* d_t_edge, void* d_ws, size_t ws_bytes, void* stream)
 {
     FGL_REQUIRE(n_rows_max >= 0 && n_cols_max >= 0 && n_edges_max >= 0, "block_transpose: negative size");
     FGL_REQUIRE(n_edges_max <= 0x7FFFFFFF, "block_transpose: edge count exceeds int32 offsets");
@@ -362,7 +443,7 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
     if (rc != FGL_OK) return rc;
     if (n_edges_max > 0 && n_rows_max > 0) {
         hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)ceil_div(n_rows_max, kBlock)), dim3(kBlock), 0, s, d_indptr,
-                           d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices);
+                           d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices, d_t_edge);
         FGL_CHECK_LAUNCH("transpose_fill_kernel");
     }
     return FGL_OK;

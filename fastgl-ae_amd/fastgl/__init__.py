@@ -3,7 +3,8 @@ name of the reference's extension module so that ``import fastgl`` in the refere
 sampler and layer code resolves to it.
 
 Operators with the reference's signatures: ``sample_node``, ``transfer_edge_id``, ``cal_deg``,
-``exclusive_sum``, ``forward_gcn``, ``backward_gcn``, ``forwaed_gin`` (sic), ``backward_gin``.
+``exclusive_sum``, ``forward_gcn``, ``backward_gcn``, ``forwaed_gin`` (sic), ``backward_gin``,
+``forward_gat``, ``backward_gat``.
 Everything runs in hand-written HIP kernels behind ``libfastgl_hip.so``; there is no CPU path.
 """
 from ._lib import LIB_PATH, build, lib  # noqa: F401
@@ -28,14 +29,18 @@ from .ops import (  # noqa: F401
 )
 from .sampler import Block, FusedMapSampler  # noqa: F401
 from .conv import (  # noqa: F401
+    GAT,
     GCN,
     GIN,
     SAGE,
+    GATConv,
     GCNConv,
     GINConv,
     MA_Function,
+    MA_Function_GAT,
     MA_Function_GIN,
     MA_Function_Mean,
     SAGEConv,
+    edge_softmax,
 )
 from . import graph  # noqa: F401

@@ -1,7 +1,8 @@
 """GNN layers over the memory-aware aggregation operators, with the class names, call
 signatures and autograd wiring of the reference's GraphConv.py (MA_Function, GCNConv, GCN,
-MA_Function_GIN, GINConv, GIN; GraphConv.py:19-195), plus a mean aggregator (GraphSAGE),
-which the reference's benchmark configurations name but its kernels do not provide.
+MA_Function_GIN, GINConv, GIN, MA_Function_GAT, GATConv, GAT; GraphConv.py:19-312), plus a mean
+aggregator (GraphSAGE), which the reference's benchmark configurations name but its kernels do
+not provide.
 
 The reference's quirks are kept where they define results: weights are drawn from
 U(-1/sqrt(out), 1/sqrt(out)) (GraphConv.py:52-55), dropout sits between layers, no activation
@@ -161,6 +162,101 @@ class GIN(nn.Module):
             edge_ptr, src_edges, _ = _block_csr(graph)
             transposed = graph.transposed() if isinstance(graph, Block) and torch.is_grad_enabled() else None
             h = layer(edge_ptr, src_edges, dst_nodes, h, neighbor_list[i], transposed)
+        return h
+
+
+# ---------------------------------------------------------------------------------------
+# attention-weighted aggregation (GAT; GraphConv.py:198-312)
+# ---------------------------------------------------------------------------------------
+class MA_Function_GAT(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, edge_ptr, edge_data, src_edges, dst_edges, dst_nodes, input_feat, num_heads, neighbor_num,
+                transposed=None):
+        X_prime = ops.forward_gat(edge_ptr, edge_data, src_edges, input_feat, neighbor_num, dst_nodes, num_heads)[0]
+        ctx.src_nodes = input_feat.size(0)
+        ctx.num_heads = num_heads
+        ctx.neighbor_num = neighbor_num
+        ctx.transposed = transposed
+        ctx.save_for_backward(edge_ptr, edge_data, src_edges, dst_edges, input_feat)
+        return X_prime
+
+    @staticmethod
+    def backward(ctx, d_input):
+        edge_ptr, edge_data, src_edges, dst_edges, input_feat = ctx.saved_tensors
+        d_input = d_input.contiguous()
+        if ctx.transposed is None:
+            d_x = ops.backward_gat(edge_ptr, edge_data, src_edges, d_input, ctx.src_nodes, ctx.num_heads)[0]
+        else:
+            t_ptr, t_idx, t_edge = ctx.transposed
+            d_x = ops.aggregate(t_ptr, t_idx, d_input, mode="edge", zero_policy="zeros", n_rows=int(ctx.src_nodes),
+                                edge_weight=edge_data, n_heads=int(ctx.num_heads), edge_index=t_edge)
+        # as in the reference (GraphConv.py:227) the attention weights receive no gradient from here
+        return None, None, None, None, None, d_x, None, None, None
+
+
+def edge_softmax(edge_ptr, dst_edges, e, n_dst):
+    """softmax of the edge scores ``e`` [E, H] over the edges of each destination (what the reference
+    takes from dgl.nn.functional.edge_softmax, GraphConv.py:272)"""
+    idx = dst_edges.long()
+    top = torch.full((n_dst, e.size(1)), float("-inf"), dtype=e.dtype, device=e.device)
+    top = top.scatter_reduce(0, idx[:, None].expand(-1, e.size(1)), e, reduce="amax", include_self=True)
+    ex = torch.exp(e - top.index_select(0, idx))
+    den = torch.zeros_like(top).index_add_(0, idx, ex)
+    return ex / den.index_select(0, idx)
+
+
+class GATConv(nn.Module):
+    def __init__(self, input_dim, output_dim, num_heads, feat_drop=0, attn_drop=0, negative_slope=0.2):
+        super().__init__()
+        self.out_feats = output_dim
+        self.num_heads = num_heads
+        self.fc = nn.Linear(input_dim, output_dim * num_heads, bias=False)
+        self.attn_l = nn.Parameter(torch.empty(1, num_heads, output_dim))
+        self.attn_r = nn.Parameter(torch.empty(1, num_heads, output_dim))
+        self.feat_drop = nn.Dropout(feat_drop)
+        self.attn_drop = nn.Dropout(attn_drop)
+        self.leaky_relu = nn.LeakyReLU(negative_slope)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        gain = nn.init.calculate_gain('relu')
+        nn.init.xavier_normal_(self.fc.weight, gain=gain)
+        nn.init.xavier_normal_(self.attn_l, gain=gain)
+        nn.init.xavier_normal_(self.attn_r, gain=gain)
+
+    def forward(self, graph, input_feat, neighbor_num):
+        dst_nodes = graph.num_dst_nodes()
+        feat_src = self.fc(input_feat).view(-1, self.num_heads, self.out_feats)
+        feat_dst = feat_src[:dst_nodes]
+        el = (feat_src * self.attn_l).sum(dim=-1)  # [n_src, H]
+        er = (feat_dst * self.attn_r).sum(dim=-1)  # [n_dst, H]
+        edge_ptr, src_edges, _ = _block_csr(graph)
+        dst_edges = graph.edges()[1].int()
+        # u_add_v + leaky_relu + edge_softmax (DGL calls in the reference, GraphConv.py:265-272)
+        e = self.leaky_relu(el.index_select(0, src_edges.long()) + er.index_select(0, dst_edges.long()))
+        edge_data = self.attn_drop(edge_softmax(edge_ptr, dst_edges, e, dst_nodes)).contiguous()
+        feat_src = feat_src.reshape(-1, self.out_feats * self.num_heads)
+        transposed = None
+        if isinstance(graph, Block) and torch.is_grad_enabled():
+            transposed = graph.transposed(edge_ids=True)
+        return MA_Function_GAT.apply(edge_ptr, edge_data.detach(), src_edges, dst_edges, dst_nodes, feat_src, self.num_heads,
+                                     neighbor_num, transposed)
+
+
+class GAT(nn.Module):
+    def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, dropout, heads=8):
+        super().__init__()
+        self.layers = nn.ModuleList()
+        self.layers.append(GATConv(in_feats, n_hidden, num_heads=heads))
+        for _ in range(1, n_layers - 1):
+            self.layers.append(GATConv(n_hidden * heads, n_hidden, num_heads=heads, feat_drop=dropout))
+        self.layers.append(GATConv(n_hidden * heads, n_classes, num_heads=1, feat_drop=dropout))
+        self.dropout = nn.Dropout(p=dropout)
+
+    def forward(self, blocks, features, neighbor_list=[5, 10, 15]):
+        h = features
+        for i, layer in enumerate(self.layers):
+            h = layer(blocks[i], h, neighbor_list[i])
         return h
 
 

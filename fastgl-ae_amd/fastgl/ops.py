@@ -242,26 +242,46 @@ def backward_gin(edge_ptr, src_edges, d_input, weight, input_feat, src_nodes):
     return [d_x, d_w]
 
 
-def forward_gat(*args, **kwargs):
-    raise NotImplementedError("fastgl.forward_gat: attention-weighted aggregation is not part of this library")
+def forward_gat(edge_ptr, edge_data, src_edges, input_feat, neighbor_num, dst_nodes, num_heads):
+    """fastgl.forward_gat (aggregate_acc.cpp, kernel aggregate_acc_kernel.cu:835-886):
+    ``[out]`` with ``out[d, f] = sum_e edge_data[e, f // (D / num_heads)] * input_feat[src[e], f]``
+    (``input_feat[d]`` if d has no edges)."""
+    _check_input(edge_ptr, "edge_ptr", _I32)
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(edge_data, "edge_data", (torch.float32,))
+    _check_input(input_feat, "input_feat", _FEAT)
+    return [aggregate(edge_ptr, src_edges, input_feat, mode="edge", zero_policy="self", n_rows=int(dst_nodes),
+                      edge_weight=edge_data.view(edge_data.size(0), -1), n_heads=int(num_heads))]
 
 
-def backward_gat(*args, **kwargs):
-    raise NotImplementedError("fastgl.backward_gat: attention-weighted aggregation is not part of this library")
+def backward_gat(edge_ptr, edge_data, src_edges, d_input, src_nodes, num_heads):
+    """fastgl.backward_gat (kernel aggregate_acc_kernel.cu:924-979): ``[d_x]`` with
+    ``d_x[s, f] = sum over the edges (s -> d) of edge_data[e, head(f)] * d_input[d, f]`` -- as a gather
+    over the transposed block instead of float atomics."""
+    _check_input(edge_ptr, "edge_ptr", _I32)
+    _check_input(src_edges, "src_edges", _I32)
+    _check_input(edge_data, "edge_data", (torch.float32,))
+    _check_input(d_input, "d_input", _FEAT)
+    n_dst = int(d_input.size(0))
+    t_ptr, t_idx, t_edge = block_transpose(edge_ptr, src_edges, n_dst, int(src_nodes), edge_ids=True)
+    return [aggregate(t_ptr, t_idx, d_input, mode="edge", zero_policy="zeros", n_rows=int(src_nodes),
+                      edge_weight=edge_data.view(edge_data.size(0), -1), n_heads=int(num_heads), edge_index=t_edge)]
 
 
 # ---------------------------------------------------------------------------------------
 # extensions
 # ---------------------------------------------------------------------------------------
-_MODES = {"sum": L.AGG_SUM, "mean": L.AGG_MEAN, "gcn": L.AGG_GCN, "colmean": L.AGG_COLMEAN}
+_MODES = {"sum": L.AGG_SUM, "mean": L.AGG_MEAN, "gcn": L.AGG_GCN, "colmean": L.AGG_COLMEAN, "edge": L.AGG_EDGE}
 _ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
 
 
 def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
-              out=None):
+              out=None, edge_weight=None, n_heads=1, edge_index=None):
     """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
-    accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean;
-    ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``."""
+    accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge;
+    ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``.
+    ``mode="edge"``: ``edge_weight`` float32 [n_entries, n_heads], weight of entry e for column f is
+    ``edge_weight[edge_index[e] if edge_index is not None else e, f // (D // n_heads)]``."""
     _check_input(indptr, "indptr", _I32)
     _check_input(indices, "indices", _I32)
     if not isinstance(feat, torch.Tensor) or not feat.is_cuda:
@@ -272,7 +292,19 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
         _check_input(row_norm, "row_norm", _I32)
     if col_norm is not None:
         _check_input(col_norm, "col_norm", _I32)
-    dev = _same_device(indptr, indices, feat, row_norm, col_norm)
+    if edge_weight is not None:
+        _check_input(edge_weight, "edge_weight", (torch.float32,))
+        if edge_weight.dim() != 2 or edge_weight.size(1) != int(n_heads):
+            raise RuntimeError("edge_weight must be [n_entries, n_heads]")
+        if edge_index is None and edge_weight.size(0) < indices.numel():
+            raise RuntimeError("edge_weight has fewer rows than there are entries")
+    if edge_index is not None:
+        _check_input(edge_index, "edge_index", _I32)
+        if edge_index.numel() < indices.numel():
+            raise RuntimeError("edge_index has fewer entries than indices")
+    if mode == "edge" and (edge_weight is None or feat.size(1) % int(n_heads) != 0):
+        raise RuntimeError("mode 'edge' needs edge_weight and a head count that divides the row length")
+    dev = _same_device(indptr, indices, feat, row_norm, col_norm, edge_weight, edge_index)
     n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
     if n < 0 or n > indptr.numel() - 1:
         raise RuntimeError("n_rows (%d) does not match indptr (%d entries)" % (n, indptr.numel()))
@@ -289,12 +321,14 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
         if n > 0:
             L.check(L.lib().fgl_aggregate(L.ptr(indptr), L.ptr(indices), n, None, L.ptr(feat), int(feat.stride(0)), D,
                                           L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
-                                          L.ptr(col_norm), L.ptr(out), int(out.stride(0)), L.stream_handle()))
+                                          L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index), L.ptr(out),
+                                          int(out.stride(0)), L.stream_handle()))
     return out
 
 
-def block_transpose(indptr, indices, n_rows, n_cols):
-    """Column-major companion ``(t_indptr[n_cols+1], t_indices[nnz])`` of a block CSR."""
+def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False):
+    """Column-major companion ``(t_indptr[n_cols+1], t_indices[nnz])`` of a block CSR; with
+    ``edge_ids=True`` also ``t_edge[nnz]``, the position in ``indices`` of every transposed entry."""
     _check_input(indptr, "indptr", _I32)
     _check_input(indices, "indices", _I32)
     dev = _same_device(indptr, indices)
@@ -304,10 +338,11 @@ def block_transpose(indptr, indices, n_rows, n_cols):
     with torch.cuda.device(dev):
         t_ptr = torch.empty(n_cols + 1, dtype=torch.int32, device=dev)
         t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
+        t_edge = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz] if edge_ids else None
         ws = L.workspace(lib.fgl_block_transpose_workspace_bytes(n_cols, nnz), dev)
         L.check(lib.fgl_block_transpose(L.ptr(indptr), L.ptr(indices), n_rows, None, n_cols, None, nnz, L.ptr(t_ptr),
-                                        L.ptr(t_idx), L.ptr(ws), ws.numel(), L.stream_handle()))
-    return t_ptr, t_idx
+                                        L.ptr(t_idx), L.ptr(t_edge), L.ptr(ws), ws.numel(), L.stream_handle()))
+    return (t_ptr, t_idx, t_edge) if edge_ids else (t_ptr, t_idx)
 
 
 def table_size(num: int, scale: int) -> int:

@@ -68,12 +68,13 @@ class Block:
             self._src_deg = ops.cal_deg(self.src_local, self._n_src)
         return self._src_deg
 
-    def transposed(self):
+    def transposed(self, edge_ids=False):
         """``(t_ptr int32[n_src+1], t_dst int32[E])``: for each source node the destination
-        rows it feeds (built on first use, kept for the backward pass)."""
+        rows it feeds (built on first use, kept for the backward pass); with ``edge_ids=True``
+        also ``t_edge int32[E]``, the position of every transposed entry in ``src_local``."""
         if self._transposed is None:
-            self._transposed = ops.block_transpose(self.edge_ptr, self.src_local, self._n_dst, self._n_src)
-        return self._transposed
+            self._transposed = ops.block_transpose(self.edge_ptr, self.src_local, self._n_dst, self._n_src, edge_ids=True)
+        return self._transposed if edge_ids else self._transposed[:2]
 
     def __repr__(self):
         return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())

@@ -49,7 +49,8 @@ enum fgl_agg_mode {
     FGL_AGG_SUM = 0,     /* w = 1                                             (GIN)  */
     FGL_AGG_MEAN = 1,    /* w = 1 / deg(row)                                  (SAGE) */
     FGL_AGG_GCN = 2,     /* w = (1/sqrt(row_norm[row])) * (1/sqrt(col_norm[col]))    */
-    FGL_AGG_COLMEAN = 3  /* w = 1 / max(col_norm[col], 1)   (backward of MEAN)        */
+    FGL_AGG_COLMEAN = 3, /* w = 1 / max(col_norm[col], 1)   (backward of MEAN)        */
+    FGL_AGG_EDGE = 4     /* w = edge_w[entry_id * n_heads + column / (D / n_heads)]  (GAT) */
 };
 
 /* what an output row with no entries gets */
@@ -186,28 +187,34 @@ int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_in
  * block transpose -- the column-major companion of a block CSR, which turns the
  * reference's atomic scatter in the backward kernels (aggregate_acc_kernel.cu:467-517,
  * 554-596) into an atomic-free gather.  d_t_indptr int32[n_cols_max+1],
- * d_t_indices int32[n_edges_max] (row ids, unordered within a column).
+ * d_t_indices int32[n_edges_max] (row ids, unordered within a column); d_t_edge (optional,
+ * may be NULL) int32[n_edges_max]: the position in d_indices each transposed entry came from
+ * (what per-edge data, e.g. attention weights, is indexed by).
  * ------------------------------------------------------------------------------- */
 size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max);
 int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
                         int64_t n_rows_max, const int32_t* d_n_rows,
                         int64_t n_cols_max, const int32_t* d_n_cols, int64_t n_edges_max,
-                        int32_t* d_t_indptr, int32_t* d_t_indices,
+                        int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge,
                         void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * aggregate -- the memory-aware aggregation kernels: replaces the device part of
- * fastgl.forward_gcn / forwaed_gin (aggregate_acc_kernel.cu:270-331, 375-427) and, on the
- * transposed block, of backward_gcn / backward_gin (:467-517, :554-596); adds mean.
+ * fastgl.forward_gcn / forwaed_gin / forward_gat (aggregate_acc_kernel.cu:270-331, 375-427,
+ * 835-886) and, on the transposed block, of backward_gcn / backward_gin / backward_gat
+ * (:467-517, :554-596, :924-979); adds mean.
  *   out[r, :] = sum over e in [indptr[r], indptr[r+1]) of w(r, indices[e]) * X[indices[e], :]
  * X: [*, D] with row stride ldx elements; out: [n_rows, D] with row stride ldo; both of
  * `dtype` (fp32, or bf16 with fp32 accumulation).  d_row_norm / d_col_norm: int32 degree
- * arrays as required by `mode` (else NULL).
+ * arrays as required by `mode` (else NULL).  FGL_AGG_EDGE: d_edge_w float[n_entries, n_heads],
+ * n_heads divides D, d_edge_index (optional) maps a position in d_indices to its row of
+ * d_edge_w (NULL: the position itself; the d_t_edge of a transposed block otherwise).
  * ------------------------------------------------------------------------------- */
 int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
                   int64_t n_rows_max, const int32_t* d_n_rows,
                   const void* d_x, int64_t ldx, int D, int dtype, int mode, int zero_policy,
                   const int32_t* d_row_norm, const int32_t* d_col_norm,
+                  const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
                   void* d_out, int64_t ldo, void* stream);
 
 /* ---------------------------------------------------------------------------------

@@ -13,6 +13,7 @@
  *   cuda_operators/utilis.cu:17-79            cal_deg (histogram), exclusive_sum (padded scan)
  *   cuda_operators/aggregate_acc_kernel.cu:270-331,375-427,467-517,554-596
  *                                             GCN / GIN forward and backward, zero-degree rule
+ *   cuda_operators/aggregate_acc_kernel.cu:835-886,924-979   GAT forward and backward
  *
  * Deliberate departures from the reference (each one is also what the HIP library does):
  *   - random picks are WITHOUT replacement (Floyd's subset algorithm) from a
@@ -32,6 +33,7 @@
  *   orc_idmap           numpy/python dict restatement, order-free invariants, hand cases
  *   orc_cal_deg, orc_exclusive_sum   numpy.bincount / numpy.cumsum
  *   orc_aggregate_f64   scipy.sparse products, all-ones / one-hot closed forms
+ *   orc_aggregate_edge_f64  scipy.sparse products per head; reduces to orc_aggregate_f64 for unit weights
  *   orc_transpose       scipy.sparse transpose (stable order)
  *   orc_rmat_keys       quadrant frequencies against (a,b,c,d); symmetry; determinism
  *   orc_aggregate_f32   (timing variant only) compared with orc_aggregate_f64
@@ -293,6 +295,32 @@ ORC_API void orc_aggregate_f64(const int32_t* indptr, const int32_t* indices, in
             else if (mode == 3) w = 1.0 / (double)(col_norm[c] > 1 ? col_norm[c] : 1);
             const float* x = X + c * ldx;
             for (int f = 0; f < D; ++f) o[f] += w * (double)x[f];
+        }
+    }
+}
+
+/* Attention-weighted aggregation (reference: aggregate_acc_kernel.cu:835-886 forward,
+ * :924-979 backward on the transposed lists):
+ *   out[r, f] = sum_e edge_w[id(e) * n_heads + f / (D / n_heads)] * X[indices[e], f]
+ * with id(e) = edge_index ? edge_index[e] : e.  Rows without entries as in orc_aggregate_f64. */
+ORC_API void orc_aggregate_edge_f64(const int32_t* indptr, const int32_t* indices, int64_t n_rows,
+                                    const float* X, int64_t ldx, int D, int zero_policy, const float* edge_w,
+                                    int n_heads, const int32_t* edge_index, double* out)
+{
+    const int unit = D / n_heads;
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        double* o = out + r * (int64_t)D;
+        int64_t a = indptr[r], b = indptr[r + 1];
+        if (a == b) {
+            for (int f = 0; f < D; ++f) o[f] = zero_policy == 0 ? (double)X[r * ldx + f] : 0.0;
+            continue;
+        }
+        for (int f = 0; f < D; ++f) o[f] = 0.0;
+        for (int64_t e = a; e < b; ++e) {
+            const float* x = X + (int64_t)indices[e] * ldx;
+            const float* w = edge_w + (int64_t)(edge_index ? edge_index[e] : e) * n_heads;
+            for (int f = 0; f < D; ++f) o[f] += (double)w[f / unit] * (double)x[f];
         }
     }
 }

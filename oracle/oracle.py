@@ -50,6 +50,8 @@ def lib():
         for f in (L.orc_aggregate_f64, L.orc_aggregate_f32):
             f.argtypes = [vp, vp, i64, vp, i64, i32, i32, i32, vp, vp, vp]
             f.restype = None
+        L.orc_aggregate_edge_f64.argtypes = [vp, vp, i64, vp, i64, i32, i32, vp, i32, vp, vp]
+        L.orc_aggregate_edge_f64.restype = None
         L.orc_rmat_keys.argtypes = [i64, i64, i32, i64, u64, vp]
         L.orc_rmat_keys.restype = None
         L.orc_num_threads.argtypes = []
@@ -165,6 +167,31 @@ def aggregate(indptr, indices, X, mode="sum", zero_policy=0, row_norm=None, col_
     fn = lib().orc_aggregate_f64 if out_dtype == np.float64 else lib().orc_aggregate_f32
     fn(_p(indptr), _p(indices), n_rows, _p(X), X.shape[1], D, m, zero_policy, _p(rn), _p(cn), _p(out))
     return out
+
+
+def aggregate_edge(indptr, indices, X, edge_w, zero_policy=0, edge_index=None):
+    """fp64 attention-weighted aggregation: edge_w is float32 [n_entries, n_heads]."""
+    indptr = _i32(indptr)
+    indices = _i32(indices)
+    X = np.ascontiguousarray(X, dtype=np.float32)
+    edge_w = np.ascontiguousarray(edge_w, dtype=np.float32)
+    ei = None if edge_index is None else _i32(edge_index)
+    n_rows = indptr.shape[0] - 1
+    D = X.shape[1]
+    assert D % edge_w.shape[1] == 0
+    out = np.zeros((n_rows, D), dtype=np.float64)
+    lib().orc_aggregate_edge_f64(_p(indptr), _p(indices), n_rows, _p(X), X.shape[1], D, zero_policy, _p(edge_w),
+                                 edge_w.shape[1], _p(ei), _p(out))
+    return out
+
+
+def transpose_with_edges(indptr, indices, n_cols: int):
+    """(t_ptr, t_idx, t_edge): the stable transpose plus, per transposed entry, its position in `indices`."""
+    indptr = _i32(indptr)
+    indices = _i32(indices)
+    order = np.argsort(indices, kind="stable").astype(np.int32)
+    t_ptr, t_idx = transpose(indptr, indices, n_cols)
+    return t_ptr, t_idx, order
 
 
 def rmat_keys(first_edge: int, n_edges: int, scale: int, n_nodes: int, seed: int):

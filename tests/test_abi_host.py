@@ -65,7 +65,7 @@ def test_argument_errors_are_reported_not_launched():
     assert b"fanout" in lib.fgl_last_error()
     assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
     assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table
-    assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 8, None) == 1
+    assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 1, None, None, 8, None) == 1
     assert b"dtype" in lib.fgl_last_error()
     assert lib.fgl_rmat_keys(0, 10, 40, 100, 0, None, None) == 1
 
@@ -78,8 +78,8 @@ def test_operator_input_checks_raise_runtime_error():
         fastgl.sample_node(cpu, cpu, cpu, cpu, 4, 2)
     with pytest.raises(RuntimeError, match="CUDA tensor"):
         fastgl.transfer_edge_id(cpu, cpu, cpu, 4, 8, 4, 4)
-    with pytest.raises(NotImplementedError):
-        fastgl.forward_gat()
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        fastgl.forward_gat(cpu, torch.zeros(4, 2), cpu, torch.zeros(4, 4), 2, 4, 2)
 
 
 def test_sampler_front_end_without_gpu():

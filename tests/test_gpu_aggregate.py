@@ -147,3 +147,32 @@ def test_microbench_shape(cuda, oracle, dtype, D):
         bwd = fastgl.aggregate(t_ptr, t_idx, dOd, mode=bmode, zero_policy="zeros", col_norm=dev_i32(deg, cuda))
         wantb = oracle.aggregate(w_tptr, w_tidx, dO.float().numpy(), bmode, 1, None, deg)
         assert rel_err(bwd.float().cpu().numpy(), wantb) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,unit", [(1, 64), (8, 8), (4, 32), (3, 5), (2, 301)])
+def test_edge_weighted_forward_backward(cuda, oracle, dtype, H, unit):
+    """GAT aggregation (per-edge, per-head weights) forward, and backward over the transposed block"""
+    import fastgl
+    print("aggregate edge mode H=%d unit=%d %s" % (H, unit, dtype), flush=True)
+    rng = np.random.default_rng(H * 100 + unit)
+    n_dst, n_src, D = 400, 1500, H * unit
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 10, hubs=[(7, 130)])
+    X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
+    alpha = rng.random((ptr[-1], H)).astype(np.float32)
+    d_ptr, d_idx, d_alpha = dev_i32(ptr, cuda), dev_i32(idx, cuda), torch.from_numpy(alpha).to(cuda)
+    (out,) = fastgl.forward_gat(d_ptr, d_alpha, d_idx, X, 10, n_dst, H)
+    want = oracle.aggregate_edge(ptr, idx, X.float().cpu().numpy(), alpha, zero_policy=0)
+    assert rel_err(out.float().cpu().numpy(), want) < TOL[dtype]
+    dO = torch.from_numpy(rng.standard_normal((n_dst, D)).astype(np.float32)).to(cuda).to(dtype)
+    (d_x,) = fastgl.backward_gat(d_ptr, d_alpha, d_idx, dO, n_src, H)
+    t_ptr, t_idx, t_edge = oracle.transpose_with_edges(ptr, idx, n_src)
+    wantb = oracle.aggregate_edge(t_ptr, t_idx, dO.float().cpu().numpy(), alpha, 1, edge_index=t_edge)
+    assert rel_err(d_x.float().cpu().numpy(), wantb) < TOL[dtype]
+    # the device transpose names the right edge for every transposed entry
+    g_ptr, g_idx, g_edge = fastgl.block_transpose(d_ptr, d_idx, n_dst, n_src, edge_ids=True)
+    g_edge = g_edge.cpu().numpy()
+    assert np.array_equal(np.sort(g_edge), np.arange(ptr[-1]))
+    assert np.array_equal(idx[g_edge], np.repeat(np.arange(n_src), np.diff(g_ptr.cpu().numpy())))
+    row_of_edge = np.repeat(np.arange(n_dst), deg)
+    assert np.array_equal(row_of_edge[g_edge], g_idx.cpu().numpy())

@@ -172,3 +172,47 @@ def test_merge_of_sorted_parts_by_key_range(cuda):
     want = torch.unique(torch.cat(parts))
     got = fastgl.graph._merge_sorted_unique(parts, cuda, max_items=40_000)
     assert torch.equal(got, want)
+
+
+def test_gat_forward_backward(cuda, oracle, small_graph):
+    """GAT model against dense fp64 torch; as in the reference the attention weights are constants
+    for the backward pass (MA_Function_GAT returns no gradient for them, GraphConv.py:227)."""
+    import fastgl
+    print("conv gat", flush=True)
+    input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
+    torch.manual_seed(2)
+    model = fastgl.GAT(20, 8, 5, 2, None, 0.0, heads=4).to(cuda)
+    x = torch.randn(input_nodes.numel(), 20, device=cuda, requires_grad=True)
+    out = model(blocks, x, neighbor_list=[4, 3])
+    assert tuple(out.shape) == (blocks[-1].num_dst_nodes(), 5)
+    gout = torch.randn_like(out)
+    out.backward(gout)
+
+    h = x.detach().cpu().double().requires_grad_(True)
+    cur = h
+    weights = []
+    for layer, block in zip(model.layers, blocks):
+        H, F = layer.num_heads, layer.out_feats
+        W = layer.fc.weight.detach().cpu().double().requires_grad_(True)
+        weights.append((layer, W))
+        al, ar = layer.attn_l.detach().cpu().double(), layer.attn_r.detach().cpu().double()
+        n_dst, n_src = block.num_dst_nodes(), block.num_src_nodes()
+        src, dst = (t.cpu().long() for t in block.edges())
+        z = (cur @ W.T).view(n_src, H, F)
+        el, er = (z * al).sum(-1), (z[:n_dst] * ar).sum(-1)
+        e = torch.nn.functional.leaky_relu(el[src] + er[dst], 0.2).detach()   # constants in the backward pass
+        alpha = torch.zeros_like(e)
+        for d in range(n_dst):
+            m = dst == d
+            if m.any():
+                alpha[m] = torch.softmax(e[m], 0)
+        msg = alpha[:, :, None] * z[src]                                        # [E, H, F]
+        agg = torch.zeros(n_dst, H, F, dtype=torch.float64).index_add_(0, dst, msg)
+        deg = torch.bincount(dst, minlength=n_dst)
+        agg = torch.where((deg == 0)[:, None, None], z[:n_dst].detach(), agg)   # pass-through, no gradient
+        cur = agg.reshape(n_dst, H * F)
+    cur.backward(gout.cpu().double())
+    assert torch.allclose(out.detach().cpu().double(), cur.detach(), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
+    for layer, W in weights:
+        assert torch.allclose(layer.fc.weight.grad.cpu().double(), W.grad, rtol=1e-4, atol=1e-5)

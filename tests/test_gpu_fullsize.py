@@ -70,7 +70,8 @@ def test_mid_shape_properties(cuda):
     ax = fastgl.aggregate(b0.edge_ptr, b0.src_local, x, mode="sum", zero_policy="zeros")
     atg = fastgl.aggregate(t_ptr, t_idx, g, mode="sum", zero_policy="zeros")
     a, b = (ax.double() * g.double()).sum().item(), (x.double() * atg.double()).sum().item()
-    assert abs(a - b) <= 1e-6 * max(abs(a), abs(b), 1.0)
+    scale = (ax.double().abs() * g.double().abs()).sum().item()  # the inner products cancel heavily: compare on this scale
+    assert abs(a - b) <= 1e-6 * scale
 
 
 def test_offsets_beyond_int32(cuda):

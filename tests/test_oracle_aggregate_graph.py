@@ -102,3 +102,30 @@ def test_rmat_csr_shape(oracle, small_graph):
     rev = indices.astype(np.int64) << 32 | rows
     assert np.array_equal(np.sort(rev), key)            # symmetric
     assert np.diff(indptr).max() > 2000                 # power-law tail
+
+
+def test_edge_weighted_aggregation(oracle):
+    """GAT aggregation: per head h, out[:, head-h columns] = (A o alpha_h) @ X[:, head-h columns]"""
+    rng = np.random.default_rng(13)
+    n_dst, n_src, H, unit = 120, 300, 3, 5
+    D = H * unit
+    indptr, indices, deg = _block(rng, n_dst, n_src, 8)
+    X = rng.standard_normal((n_src, D)).astype(np.float32)
+    alpha = rng.random((indptr[-1], H)).astype(np.float32)
+    got = oracle.aggregate_edge(indptr, indices, X, alpha, zero_policy=1)
+    want = np.zeros((n_dst, D))
+    for h in range(H):
+        A = sp.csr_matrix((alpha[:, h].astype(np.float64), indices, indptr), shape=(n_dst, n_src))
+        want[:, h * unit:(h + 1) * unit] = A @ X[:, h * unit:(h + 1) * unit].astype(np.float64)
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+    passthrough = oracle.aggregate_edge(indptr, indices, X, alpha, zero_policy=0)
+    assert np.array_equal(passthrough[deg == 0], X[:n_dst][deg == 0].astype(np.float64))
+    # unit weights reduce it to the plain sum
+    ones = np.ones_like(alpha)
+    assert np.allclose(oracle.aggregate_edge(indptr, indices, X, ones, 1), oracle.aggregate(indptr, indices, X, "sum", 1))
+    # backward = the same sum over the transposed lists, weights looked up through the edge ids
+    t_ptr, t_idx, t_edge = oracle.transpose_with_edges(indptr, indices, n_src)
+    assert np.array_equal(indices[t_edge], np.repeat(np.arange(n_src), np.diff(t_ptr)))
+    y = rng.standard_normal((n_dst, D)).astype(np.float32)
+    aty = oracle.aggregate_edge(t_ptr, t_idx, y, alpha, 1, edge_index=t_edge)
+    assert np.isclose((want * y).sum(), (X * aty).sum(), rtol=1e-9)
