@@ -321,11 +321,12 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
     }
 }
 
-size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
+size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)
 {
     Carver c(nullptr);
     c.take<int32_t>((size_t)n_edges_max);
     c.take<char>(scan_workspace_bytes(n_cols_max));
+    if (sorted) c.take<char>(sorted_transpose_workspace_bytes(n_cols_max, n_edges_max));
     return c.used();
 }
 
@@ -408,23 +409,25 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     return launch_agg_vec<uint16_t, 1>(mode, s, g);
 }
 
-FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max)
+FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)
 {
     if (n_cols_max < 0 || n_edges_max < 0) return 0;
-    return transpose_workspace_bytes(n_cols_max, n_edges_max);
+    return transpose_workspace_bytes(n_cols_max, n_edges_max, sorted);
 }
 
 FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
                                    const int32_t* d_n_rows, int64_t n_cols_max, const int32_t* d_n_cols,
                                    int64_t n_edges_max, int32_t* d_t_indptr, int32_t* d_t_indices,
-                                   int32_t* d_t_edge, void* d_ws, size_t ws_bytes, void* stream)
+                                   int32_t* d_t_edge, int sorted, void* d_ws, size_t ws_bytes, void* stream)
 {
+    FGL_REQUIRE(sorted == 0 || (d_n_rows == nullptr && d_n_cols == nullptr),
+                "block_transpose: the sorted variant needs exact sizes (no device-side counts)");
     FGL_REQUIRE(n_rows_max >= 0 && n_cols_max >= 0 && n_edges_max >= 0, "block_transpose: negative size");
     FGL_REQUIRE(n_edges_max <= 0x7FFFFFFF, "block_transpose: edge count exceeds int32 offsets");
     FGL_REQUIRE(d_t_indptr != nullptr, "block_transpose: null output");
     FGL_REQUIRE(n_edges_max == 0 || (d_indptr && d_indices && d_t_indices), "block_transpose: null pointer");
-    if (d_ws == nullptr || ws_bytes < transpose_workspace_bytes(n_cols_max, n_edges_max)) {
-        set_error("block_transpose: workspace too small (%zu < %zu)", ws_bytes, transpose_workspace_bytes(n_cols_max, n_edges_max));
+    if (d_ws == nullptr || ws_bytes < transpose_workspace_bytes(n_cols_max, n_edges_max, sorted)) {
+        set_error("block_transpose: workspace too small (%zu < %zu)", ws_bytes, transpose_workspace_bytes(n_cols_max, n_edges_max, sorted));
         return FGL_ERR_WORKSPACE;
     }
     hipStream_t s = as_stream(stream);
@@ -441,6 +444,12 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
     }
     rc = launch_exclusive_sum(d_t_indptr, n_cols_max, d_n_cols, d_t_indptr, nullptr, scan_ws, scan_workspace_bytes(n_cols_max), s);
     if (rc != FGL_OK) return rc;
+    if (sorted) {
+        const size_t sort_bytes = sorted_transpose_workspace_bytes(n_cols_max, n_edges_max);
+        char* sort_ws = c.take<char>(sort_bytes);
+        return launch_sorted_transpose_fill(d_indptr, d_indices, n_rows_max, n_cols_max, n_rows_max > 0 ? n_edges_max : 0,
+                                            d_t_indices, d_t_edge, sort_ws, sort_bytes, s);
+    }
     if (n_edges_max > 0 && n_rows_max > 0) {
         hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)ceil_div(n_rows_max, kBlock)), dim3(kBlock), 0, s, d_indptr,
                            d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices, d_t_edge);

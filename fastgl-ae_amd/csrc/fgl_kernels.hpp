@@ -34,4 +34,10 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          int32_t* d_n_total_out, int32_t* d_uniq, int64_t uniq_capacity, int flags,
                          uint32_t* d_status, void* d_ws, size_t ws_bytes, hipStream_t stream);
 
+// deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
+size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);
+int launch_sorted_transpose_fill(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows, int64_t n_cols,
+                                 int64_t n_edges, int32_t* d_t_indices, int32_t* d_t_edge, void* d_ws, size_t ws_bytes,
+                                 hipStream_t stream);
+
 }  // namespace fgl

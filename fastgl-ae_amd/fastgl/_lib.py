@@ -44,8 +44,8 @@ SIGNATURES = {
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64]),
-    "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64, _i32]),
+    "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _vp, _sz, _vp]),
     "fgl_aggregate": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _i64, _vp]),
     "fgl_rmat_keys": (_i32, [_i64, _i64, _i32, _i64, _u64, _vp, _vp]),
 }

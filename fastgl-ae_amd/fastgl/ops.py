@@ -326,9 +326,11 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     return out
 
 
-def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False):
+def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False, sorted_rows=False):
     """Column-major companion ``(t_indptr[n_cols+1], t_indices[nnz])`` of a block CSR; with
-    ``edge_ids=True`` also ``t_edge[nnz]``, the position in ``indices`` of every transposed entry."""
+    ``edge_ids=True`` also ``t_edge[nnz]``, the position in ``indices`` of every transposed entry.
+    ``sorted_rows=True`` lists every column's rows in ascending order (deterministic; the default
+    leaves the order within a column to scheduling and is faster)."""
     _check_input(indptr, "indptr", _I32)
     _check_input(indices, "indices", _I32)
     dev = _same_device(indptr, indices)
@@ -339,9 +341,10 @@ def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False):
         t_ptr = torch.empty(n_cols + 1, dtype=torch.int32, device=dev)
         t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
         t_edge = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz] if edge_ids else None
-        ws = L.workspace(lib.fgl_block_transpose_workspace_bytes(n_cols, nnz), dev)
+        ws = L.workspace(lib.fgl_block_transpose_workspace_bytes(n_cols, nnz, int(sorted_rows)), dev)
         L.check(lib.fgl_block_transpose(L.ptr(indptr), L.ptr(indices), n_rows, None, n_cols, None, nnz, L.ptr(t_ptr),
-                                        L.ptr(t_idx), L.ptr(t_edge), L.ptr(ws), ws.numel(), L.stream_handle()))
+                                        L.ptr(t_idx), L.ptr(t_edge), int(sorted_rows), L.ptr(ws), ws.numel(),
+                                        L.stream_handle()))
     return (t_ptr, t_idx, t_edge) if edge_ids else (t_ptr, t_idx)
 
 

@@ -23,7 +23,8 @@ class Block:
     nodes), stored as a CSR over destination rows: ``edge_ptr`` int32[n_dst+1],
     ``src_local`` int32[E].  ``src_global`` (optional) holds the same edges with graph ids."""
 
-    def __init__(self, edge_ptr, src_local, n_src, n_dst, src_global=None):
+    def __init__(self, edge_ptr, src_local, n_src, n_dst, src_global=None, sorted_transpose=False):
+        self.sorted_transpose = bool(sorted_transpose)  # deterministic order inside the transposed lists
         self.edge_ptr = edge_ptr
         self.src_local = src_local
         self._n_src = int(n_src)
@@ -73,7 +74,8 @@ class Block:
         rows it feeds (built on first use, kept for the backward pass); with ``edge_ids=True``
         also ``t_edge int32[E]``, the position of every transposed entry in ``src_local``."""
         if self._transposed is None:
-            self._transposed = ops.block_transpose(self.edge_ptr, self.src_local, self._n_dst, self._n_src, edge_ids=True)
+            self._transposed = ops.block_transpose(self.edge_ptr, self.src_local, self._n_dst, self._n_src, edge_ids=True,
+                                                   sorted_rows=self.sorted_transpose)
         return self._transposed if edge_ids else self._transposed[:2]
 
     def __repr__(self):
@@ -83,7 +85,7 @@ class Block:
 class FusedMapSampler:
     def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
                  prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0,
-                 id_order="first"):
+                 id_order="first", deterministic=False):
         if mask is not None and prob is not None:
             raise ValueError('Mask and probability arguments are mutually exclusive. '
                              'Consider multiplying the probability with the mask to achieve the same goal.')
@@ -101,6 +103,11 @@ class FusedMapSampler:
         if id_order not in ("first", "arrival"):
             raise ValueError("id_order must be 'first' or 'arrival'")
         self.id_order = id_order  # numbering of new node ids (fused path): see ops.sample_blocks_fused
+        # deterministic=True also fixes the order inside each block's transposed lists, so that the
+        # fp32 sums of the backward pass are reproducible bit for bit (costs one radix sort per block)
+        self.deterministic = bool(deterministic)
+        if self.deterministic and id_order != "first":
+            raise ValueError("deterministic=True needs id_order='first'")
         self.rng_seed = int(rng_seed)
         self.batches = 0
         self.nodes_num = 0
@@ -176,7 +183,7 @@ class FusedMapSampler:
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]
             blocks.insert(0, Block(bptr[h][:n_dst + 1], src_l[h][:n_e], n_src, n_dst,
-                                   None if src_g[h] is None else src_g[h][:n_e]))
+                                   None if src_g[h] is None else src_g[h][:n_e], sorted_transpose=self.deterministic))
         return uniq[:c[H]], seeds, blocks
 
     def _sample_layerwise(self, seeds, stream_base):
@@ -200,7 +207,8 @@ class FusedMapSampler:
                 src_global = src_out.clone() if block_index == len(self.fanouts) - 1 else None
                 src_edges, _dst_edges, seed_nodes_acc = ops.transfer_edge_id(src_out, dst_out, dst_unique, dst_nodes,
                                                                              dst_nodes + edge_nums, max_src_num, edge_nums)
-                blocks.insert(0, Block(block_ptr, src_edges, int(seed_nodes_acc.size(0)), n_dst, src_global))
+                blocks.insert(0, Block(block_ptr, src_edges, int(seed_nodes_acc.size(0)), n_dst, src_global,
+                                       sorted_transpose=self.deterministic))
                 dst_nodes = int(seed_nodes_acc.size(0))
         finally:
             ops._rng_state.update(saved)

@@ -189,13 +189,16 @@ int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_in
  * 554-596) into an atomic-free gather.  d_t_indptr int32[n_cols_max+1],
  * d_t_indices int32[n_edges_max] (row ids, unordered within a column); d_t_edge (optional,
  * may be NULL) int32[n_edges_max]: the position in d_indices each transposed entry came from
- * (what per-edge data, e.g. attention weights, is indexed by).
+ * (what per-edge data, e.g. attention weights, is indexed by).  sorted = 1 orders every column
+ * by ascending row (deterministic output, needs exact sizes: d_n_rows = d_n_cols = NULL, and
+ * n_edges_max = the number of entries); sorted = 0 is faster and leaves the order within a
+ * column to scheduling.
  * ------------------------------------------------------------------------------- */
-size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max);
+size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted);
 int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
                         int64_t n_rows_max, const int32_t* d_n_rows,
                         int64_t n_cols_max, const int32_t* d_n_cols, int64_t n_edges_max,
-                        int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge,
+                        int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge, int sorted,
                         void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------

@@ -176,3 +176,41 @@ def test_edge_weighted_forward_backward(cuda, oracle, dtype, H, unit):
     assert np.array_equal(idx[g_edge], np.repeat(np.arange(n_src), np.diff(g_ptr.cpu().numpy())))
     row_of_edge = np.repeat(np.arange(n_dst), deg)
     assert np.array_equal(row_of_edge[g_edge], g_idx.cpu().numpy())
+
+
+@pytest.mark.parametrize("n_dst,n_src,max_deg", [(3000, 9000, 15), (1, 5, 3), (50, 1, 4), (200, 70000, 2)])
+def test_sorted_transpose_is_the_stable_transpose(cuda, oracle, n_dst, n_src, max_deg):
+    """sorted_rows=True: offsets, row lists and edge ids equal the oracle's stable counting sort exactly,
+    run after run (the default variant matches only up to the order inside a column)."""
+    import fastgl
+    print("sorted transpose %d %d" % (n_dst, n_src), flush=True)
+    rng = np.random.default_rng(n_dst + n_src)
+    ptr, idx, deg = make_block(rng, n_dst, n_src, max_deg, hubs=[(0, 700)] if n_dst > 100 else ())
+    if n_dst > 100:
+        idx[:2000] = 3  # a hub column
+    w_ptr, w_idx, w_edge = oracle.transpose_with_edges(ptr, idx, n_src)
+    for _ in range(2):
+        t_ptr, t_idx, t_edge = fastgl.block_transpose(dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src, edge_ids=True,
+                                                      sorted_rows=True)
+        assert np.array_equal(t_ptr.cpu().numpy(), w_ptr)
+        assert np.array_equal(t_idx.cpu().numpy(), w_idx)
+        assert np.array_equal(t_edge.cpu().numpy(), w_edge)
+    t_ptr, t_idx = fastgl.block_transpose(dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src, sorted_rows=True)
+    assert np.array_equal(t_idx.cpu().numpy(), w_idx)
+
+
+def test_deterministic_sampler_gives_bitwise_reproducible_gradients(cuda, oracle, small_graph):
+    import fastgl
+    print("deterministic backward", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = torch.from_numpy(indptr).to(cuda), dev_i32(indices, cuda)
+    seeds = dev_i32(np.argsort(-np.diff(indptr))[:2048], cuda)  # hub seeds: long transposed lists
+    grads = []
+    for _ in range(2):
+        sampler = fastgl.FusedMapSampler([10, 10], rng_seed=1, deterministic=True).set_graph(ptr, idx)
+        _, _, blocks = sampler.sample_blocks(None, seeds)
+        b = blocks[0]
+        g = torch.randn(b.num_dst_nodes(), 64, device=cuda, generator=torch.Generator(device=cuda).manual_seed(5))
+        t_ptr, t_idx = b.transposed()
+        grads.append(fastgl.aggregate(t_ptr, t_idx, g, mode="sum", zero_policy="zeros"))
+    assert torch.equal(grads[0], grads[1])
