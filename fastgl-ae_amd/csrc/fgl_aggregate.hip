@@ -298,6 +298,7 @@ __global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* 
     else rank[e] = -1;
 }
 
+// sixteen lanes per row: the row's entries are read coalesced and scattered in parallel
 __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* __restrict__ indptr,
                                                                 const int32_t* __restrict__ indices, int64_t n_rows_max,
                                                                 const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
@@ -306,17 +307,21 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
                                                                 int32_t* __restrict__ t_indices,
                                                                 int32_t* __restrict__ t_edge)
 {
+    constexpr int kLanes = 16;
     const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= n_rows) return;
-    int64_t a = indptr[r], b = indptr[r + 1];
-    if (b > n_edges_max) b = n_edges_max;
-    for (int64_t e = a; e < b; ++e) {
-        const int32_t k = rank[e];
-        if (k >= 0) {
-            const int64_t pos = (int64_t)t_indptr[indices[e]] + k;
-            t_indices[pos] = (int32_t)r;
-            if (t_edge) t_edge[pos] = (int32_t)e;
+    const int lane = (int)threadIdx.x % kLanes;
+    const int64_t stride = (int64_t)gridDim.x * (kBlock / kLanes);
+    for (int64_t r = (int64_t)blockIdx.x * (kBlock / kLanes) + (int)threadIdx.x / kLanes; r < n_rows; r += stride) {
+        const int64_t a = indptr[r];
+        int64_t b = indptr[r + 1];
+        if (b > n_edges_max) b = n_edges_max;
+        for (int64_t e = a + lane; e < b; e += kLanes) {
+            const int32_t k = rank[e];
+            if (k >= 0) {
+                const int64_t pos = (int64_t)t_indptr[indices[e]] + k;
+                t_indices[pos] = (int32_t)r;
+                if (t_edge) t_edge[pos] = (int32_t)e;
+            }
         }
     }
 }
@@ -451,7 +456,9 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
                                             d_t_indices, d_t_edge, sort_ws, sort_bytes, s);
     }
     if (n_edges_max > 0 && n_rows_max > 0) {
-        hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)ceil_div(n_rows_max, kBlock)), dim3(kBlock), 0, s, d_indptr,
+        int64_t fill_blocks = ceil_div(n_rows_max, kBlock / 16);
+        if (fill_blocks > 16384) fill_blocks = 16384;
+        hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)fill_blocks), dim3(kBlock), 0, s, d_indptr,
                            d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices, d_t_edge);
         FGL_CHECK_LAUNCH("transpose_fill_kernel");
     }
