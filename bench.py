@@ -27,7 +27,7 @@ for _p in (ROOT, os.path.join(ROOT, "fastgl-ae_amd")):
 HBM_PEAK_GBPS = 8000.0
 # HBM traffic per launch of the dominant kernel on workload c3, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE 369898 KiB x 1.898 + WRITE_SIZE 55671 KiB x 1.000, the factors being what the same
-# counters read for this kernel run as a plain copy of known size; profiles/aggregate_kernel_c3_pmc.md)
+# counters read for this kernel run as a plain copy of known size)
 TRAFFIC_BYTES_C3 = 369898 * 1024 * 1.898 + 55671 * 1024 * 1.0
 
 WORKLOADS = {
@@ -125,13 +125,15 @@ def main():
     ap.add_argument("--cpu-batches", type=int, default=2, help="mini-batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
                     help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
+    ap.add_argument("--overlap", action="store_true",
+                    help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
-              "(mini-batches shard over GPUs by seed partition with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(mini-batches shard over GPUs by seed partition with no exchange between them)", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -225,6 +227,30 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
 
+    # ---- optional: the same steps with sampling of batch i+1 overlapped with aggregation of batch i ----
+    ms_overlapped = None
+    if args.overlap:
+        def aggregate_only(blocks):
+            b0 = blocks[0]
+            fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
+            hid, grad = inner_buffers(max([b.num_src_nodes() for b in blocks[1:]] + [1]))
+            for b in blocks[1:]:
+                fastgl.aggregate(b.edge_ptr, b.src_local, hid[:b.num_src_nodes()], mode="mean", zero_policy="zeros")
+            for b in blocks[1:]:
+                t_ptr, t_idx = b.transposed()
+                fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",
+                                 col_norm=b.in_degrees().contiguous())
+        batches = [train[(i % n_batches) * B:(i % n_batches) * B + B] for i in range(args.warmup + args.steps)]
+        torch.cuda.synchronize()
+        for i, (_, _, blocks) in enumerate(sampler.iter_batches(batches)):
+            if i == args.warmup:
+                torch.cuda.synchronize()
+                t_ov = time.perf_counter()
+            aggregate_only(blocks)
+        torch.cuda.synchronize()
+        ms_overlapped = (time.perf_counter() - t_ov) / args.steps * 1e3
+        log("overlapped: %.3f ms per step" % ms_overlapped)
+
     # ---- duration of the dominant kernel -------------------------------------------------
     # The stage interval above starts right after the sampler's host read-back, when the queue
     # is empty, so it contains the host's launch latency.  For the roofline the same launches
@@ -316,6 +342,7 @@ def main():
         "steps": K,
         "warmup": args.warmup,
         "ms_per_step": wall / K * 1e3,
+        "ms_per_step_overlapped": ms_overlapped,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

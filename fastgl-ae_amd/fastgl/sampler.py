@@ -118,6 +118,7 @@ class FusedMapSampler:
         self._shape = None
         self._plans = {}        # node-capacity tuple (None = worst case) -> BlocksPlan
         self._nodes_seen = None  # per hop: the largest node count any mini-batch has reached
+        self._side = None        # second stream of iter_batches
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
         self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
@@ -139,52 +140,114 @@ class FusedMapSampler:
             return self._sample_fused(seeds, stream_base)
         return self._sample_layerwise(seeds, stream_base)
 
-    def _sample_fused(self, seeds, stream_base):
-        hop_fanouts = list(reversed(self.fanouts))
-        H = len(hop_fanouts)
-        lib = ops.L.lib()
-        n_seeds = int(seeds.numel())
-        shape = (n_seeds, tuple(hop_fanouts), self.nodes_num, seeds.device)
-        if self._shape != shape:
-            self._shape, self._plans, self._nodes_seen = shape, {}, None
+    # -- fused path: enqueue (no host synchronisation) / finish (one read-back) -----------------
+    def _caps(self, n_seeds):
         # Worst-case bounds assume that no neighbour ever repeats: 8.6 M nodes for 8192 seeds and
         # fanouts 5/10/15 where real batches hold ~1 M, and the whole graph for deep fanouts.  A hash
         # table that fits the caches is much faster and output buffers sized by the bound cost GBs,
         # so after the first batch both are sized from the largest batch seen (x1.5, table load <=
         # 1/4).  A batch that outgrows them is detected by the kernels (status word) and simply
         # redone with the worst-case plan; results do not depend on the sizes.
-        caps = None
-        if self._nodes_seen is not None:
-            caps = tuple(max(n_seeds, -(-int(1.5 * n) // 4096) * 4096) for n in self._nodes_seen)
-        while True:
-            plan = self._plans.get(caps)
-            if plan is None:
-                plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
-                self._plans = {k: v for k, v in self._plans.items() if k is None}  # keep the worst-case plan only
-                self._plans[caps] = plan
-            slots = plan.slots
-            if caps is not None:
-                slots = min(slots, max(lib.fgl_idmap_slots(2 * self._nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
-            uniq, bptr, src_l, src_g, counts = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds,
-                                                                       self.rng_seed, stream_base, keep_global=(H - 1,),
-                                                                       table_slots=slots, id_order=self.id_order)
-            c = counts.tolist()  # the one host synchronisation of the mini-batch
+        if self._nodes_seen is None:
+            return None
+        return tuple(max(n_seeds, -(-int(1.5 * n) // 4096) * 4096) for n in self._nodes_seen)
+
+    def _launch_fused(self, seeds, stream_base, caps):
+        hop_fanouts = list(reversed(self.fanouts))
+        lib = ops.L.lib()
+        n_seeds = int(seeds.numel())
+        shape = (n_seeds, tuple(hop_fanouts), self.nodes_num, seeds.device)
+        if self._shape != shape:
+            self._shape, self._plans, self._nodes_seen, caps = shape, {}, None, None
+        plan = self._plans.get(caps)
+        if plan is None:
+            plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
+            self._plans = {k: v for k, v in self._plans.items() if k is None}  # keep the worst-case plan only
+            self._plans[caps] = plan
+        slots = plan.slots
+        if caps is not None:
+            slots = min(slots, max(lib.fgl_idmap_slots(2 * self._nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
+        out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
+                                      keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order)
+        return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out)
+
+    def _finish_fused(self, pending, counts_host):
+        """counts_host: the batch's counts as a python list (already read back)."""
+        H = len(self.fanouts)
+        c = counts_host
+        status = c[2 * H + 1]
+        if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and pending["caps"] is not None:
+            self._nodes_seen = None
+            pending = self._launch_fused(pending["seeds"], pending["stream_base"], None)
+            c = pending["out"][4].tolist()
             status = c[2 * H + 1]
-            if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and caps is not None:
-                caps = None
-                self._nodes_seen = None
-                continue
-            break
         if status:
             ops._raise_status(status, "sample_blocks")
         seen = c[:H + 1]
         self._nodes_seen = seen if self._nodes_seen is None else [max(a, b) for a, b in zip(seen, self._nodes_seen)]
+        uniq, bptr, src_l, src_g, _ = pending["out"]
         blocks = []
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]
             blocks.insert(0, Block(bptr[h][:n_dst + 1], src_l[h][:n_e], n_src, n_dst,
                                    None if src_g[h] is None else src_g[h][:n_e], sorted_transpose=self.deterministic))
-        return uniq[:c[H]], seeds, blocks
+        return uniq[:c[H]], pending["seeds"], blocks
+
+    def _sample_fused(self, seeds, stream_base):
+        pending = self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel())))
+        return self._finish_fused(pending, pending["out"][4].tolist())  # the one host synchronisation of the mini-batch
+
+    def iter_batches(self, seed_batches):
+        """Yields ``(input_nodes, output_nodes, blocks)`` for every seed batch, sampling batch i+1 on
+        a second HIP stream while the caller works on batch i (the sampling kernels are bound by
+        random-access latency, the aggregation kernels by bandwidth: they overlap well).  Results are
+        identical to calling ``sample_blocks`` batch by batch."""
+        if not self.fused:
+            for seeds in seed_batches:
+                yield self.sample_blocks(None, seeds)
+            return
+        dev = self.edge_src.device
+        main = torch.cuda.current_stream(dev)
+        if self._side is None:
+            self._side = torch.cuda.Stream(device=dev)  # default priority
+        side = self._side
+        H = len(self.fanouts)
+
+        def launch(seed_nodes):
+            seeds = seed_nodes.to(device=dev, dtype=torch.int32).contiguous()
+            stream_base = (self.batches * 64) & 0xFFFFFFFF
+            self.batches += 1
+            side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
+            with torch.cuda.stream(side):
+                pending = self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel())))
+                host = torch.empty(2 * H + 2, dtype=torch.int32, pin_memory=True)
+                host.copy_(pending["out"][4], non_blocking=True)
+                done = torch.cuda.Event()
+                done.record(side)
+            return pending, host, done
+
+        def finish(item):
+            pending, host, done = item
+            done.synchronize()
+            with torch.cuda.stream(side):  # a batch that outgrew its buffers is redone here, synchronously
+                result = self._finish_fused(pending, host.tolist())
+                redo = torch.cuda.Event()
+                redo.record(side)
+            main.wait_event(redo)
+            for t in (result[0],) + tuple(x for b in result[2] for x in (b.edge_ptr, b.src_local, b.src_global) if x is not None):
+                t.record_stream(main)  # allocated on the side stream, consumed on the caller's
+            return result
+
+        it = iter(seed_batches)
+        try:
+            item = launch(next(it))
+        except StopIteration:
+            return
+        for nxt in it:
+            ahead = launch(nxt)
+            yield finish(item)
+            item = ahead
+        yield finish(item)
 
     def _sample_layerwise(self, seeds, stream_base):
         # the reference loop (FusedMapSampler.py:72-107), one drop-in call per step

@@ -76,11 +76,16 @@ def run(args):
         n_edges = n_inputs = 0
         sync()
         tic = time.time()
+        seed_batches = (order[i * args.batch_size:(i + 1) * args.batch_size] for i in range(steps))
+        stream = sampler.iter_batches(seed_batches) if args.prefetch else None
         for step in range(steps):
-            seeds = order[step * args.batch_size:(step + 1) * args.batch_size]
             t0 = time.time()
-            input_nodes, output_nodes, blocks = sampler.sample_blocks(None, seeds)
-            sync()
+            if args.prefetch:  # batch step+1 is being sampled on a second stream while this one trains
+                input_nodes, output_nodes, blocks = next(stream)
+            else:
+                seeds = order[step * args.batch_size:(step + 1) * args.batch_size]
+                input_nodes, output_nodes, blocks = sampler.sample_blocks(None, seeds)
+                sync()
             t1 = time.time()
             batch_labels = label.index_select(0, output_nodes.long())
             if args.model == "sage":
@@ -157,6 +162,7 @@ def parse_args(argv=None):
     ap.add_argument("--weight_decay", type=float, default=0.0005)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--id_order", default="first", choices=["first", "arrival"])
+    ap.add_argument("--prefetch", type=int, default=1, help="1: sample the next mini-batch on a second stream (default)")
     ap.add_argument("--log_every", type=int, default=10)
     ap.add_argument("--log_path", default="")
     return ap.parse_args(argv)

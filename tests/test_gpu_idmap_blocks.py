@@ -192,3 +192,27 @@ def test_arrival_order_equals_oracle_after_canonical_sort(cuda, oracle, small_gr
             assert set(uniq[:b.num_src_nodes()].tolist()) == set(w_inp[:w["n_src"]].tolist())
             if b.src_global is not None:
                 assert np.array_equal(uniq[src_l], b.src_global.cpu().numpy())
+
+
+def test_pipelined_iterator_equals_batch_by_batch(cuda, oracle, small_graph):
+    """iter_batches samples ahead on a second stream; every batch must equal the oracle's (and hence
+    sample_blocks'), also while the consumer keeps the main stream busy."""
+    import fastgl
+    print("sample_blocks pipelined iterator", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    rng = np.random.default_rng(77)
+    batches = [rng.permutation(indptr.size - 1)[:700].astype(np.int32) for _ in range(6)]
+    batches[3] = np.argsort(-np.diff(indptr))[:700].astype(np.int32)  # outgrows the buffers sized by experience
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=21).set_graph(ptr, idx)
+    feat = torch.randn(indptr.size - 1, 64, device=cuda)
+    n = 0
+    for i, got in enumerate(sampler.iter_batches(dev_i32(b, cuda) for b in batches)):
+        check_blocks(oracle, indptr, indices, batches[i], [15, 10, 5], got, 21, i * 64)
+        b0 = got[2][0]
+        out = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")  # main-stream consumer
+        want = oracle.aggregate(b0.edge_ptr.cpu().numpy(), b0.src_global.cpu().numpy(), feat.cpu().numpy(), "mean", 1)
+        assert np.abs(out.cpu().numpy() - want).max() < 1e-5
+        n += 1
+    assert n == len(batches)
+    assert list(sampler.iter_batches([])) == []
