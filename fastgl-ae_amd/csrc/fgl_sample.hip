@@ -263,8 +263,10 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds, TS,
                                 stream);
     if (rc != FGL_OK) return rc;
-    if constexpr (TS == 256) if (fanout <= 32) {
-        const size_t lds_reg = (size_t)fanout * TS * sizeof(int32_t) * (d_dst_out ? 2 : 1);
+    // the register variant stages the tile's output (and, if wanted, the seed ids) in LDS: it is used
+    // while that fits comfortably in the 64 KiB a workgroup may take
+    const size_t lds_reg = (size_t)fanout * TS * sizeof(int32_t) * (d_dst_out ? 2 : 1);
+    if constexpr (TS == 256) if (fanout <= 32 && lds_reg <= 60 * 1024) {
 #define FGL_LAUNCH_REG(F)                                                                                           \
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \

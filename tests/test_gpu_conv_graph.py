@@ -216,3 +216,26 @@ def test_gat_forward_backward(cuda, oracle, small_graph):
     assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
     for layer, W in weights:
         assert torch.allclose(layer.fc.weight.grad.cpu().double(), W.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_sage_bf16_features(cuda, oracle, small_graph):
+    """bf16 feature table and activations (fp32 accumulation inside the kernels): forward and the
+    gradient of the inner layer stay within the bf16 tolerance of an fp32 run"""
+    import fastgl
+    print("conv sage bf16", flush=True)
+    indptr, _ = small_graph
+    input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
+    torch.manual_seed(3)
+    feat = torch.randn(indptr.size - 1, 32, device=cuda)
+    model = fastgl.SAGE(32, 16, 4, 2, dropout=0.0).to(cuda)
+    ref = model(blocks, feat, input_nodes=input_nodes)
+    ref.sum().backward()
+    g_ref = [p.grad.clone() for p in model.parameters()]
+    model.zero_grad()
+    model_bf = model.to(torch.bfloat16)
+    out = model_bf(blocks, feat.to(torch.bfloat16), input_nodes=input_nodes)
+    assert out.dtype == torch.bfloat16
+    assert (out.float() - ref).norm() <= 0.02 * ref.norm()
+    out.float().sum().backward()
+    for p, g in zip(model_bf.parameters(), g_ref):  # norm-wise and loose: the weights themselves are rounded to bf16 and ReLUs flip
+        assert (p.grad.float() - g).norm() <= 0.15 * g.norm() + 1e-3

@@ -216,3 +216,21 @@ def test_pipelined_iterator_equals_batch_by_batch(cuda, oracle, small_graph):
         n += 1
     assert n == len(batches)
     assert list(sampler.iter_batches([])) == []
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_sample_blocks_degenerate_batches(cuda, oracle, small_graph, fused):
+    """no seeds, repeated seeds, seeds without neighbours: same answers as the oracle"""
+    import fastgl
+    print("sample_blocks degenerate fused=%s" % fused, flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    iso = np.flatnonzero(np.diff(indptr) == 0)[:40].astype(np.int32)
+    hub = np.argsort(-np.diff(indptr))[:3].astype(np.int32)
+    cases = [np.zeros(0, np.int32), iso, np.concatenate([hub, hub, iso[:2], hub[:1]]), np.repeat(hub[:1], 100)]
+    for k, seeds in enumerate(cases):
+        sampler = fastgl.FusedMapSampler([6, 4], fused=fused, rng_seed=4).set_graph(ptr, idx)
+        got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        check_blocks(oracle, indptr, indices, seeds, [6, 4], got, 4, 0)
+        if k == 1:
+            assert all(b.num_edges() == 0 for b in got[2]) and got[0].numel() == iso.size

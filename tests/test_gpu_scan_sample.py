@@ -42,7 +42,7 @@ def _sample(cuda, indptr, indices, seeds, fanout, seed, stream):
 
 
 @pytest.mark.parametrize("ptr_dtype", [np.int32, np.int64])
-@pytest.mark.parametrize("fanout", [1, 5, 15, 48, 49, 64, 192])
+@pytest.mark.parametrize("fanout", [1, 5, 8, 9, 15, 16, 17, 20, 29, 30, 32, 33, 48, 49, 64, 192])
 def test_sample_bit_exact_vs_oracle(cuda, oracle, small_graph, ptr_dtype, fanout):
     print("sample fanout=%d ptr=%s" % (fanout, ptr_dtype.__name__), flush=True)
     indptr, indices = small_graph
