@@ -19,13 +19,16 @@
 //                 so a bound much larger than the batch costs nothing)
 //   4. assign     per tile: scan of the flags -> local ids for the first edges; writes the
 //                 slot's val and appends the id to the unique list
-//   5. relabel    per edge: src_out[e] = val of the remembered slot
+//   5. relabel    src_out[e] = val of the remembered slot, for the edges that mention an id new in
+//                 this call.  Edges whose id was numbered before were already relabelled by pass 1
+//                 from the val it had loaded anyway.
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
 namespace fgl {
 
 constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+constexpr uint32_t kDone = 0xFFFFFFFEu;  // slot_of[] marker: the edge already has its local id
 constexpr uint32_t kHashMul = 0x9E3779B1u;
 constexpr int kItems = 8;
 constexpr int kTile = kBlock * kItems;
@@ -66,7 +69,8 @@ constexpr uint32_t kMaxProbes = 4096;
 // key and vals only ever decrease while inserts run, so an ordinary (cacheable, possibly stale)
 // load is enough for the first look: a stale "empty" is settled by the 64-bit CAS, which
 // installs key and val in one atomic, and a stale val can only cause a redundant atomicMin.
-__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new)
+// *seen_val receives the val found with the key (val_if_new if this call installed the key).
+__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new, uint32_t* seen_val)
 {
     unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
     const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)val_if_new << 32);
@@ -76,11 +80,15 @@ __device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id
         unsigned long long s = slots[p];
         if ((uint32_t)s == kEmpty) {
             const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
-            if (seen == ~0ull) return p;
+            if (seen == ~0ull) {
+                *seen_val = val_if_new;
+                return p;
+            }
             s = seen;
         }
         if ((uint32_t)s == id) {
-            if ((uint32_t)(s >> 32) > val_if_new) atomicMin(&t.words[2 * (size_t)p + 1], val_if_new);
+            *seen_val = (uint32_t)(s >> 32);
+            if (*seen_val > val_if_new) atomicMin(&t.words[2 * (size_t)p + 1], val_if_new);
             return p;
         }
         p = (p + 1) & t.mask;
@@ -111,14 +119,17 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, co
     if (i >= n) return;
     const int32_t id = ids[i];
     if (uniq != nullptr && uniq != ids) uniq[i] = id;
-    const uint32_t p = find_or_insert(t, (uint32_t)id, (uint32_t)i);  // a repeated id keeps its first position
+    uint32_t seen;
+    const uint32_t p = find_or_insert(t, (uint32_t)id, (uint32_t)i, &seen);  // a repeated id keeps its first position
     if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
 }
 
-__global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* __restrict__ src,
+// `src` and `out` may be the same array (relabelling in place): neither is __restrict__.
+__global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* src,
                                                                   int64_t e_max, const int32_t* __restrict__ d_e,
                                                                   int64_t n_base_h, const int32_t* __restrict__ d_n_base,
-                                                                  uint32_t* __restrict__ slot_of, uint32_t* __restrict__ d_status)
+                                                                  uint32_t* __restrict__ slot_of, int32_t* out,
+                                                                  uint32_t* __restrict__ d_status)
 {
     const int64_t n_e = actual_count(e_max, d_e);
     const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
@@ -126,9 +137,17 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         // ids numbered earlier hold val < n_base and stay as they are; a new id keeps the smallest
         // n_base + (edge index) among the edges that mention it
-        const uint32_t p = find_or_insert(t, (uint32_t)src[e], n_base + (uint32_t)e);
+        uint32_t seen;
+        uint32_t p = find_or_insert(t, (uint32_t)src[e], n_base + (uint32_t)e, &seen);
+        if (p == kEmpty) {
+            if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+        } else if (seen < n_base) {
+            // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
+            // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
+            out[e] = (int32_t)seen;
+            p = kDone;
+        }
         slot_of[e] = p;
-        if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
     }
 }
 
@@ -151,11 +170,11 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
         for (int j = 0; j < kItems; ++j) p[j] = (first + j < n_e) ? slot_of[first + j] : kEmpty;
         uint32_t v[kItems];
 #pragma unroll
-        for (int j = 0; j < kItems; ++j) v[j] = (p[j] != kEmpty) ? t.words[2 * (size_t)p[j] + 1] : 0u;
+        for (int j = 0; j < kItems; ++j) v[j] = (p[j] < kDone) ? t.words[2 * (size_t)p[j] + 1] : 0u;
         uint32_t bits = 0;
 #pragma unroll
         for (int j = 0; j < kItems; ++j)
-            if (p[j] != kEmpty && v[j] == n_base + (uint32_t)(first + j)) bits |= 1u << j;
+            if (p[j] < kDone && v[j] == n_base + (uint32_t)(first + j)) bits |= 1u << j;
         flags8[tile * kBlock + threadIdx.x] = (uint8_t)bits;
         int total;
         (void)block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
@@ -225,14 +244,18 @@ __global__ __launch_bounds__(kBlock) void idmap_assign_kernel(TableRef t, const 
     }
 }
 
+// Edges whose id was numbered before this call were relabelled by the insert pass; the others
+// (mentions of ids that are new in this call) read their local id from the remembered slot.
+// (Letting the assign pass relabel the first mention itself was measured: its scattered 4-byte
+// writes cost more than the table reads they save here.)
 __global__ __launch_bounds__(kBlock) void idmap_relabel_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
-                                                               const uint32_t* __restrict__ slot_of,
-                                                               int32_t* __restrict__ out)
+                                                               const uint32_t* __restrict__ slot_of, int32_t* __restrict__ out)
 {
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
+        if (p == kDone) continue;
         out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
     }
 }
@@ -412,7 +435,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     }
 
     hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
-                       n_edges_max, d_n_edges, n_base, d_n_base, slot_of, d_status);
+                       n_edges_max, d_n_edges, n_base, d_n_base, slot_of, d_src_out, d_status);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges, n_base,
                        d_n_base, slot_of, flags8, sums);
