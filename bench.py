@@ -269,6 +269,21 @@ def main():
     torch.cuda.synchronize()
     t_kernel0 = ra.elapsed_time(rb)
 
+    # ---- context: what a plain streaming copy reaches on this box ---------------------------
+    cp_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    cp_dst = torch.empty_like(cp_src)
+    cp_dst.copy_(cp_src)
+    ca, cb = ev(), ev()
+    torch.cuda.synchronize()
+    ca.record()
+    for _ in range(10):
+        cp_dst.copy_(cp_src)
+    cb.record()
+    torch.cuda.synchronize()
+    stream_gbps = 10 * 2 * (1 << 30) / (ca.elapsed_time(cb) * 1e-3) / 1e9  # bytes read + bytes written
+    del cp_src, cp_dst
+    log("1 GiB device copy: %.0f GB/s (read + write)" % stream_gbps)
+
     if args.pmc_copy_mib > 0:
         a = torch.zeros(args.pmc_copy_mib << 20, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
@@ -354,7 +369,8 @@ def main():
                            "feature table); block transpose + bwd gather on the inner blocks; no dense layers"},
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
                       "transpose_agg_bwd_inner": t_bwd / K},
-        "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS},
+        "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,
+                        "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
