@@ -270,10 +270,25 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
                 IO::fma(part, w3, r3);
             }
         }
-        for (; t < cnt; ++t) {
+        // the last one to three entries: their loads are issued together as well (most lists of a
+        // transposed block have only this tail)
+        const int rem = cnt - t;
+        if (rem > 0) {
             const int c0 = __shfl(my_col, t, LPR);
+            const int c1 = __shfl(my_col, rem > 1 ? t + 1 : t, LPR);
+            const int c2 = __shfl(my_col, rem > 2 ? t + 2 : t, LPR);
             const float w0 = __shfl(my_w, t, LPR);
-            if (live) IO::fma(part, w0, load_row(X + (int64_t)c0 * ldx + col0));
+            const float w1 = __shfl(my_w, rem > 1 ? t + 1 : t, LPR);
+            const float w2 = __shfl(my_w, rem > 2 ? t + 2 : t, LPR);
+            if (live) {
+                const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
+                typename IO::Raw r1 = r0, r2 = r0;
+                if (rem > 1) r1 = load_row(X + (int64_t)c1 * ldx + col0);
+                if (rem > 2) r2 = load_row(X + (int64_t)c2 * ldx + col0);
+                IO::fma(part, w0, r0);
+                if (rem > 1) IO::fma(part, w1, r1);
+                if (rem > 2) IO::fma(part, w2, r2);
+            }
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] += part[i];
