@@ -234,3 +234,40 @@ def test_sample_blocks_degenerate_batches(cuda, oracle, small_graph, fused):
         check_blocks(oracle, indptr, indices, seeds, [6, 4], got, 4, 0)
         if k == 1:
             assert all(b.num_edges() == 0 for b in got[2]) and got[0].numel() == iso.size
+
+
+def _colliding_ids(n, lg_slots):
+    """n distinct non-negative ids whose multiplicative hash lands in ONE home slot of a 2^lg table"""
+    inv = pow(0x9E3779B1, -1, 1 << 32)
+    ids, j = [], 0
+    while len(ids) < n:
+        v = (inv * ((0x5A << (32 - 8)) + j)) % (1 << 32)  # id * M mod 2^32 == fixed top bits | j
+        j += 1
+        if v < (1 << 31):
+            ids.append(v)
+    ids = np.array(ids, dtype=np.int64)
+    home = ((ids * 0x9E3779B1) % (1 << 32)) >> (32 - lg_slots)
+    assert np.unique(home).size == 1 and np.unique(ids).size == n
+    return ids.astype(np.int32)
+
+
+def test_hash_collisions_and_probe_limit(cuda, oracle):
+    """2000 ids that all hash to one slot: long probe chains, same answer as the oracle.  5000 of them
+    exceed the probe limit: reported through the status word, not by an endless loop."""
+    import fastgl
+    print("idmap collisions", flush=True)
+    rng = np.random.default_rng(0)
+    for n_ids, ok in ((2000, True), (5000, False)):
+        n_edges = 20000
+        lg = int(np.log2(fastgl.lib().fgl_idmap_slots(16 + n_edges)))
+        ids = _colliding_ids(n_ids, lg)
+        dst_unique = ids[:16].copy()
+        src = ids[rng.integers(0, n_ids, size=n_edges)]
+        dst = dst_unique[np.sort(rng.integers(0, 16, size=n_edges))]
+        if ok:
+            s, d, u = run_transfer(cuda, src, dst, dst_unique, 1 << 31)
+            ws, wd, wu = oracle.idmap(src, dst, dst_unique)
+            assert np.array_equal(s, ws) and np.array_equal(d, wd) and np.array_equal(u, wu)
+        else:
+            with pytest.raises(RuntimeError, match="hash table full"):
+                run_transfer(cuda, src, dst, dst_unique, 1 << 31)
