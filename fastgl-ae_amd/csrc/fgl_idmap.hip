@@ -5,23 +5,26 @@
 // hash = (id * 0x9E3779B1) >> (32 - log2 slots), linear probing (8 slots per 64-byte line),
 // every probe loop bounded by the slot count.  `val` is the node's local id once the id is
 // numbered; while a batch of new ids is being numbered it transiently holds
-// n_base + (index of the first edge that mentions the id), maintained with atomicMin, so that
+// kPending | (index of the first edge that mentions the id), maintained with atomicMin, so that
 // new ids are numbered in first-occurrence order -- deterministic, and the order DGL's
 // to_block gives -- instead of the reference's race on one global counter (id_map.cu:317-320).
 //
-// map_src = five launches:
-//   1. insert     per edge: probe (one 8-byte load per slot), install {key, first-edge index}
-//                 with one 64-bit CAS if new, else atomicMin the first-edge index; remember the slot
+// map_src = four launches:
+//   1. insert     per edge: probe (one 8-byte load per slot), install {key, pending first-edge index}
+//                 with one 64-bit CAS if new, else atomicMin the first-edge index; remember the slot.
+//                 An id that was numbered before this call is relabelled on the spot from the val
+//                 the probe has loaded anyway, and the edge takes no further part.
 //   2. mark       per edge: "am I the first edge of a new id?" -> one flag bit per edge
-//                 (8 edges per lane, one byte) + per-tile counts
+//                 (8 edges per lane, one byte), the count of flags before each byte within its tile
+//                 of 2048 edges, and per-tile counts
 //   3. prefix     single workgroup over the tile counts; publishes the new node total
 //                 (the edge-parallel launches are grid-stride loops over the actual count,
 //                 so a bound much larger than the batch costs nothing)
-//   4. assign     per tile: scan of the flags -> local ids for the first edges; writes the
-//                 slot's val and appends the id to the unique list
-//   5. relabel    src_out[e] = val of the remembered slot, for the edges that mention an id new in
-//                 this call.  Edges whose id was numbered before were already relabelled by pass 1
-//                 from the val it had loaded anyway.
+//   4. number     per edge, coalesced: a first edge computes its id's local id from the three
+//                 counts, stores it in the slot, appends the id to the unique list and relabels
+//                 itself without reading the table; a later mention reads the slot and, if the
+//                 val there is still the pending first-edge index, computes the same local id
+//                 from that edge's counts -- either way the same number, so the race is benign.
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
@@ -29,6 +32,7 @@ namespace fgl {
 
 constexpr uint32_t kEmpty = 0xFFFFFFFFu;
 constexpr uint32_t kDone = 0xFFFFFFFEu;  // slot_of[] marker: the edge already has its local id
+constexpr uint32_t kPending = 0x80000000u;  // val = kPending | first edge index until the id is numbered
 constexpr uint32_t kHashMul = 0x9E3779B1u;
 constexpr int kItems = 8;
 constexpr int kTile = kBlock * kItems;
@@ -127,21 +131,19 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, co
 // `src` and `out` may be the same array (relabelling in place): neither is __restrict__.
 __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* src,
                                                                   int64_t e_max, const int32_t* __restrict__ d_e,
-                                                                  int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                   uint32_t* __restrict__ slot_of, int32_t* out,
                                                                   uint32_t* __restrict__ d_status)
 {
     const int64_t n_e = actual_count(e_max, d_e);
-    const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
-        // ids numbered earlier hold val < n_base and stay as they are; a new id keeps the smallest
-        // n_base + (edge index) among the edges that mention it
+        // ids numbered earlier hold a local id (no pending bit) and stay as they are; a new id keeps
+        // the smallest pending edge index among the edges that mention it
         uint32_t seen;
-        uint32_t p = find_or_insert(t, (uint32_t)src[e], n_base + (uint32_t)e, &seen);
+        uint32_t p = find_or_insert(t, (uint32_t)src[e], kPending | (uint32_t)e, &seen);
         if (p == kEmpty) {
             if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
-        } else if (seen < n_base) {
+        } else if (!(seen & kPending)) {
             // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
             // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
             out[e] = (int32_t)seen;
@@ -153,15 +155,15 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
 
 __device__ __forceinline__ int64_t tiles_of(int64_t n) { return (n + kTile - 1) / kTile; }
 
-// flags8[tile*256 + lane] bit j  <=>  edge (tile*2048 + lane*8 + j) is the first edge of a new id
+// flags8[tile*256 + lane] bit j  <=>  edge (tile*2048 + lane*8 + j) is the first edge of a new id;
+// before8[tile*256 + lane] = number of flagged edges of the tile before edge tile*2048 + lane*8
 __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
-                                                            int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                             const uint32_t* __restrict__ slot_of,
-                                                            uint8_t* __restrict__ flags8, int32_t* __restrict__ tile_sums)
+                                                            uint8_t* __restrict__ flags8, uint16_t* __restrict__ before8,
+                                                            int32_t* __restrict__ tile_sums)
 {
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
-    const uint32_t n_base = d_n_base ? (uint32_t)(*d_n_base) : (uint32_t)n_base_h;
     const int64_t n_tiles = tiles_of(n_e);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t first = tile * kTile + (int64_t)threadIdx.x * kItems;
@@ -174,10 +176,11 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
         uint32_t bits = 0;
 #pragma unroll
         for (int j = 0; j < kItems; ++j)
-            if (p[j] < kDone && v[j] == n_base + (uint32_t)(first + j)) bits |= 1u << j;
+            if (p[j] < kDone && v[j] == (kPending | (uint32_t)(first + j))) bits |= 1u << j;
         flags8[tile * kBlock + threadIdx.x] = (uint8_t)bits;
         int total;
-        (void)block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
+        const int before = block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
+        before8[tile * kBlock + threadIdx.x] = (uint16_t)before;
         if (threadIdx.x == 0) tile_sums[tile] = total;
     }
 }
@@ -213,50 +216,54 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
     }
 }
 
-__global__ __launch_bounds__(kBlock) void idmap_assign_kernel(TableRef t, const int32_t* __restrict__ src, int64_t e_max,
+// Local id of the new node whose first mention is edge e (an edge that the mark pass flagged).
+__device__ __forceinline__ int64_t local_of_first_edge(int64_t n_base, int64_t e, uint32_t byte_flags,
+                                                       const uint16_t* __restrict__ before8,
+                                                       const int32_t* __restrict__ tile_prefix)
+{
+    return n_base + tile_prefix[e / kTile] + before8[e >> 3] + __popc(byte_flags & ((1u << (e & 7)) - 1u));
+}
+
+// Lane per edge.  `src` and `out` may be the same array: an entry is read and written by one lane only.
+// (Edges whose id was numbered before this call were relabelled by the insert pass.)
+__global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const int32_t* src, int64_t e_max,
                                                               const int32_t* __restrict__ d_e, int64_t n_base_h,
                                                               const int32_t* __restrict__ d_n_base,
                                                               const uint32_t* __restrict__ slot_of,
                                                               const uint8_t* __restrict__ flags8,
+                                                              const uint16_t* __restrict__ before8,
                                                               const int32_t* __restrict__ tile_prefix,
-                                                              int32_t* __restrict__ uniq, int64_t capacity)
+                                                              int32_t* __restrict__ uniq, int64_t capacity, int32_t* out)
 {
-    __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-    const int64_t n_tiles = tiles_of(n_e);
-    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const int64_t first = tile * kTile + (int64_t)threadIdx.x * kItems;
-        const uint32_t bits = first < n_e ? flags8[tile * kBlock + threadIdx.x] : 0u;
-        int total;
-        int64_t local = n_base + tile_prefix[tile] + block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
-#pragma unroll
-        for (int j = 0; j < kItems; ++j) {
-            if (bits & (1u << j)) {
-                const int64_t e = first + j;
-                if (local < capacity) {
-                    t.words[2 * (size_t)slot_of[e] + 1] = (uint32_t)local;
-                    uniq[local] = src[e];
-                }
-                ++local;
-            }
-        }
-    }
-}
-
-// Edges whose id was numbered before this call were relabelled by the insert pass; the others
-// (mentions of ids that are new in this call) read their local id from the remembered slot.
-// (Letting the assign pass relabel the first mention itself was measured: its scattered 4-byte
-// writes cost more than the table reads they save here.)
-__global__ __launch_bounds__(kBlock) void idmap_relabel_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
-                                                               const uint32_t* __restrict__ slot_of, int32_t* __restrict__ out)
-{
-    const int64_t n_e = actual_count(e_max, d_e);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
         if (p == kDone) continue;
-        out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
+        int64_t local = -1;
+        if (p != kEmpty) {
+            const uint32_t f = flags8[e >> 3];
+            if ((f >> (e & 7)) & 1u) {
+                local = local_of_first_edge(n_base, e, f, before8, tile_prefix);
+                if (local < capacity) {
+                    t.words[2 * (size_t)p + 1] = (uint32_t)local;
+                    uniq[local] = src[e];
+                }
+            } else {
+                const uint32_t v = t.words[2 * (size_t)p + 1];
+                if (!(v & kPending)) {
+                    local = (int64_t)v;
+                } else {
+                    // the first edge's lane has not stored the local id yet (or this lane's cache has
+                    // not seen it): derive it the way that lane does
+                    const int64_t ef = (int64_t)(v & ~kPending);
+                    if (ef < n_e) local = local_of_first_edge(n_base, ef, flags8[ef >> 3], before8, tile_prefix);
+                }
+            }
+            if (local >= capacity) local = -1;  // the unique list is full (reported by the prefix pass)
+        }
+        out[e] = (int32_t)local;
     }
 }
 
@@ -391,6 +398,7 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
     Carver c(nullptr);
     c.take<uint32_t>((size_t)n_edges_max);      // slot_of
     c.take<uint8_t>((size_t)tiles * kBlock);    // flags8
+    c.take<uint16_t>((size_t)tiles * kBlock);   // before8
     c.take<int32_t>((size_t)tiles);             // tile sums
     c.take<int32_t>((size_t)tiles);             // tile prefix
     return c.used();
@@ -404,7 +412,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE(flags == FGL_IDMAP_ORDERED || flags == FGL_IDMAP_ARRIVAL, "idmap_map_src: unknown flags %d", flags);
     FGL_REQUIRE(n_edges_max >= 0 && n_base >= 0 && uniq_capacity >= 0, "idmap_map_src: negative size");
-    FGL_REQUIRE(n_base + n_edges_max <= 0xFFFFFFFEll, "idmap_map_src: n_base + n_edges exceeds 32 bits");
+    FGL_REQUIRE(n_base + n_edges_max <= 0x7FFFFFFFll, "idmap_map_src: n_base + n_edges exceeds 31 bits");
     FGL_REQUIRE(n_edges_max == 0 || (d_src_in && d_src_out && d_uniq), "idmap_map_src: null pointer");
     FGL_REQUIRE(d_n_total_out == nullptr || d_n_total_out != d_n_base, "idmap_map_src: n_total_out must not alias n_base");
     if (d_ws == nullptr || ws_bytes < idmap_map_src_workspace_bytes(n_edges_max)) {
@@ -415,6 +423,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     Carver c(d_ws);
     uint32_t* slot_of = c.take<uint32_t>((size_t)n_edges_max);
     uint8_t* flags8 = c.take<uint8_t>((size_t)tiles * kBlock);
+    uint16_t* before8 = c.take<uint16_t>((size_t)tiles * kBlock);
     int32_t* sums = c.take<int32_t>((size_t)tiles);
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
     const TableRef t = make_ref(d_table, slots);
@@ -435,20 +444,17 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     }
 
     hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
-                       n_edges_max, d_n_edges, n_base, d_n_base, slot_of, d_src_out, d_status);
+                       n_edges_max, d_n_edges, slot_of, d_src_out, d_status);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
-    hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges, n_base,
-                       d_n_base, slot_of, flags8, sums);
+    hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
+                       slot_of, flags8, before8, sums);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
     hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max, d_n_edges,
                        n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
     FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
-    hipLaunchKernelGGL(idmap_assign_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
-                       d_n_edges, n_base, d_n_base, slot_of, flags8, prefix, d_uniq, uniq_capacity);
-    FGL_CHECK_LAUNCH("idmap_assign_kernel");
-    hipLaunchKernelGGL(idmap_relabel_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max,
-                       d_n_edges, slot_of, d_src_out);
-    FGL_CHECK_LAUNCH("idmap_relabel_kernel");
+    hipLaunchKernelGGL(idmap_number_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
+                       d_n_edges, n_base, d_n_base, slot_of, flags8, before8, prefix, d_uniq, uniq_capacity, d_src_out);
+    FGL_CHECK_LAUNCH("idmap_number_kernel");
     return FGL_OK;
 }
 

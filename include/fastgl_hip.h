@@ -131,7 +131,8 @@ int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids,
  * New ids get n_base, n_base+1, ... and are appended to d_uniq -- in order of first
  * occurrence in d_src_in (flags = FGL_IDMAP_ORDERED) or of arrival (FGL_IDMAP_ARRIVAL);
  * d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
- * *d_n_total_out = n_base + number of new ids (must not alias d_n_base). */
+ * *d_n_total_out = n_base + number of new ids (must not alias d_n_base).
+ * n_base + n_edges_max must stay below 2^31. */
 size_t fgl_idmap_map_src_workspace_bytes(int64_t n_edges_max);
 int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
                       int64_t n_edges_max, const int32_t* d_n_edges,
