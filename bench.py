@@ -283,6 +283,21 @@ def main():
     stream_gbps = 10 * 2 * (1 << 30) / (ca.elapsed_time(cb) * 1e-3) / 1e9  # bytes read + bytes written
     del cp_src, cp_dst
     log("1 GiB device copy: %.0f GB/s (read + write)" % stream_gbps)
+    # ---- context: the rate of independent random 4-byte reads from the graph's edge array (what
+    # bounds the sampling kernels), measured with a library gather of 16 M random positions
+    ra_idx = torch.randint(0, edge_src.numel(), (1 << 24,), device=dev, dtype=torch.int64)
+    ra_out = torch.empty(1 << 24, dtype=edge_src.dtype, device=dev)
+    torch.index_select(edge_src, 0, ra_idx, out=ra_out)
+    ca, cb = ev(), ev()
+    torch.cuda.synchronize()
+    ca.record()
+    for _ in range(5):
+        torch.index_select(edge_src, 0, ra_idx, out=ra_out)
+    cb.record()
+    torch.cuda.synchronize()
+    random_read_gps = 5 * (1 << 24) / (ca.elapsed_time(cb) * 1e-3) / 1e9
+    del ra_idx, ra_out
+    log("random 4-byte reads from the edge array: %.1f G/s" % random_read_gps)
 
     if args.pmc_copy_mib > 0:
         a = torch.zeros(args.pmc_copy_mib << 20, dtype=torch.uint8, device=dev)
@@ -371,6 +386,7 @@ def main():
                       "transpose_agg_bwd_inner": t_bwd / K},
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,
                         "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
+        "random_read_Gps": random_read_gps,
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
