@@ -130,6 +130,8 @@ struct AggArgs {
     // FGL_AGG_EDGE only: per-entry, per-head weights w[entry_id * n_heads + head(column)]
     const float* edge_w;
     const int32_t* edge_index;  // entry -> entry_id (NULL: the entry's own position)
+    const int32_t* longest_row; // device: entry count of the longest row, if the caller has it (NULL: unknown)
+    int skip_rows_longer_than;  // aggregate_kernel leaves rows with more entries to aggregate_long_rows_kernel
     int n_heads;
     int unit_dim;               // D / n_heads
 };
@@ -146,91 +148,40 @@ __device__ __forceinline__ float edge_weight(int col, float row_factor, const in
     return row_factor;  // SUM: 1, MEAN: 1/deg(row)
 }
 
-template <typename T, int VEC, int LPR, int MODE>
-__global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
-{
+// A lane's share of a row: VEC consecutive columns starting at col0 (possibly cut off by the row's end).
+template <typename T, int VEC>
+struct LaneSlice {
     using IO = RowIO<T, VEC>;
-    constexpr int kGroups = kBlock / LPR;
-    const int32_t* __restrict__ indptr = g.indptr;
-    const int32_t* __restrict__ indices = g.indices;
-    const T* __restrict__ X = static_cast<const T*>(g.x);
-    T* __restrict__ out = static_cast<T*>(g.out);
-    const int64_t ldx = g.ldx, ldo = g.ldo;
-    const int D = g.D;
-
-    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
-    const int gl = (int)threadIdx.x % LPR;  // lane within the group
-    const int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
-    if (row >= n_rows) return;  // uniform per group: the cross-lane reads below stay inside the group
-    const int col0 = ((int)blockIdx.y * LPR + gl) * VEC;
-    const int nvalid = D - col0;       // elements of this lane's vector that exist in the row
-    const bool live = nvalid > 0;
-    const bool full = nvalid >= VEC;   // false only for the last lane of a row with D % VEC != 0
-    auto load_row = [&](const T* p) { return full ? IO::load(p) : IO::load_partial(p, nvalid); };
-    auto store_row = [&](T* p, const float (&a)[VEC]) {
+    int col0;
+    int nvalid;  // elements of this lane's vector that exist in the row
+    bool live;
+    bool full;   // false only for the last lane of a row with D % VEC != 0
+    __device__ __forceinline__ LaneSlice(int slice, int lanes, int gl, int D)
+    {
+        col0 = (slice * lanes + gl) * VEC;
+        nvalid = D - col0;
+        live = nvalid > 0;
+        full = nvalid >= VEC;
+    }
+    __device__ __forceinline__ typename IO::Raw load(const T* p) const { return full ? IO::load(p) : IO::load_partial(p, nvalid); }
+    __device__ __forceinline__ void store(T* p, const float (&a)[VEC]) const
+    {
         if (full) IO::store(p, a);
         else IO::store_partial(p, a, nvalid);
-    };
-
-    const int a = indptr[row], b = indptr[row + 1];
-    float acc[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
-
-    if (a == b) {
-        if (live) {
-            if (g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, load_row(X + row * ldx + col0));
-            store_row(out + row * ldo + col0, acc);
-        }
-        return;
     }
+};
 
-    if constexpr (MODE == FGL_AGG_EDGE) {
-        // attention-style weights: one float per (entry, head); a lane's VEC columns lie in one
-        // head when unit_dim is a multiple of VEC, else each column looks its head up
-        const float* __restrict__ ew = g.edge_w;
-        const int H = g.n_heads, unit = g.unit_dim;
-        const bool one_head = (unit % VEC) == 0;
-        int head[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const int c = col0 + i < D ? col0 + i : D - 1;
-            head[i] = c / unit;
-        }
-        for (int base = a; base < b; base += LPR) {
-            const int cnt = (b - base) < LPR ? (b - base) : LPR;
-            int my_col = 0, my_eid = 0;
-            if (gl < cnt) {
-                my_col = indices[base + gl];
-                my_eid = g.edge_index ? g.edge_index[base + gl] : base + gl;
-            }
-            float part[VEC];  // this chunk's sum (see the note on two-level summation below)
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
-            for (int t = 0; t < cnt; ++t) {
-                const int c0 = __shfl(my_col, t, LPR);
-                const int64_t e0 = __shfl(my_eid, t, LPR);
-                if (live) {
-                    const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
-                    if (one_head) {
-                        IO::fma(part, ew[e0 * H + head[0]], r0);
-                    } else {
-                        float x[VEC];
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i) x[i] = 0.0f;
-                        IO::fma(x, 1.0f, r0);
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i) part[i] += ew[e0 * H + head[i]] * x[i];
-                    }
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] += part[i];
-        }
-        if (live) store_row(out + row * ldo + col0, acc);
-        return;
-    }
-
+// acc += sum over the entries [a, b) of one row (a < b), all modes except FGL_AGG_EDGE.
+template <typename T, int VEC, int LPR, int MODE>
+__device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, VEC>& ls, int gl, int64_t row, int a, int b,
+                                           float (&acc)[VEC])
+{
+    using IO = RowIO<T, VEC>;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    const int64_t ldx = g.ldx;
+    const int col0 = ls.col0;
+    const bool live = ls.live;
     float row_factor = 1.0f;
     if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
     if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
@@ -260,10 +211,10 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
             const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
             const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
             if (live) {
-                const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
-                const typename IO::Raw r1 = load_row(X + (int64_t)c1 * ldx + col0);
-                const typename IO::Raw r2 = load_row(X + (int64_t)c2 * ldx + col0);
-                const typename IO::Raw r3 = load_row(X + (int64_t)c3 * ldx + col0);
+                const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r1 = ls.load(X + (int64_t)c1 * ldx + col0);
+                const typename IO::Raw r2 = ls.load(X + (int64_t)c2 * ldx + col0);
+                const typename IO::Raw r3 = ls.load(X + (int64_t)c3 * ldx + col0);
                 IO::fma(part, w0, r0);
                 IO::fma(part, w1, r1);
                 IO::fma(part, w2, r2);
@@ -281,10 +232,10 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
             const float w1 = __shfl(my_w, rem > 1 ? t + 1 : t, LPR);
             const float w2 = __shfl(my_w, rem > 2 ? t + 2 : t, LPR);
             if (live) {
-                const typename IO::Raw r0 = load_row(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
                 typename IO::Raw r1 = r0, r2 = r0;
-                if (rem > 1) r1 = load_row(X + (int64_t)c1 * ldx + col0);
-                if (rem > 2) r2 = load_row(X + (int64_t)c2 * ldx + col0);
+                if (rem > 1) r1 = ls.load(X + (int64_t)c1 * ldx + col0);
+                if (rem > 2) r2 = ls.load(X + (int64_t)c2 * ldx + col0);
                 IO::fma(part, w0, r0);
                 if (rem > 1) IO::fma(part, w1, r1);
                 if (rem > 2) IO::fma(part, w2, r2);
@@ -293,7 +244,198 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] += part[i];
     }
-    if (live) store_row(out + row * ldo + col0, acc);
+}
+
+// A list with more entries than this is left to aggregate_long_rows_kernel when the caller cannot rule
+// such lists out: a hub of a transposed block can hold thousands of entries, the one lane group that
+// walks a list here would outlast the rest of the launch, and hubs sit next to each other.  (Measured on
+// the transposed outer block of a 2.4 M-node graph, 256 floats per row: 432 us with every list walked
+// here, 250 us with lists beyond 256 entries handed over, less with 128.)  Sampled blocks stay below it
+// for fanouts up to 128.
+constexpr int kLongRowEntries = 128;
+
+template <typename T, int VEC, int LPR, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int kGroups = kBlock / LPR;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx, ldo = g.ldo;
+    const int D = g.D;
+
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int gl = (int)threadIdx.x % LPR;  // lane within the group
+    const int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
+    if (row >= n_rows) return;  // uniform per group: the cross-lane reads below stay inside the group
+    const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, D);
+    const int col0 = ls.col0;
+    const bool live = ls.live;
+
+    const int a = indptr[row], b = indptr[row + 1];
+    {
+        // rows left to aggregate_long_rows_kernel -- unless the caller's device-side count rules long
+        // rows out, in which case that kernel ends at once and every row is summed here
+        int skip = g.skip_rows_longer_than;
+        if (g.longest_row != nullptr && *g.longest_row <= skip) skip = 0x7FFFFFFF;
+        if (b - a > skip) return;
+    }
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+
+    if (a == b) {
+        if (live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + col0));
+    } else if constexpr (MODE == FGL_AGG_EDGE) {
+        // attention-style weights: one float per (entry, head); a lane's VEC columns lie in one
+        // head when unit_dim is a multiple of VEC, else each column looks its head up
+        const float* __restrict__ ew = g.edge_w;
+        const int H = g.n_heads, unit = g.unit_dim;
+        const bool one_head = (unit % VEC) == 0;
+        int head[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int c = col0 + i < D ? col0 + i : D - 1;
+            head[i] = c / unit;
+        }
+        for (int base = a; base < b; base += LPR) {
+            const int cnt = (b - base) < LPR ? (b - base) : LPR;
+            int my_col = 0, my_eid = 0;
+            if (gl < cnt) {
+                my_col = indices[base + gl];
+                my_eid = g.edge_index ? g.edge_index[base + gl] : base + gl;
+            }
+            float part[VEC];  // this chunk's sum (see the note on two-level summation in gather_row)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
+            for (int t = 0; t < cnt; ++t) {
+                const int c0 = __shfl(my_col, t, LPR);
+                const int64_t e0 = __shfl(my_eid, t, LPR);
+                if (live) {
+                    const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                    if (one_head) {
+                        IO::fma(part, ew[e0 * H + head[0]], r0);
+                    } else {
+                        float x[VEC];
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) x[i] = 0.0f;
+                        IO::fma(x, 1.0f, r0);
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) part[i] += ew[e0 * H + head[i]] * x[i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += part[i];
+        }
+    } else {
+        gather_row<T, VEC, LPR, MODE>(g, ls, gl, row, a, b, acc);
+    }
+    if (live) ls.store(out + row * ldo + col0, acc);
+}
+
+// The rows that aggregate_kernel skipped.  Every workgroup (512 lanes) looks through its share of the
+// row offsets and sums each long list it finds with all of its lane groups: group k takes the chunks
+// k, k + groups, ... into a partial row, sixteen row loads in flight per lane, and the partials are added up
+// through LDS in group order -- a fixed order, so the result does not depend on scheduling -- by the
+// first group, which writes the row.  Few workgroups find anything, so this kernel is built for the
+// latency of one long list, not for occupancy.  When the caller supplies the longest row's entry count
+// on the device and it rules long lists out, every workgroup leaves after one scalar load.
+constexpr int kLongBlock = 512;
+
+template <typename T, int VEC, int LPR, int MODE>
+__global__ __launch_bounds__(kLongBlock) void aggregate_long_rows_kernel(const AggArgs g)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int kGroups = kLongBlock / LPR;
+    constexpr int kInFlight = 16;
+    const int threshold = g.skip_rows_longer_than;
+    if (g.longest_row != nullptr && *g.longest_row <= threshold) return;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx;
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int gl = (int)threadIdx.x % LPR;
+    const int grp = (int)threadIdx.x / LPR;
+    const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, g.D);
+    const int col0 = ls.col0;
+
+    __shared__ int found[kLongBlock];  // the lanes that met a long row in the current pass
+    __shared__ int n_found;
+    __shared__ float partial[kLongBlock * VEC];
+    // Rows are dealt out one by one, round robin over the workgroups: hubs tend to sit next to each other
+    // (the lowest local ids of a sampled block), and this gives neighbouring hubs to different workgroups.
+    // (The offset reads are strided by that; they are a small part of the launch.)
+    const int64_t per_pass = (int64_t)gridDim.x * kLongBlock;
+    const int64_t passes = (n_rows + per_pass - 1) / per_pass;
+    for (int64_t pass = 0; pass < passes; ++pass) {  // trip count uniform over the workgroup
+        const int64_t r = (pass * kLongBlock + (int)threadIdx.x) * gridDim.x + blockIdx.x;
+        const bool is_long = r < n_rows && indptr[r + 1] - indptr[r] > threshold;
+        if (threadIdx.x == 0) n_found = 0;
+        __syncthreads();
+        if (is_long) found[atomicAdd(&n_found, 1)] = (int)threadIdx.x;
+        __syncthreads();
+        const int n = n_found;
+        for (int i = 0; i < n; ++i) {
+            // the order in which the long rows of a pass are taken does not matter: each is summed on its own
+            const int64_t row = (pass * kLongBlock + found[i]) * gridDim.x + blockIdx.x;
+            const int a = indptr[row], b = indptr[row + 1];
+            float row_factor = 1.0f;
+            if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
+            if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
+            float acc[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+            for (int64_t base = (int64_t)a + (int64_t)grp * LPR; base < b; base += (int64_t)kGroups * LPR) {
+                const int cnt = (b - base) < LPR ? (int)(b - base) : LPR;
+                int my_col = 0;
+                float my_w = 0.0f;
+                if (gl < cnt) {
+                    my_col = indices[base + gl];
+                    my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                }
+                float part[VEC];  // two-level summation, as in gather_row
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) part[k] = 0.0f;
+                for (int t = 0; t < cnt; t += kInFlight) {
+                    int c[kInFlight];
+                    float w[kInFlight];
+                    typename IO::Raw x[kInFlight];
+#pragma unroll
+                    for (int j = 0; j < kInFlight; ++j) {
+                        const int src = t + j < cnt ? t + j : t;  // lanes past the end repeat entry t and are not added
+                        c[j] = __shfl(my_col, src, LPR);
+                        w[j] = __shfl(my_w, src, LPR);
+                    }
+                    if (ls.live) {
+#pragma unroll
+                        for (int j = 0; j < kInFlight; ++j) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+#pragma unroll
+                        for (int j = 0; j < kInFlight; ++j)
+                            if (t + j < cnt) IO::fma(part, w[j], x[j]);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] += part[k];
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) partial[(int)threadIdx.x * VEC + k] = acc[k];
+            __syncthreads();
+            if (grp == 0 && ls.live) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+                for (int q = 0; q < kGroups; ++q)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] += partial[(q * LPR + gl) * VEC + k];
+                ls.store(out + row * g.ldo + col0, acc);
+            }
+            __syncthreads();  // partial[] and found[] are reused
+        }
+    }
 }
 
 // ---- block transpose ---------------------------------------------------------------
@@ -301,7 +443,7 @@ __global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* 
                                                                  const int32_t* __restrict__ indices, int64_t n_rows_max,
                                                                  const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
                                                                  int64_t n_cols_max, int32_t* __restrict__ counts,
-                                                                 int32_t* __restrict__ rank)
+                                                                 int32_t* __restrict__ rank, int32_t* __restrict__ longest)
 {
     const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
     int64_t n_e = n_rows > 0 ? (int64_t)indptr[n_rows] : 0;
@@ -309,8 +451,18 @@ __global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* 
     const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (e >= n_e) return;
     const int32_t c = indices[e];
-    if (c >= 0 && (int64_t)c < n_cols_max) rank[e] = atomicAdd(&counts[c], 1);
-    else rank[e] = -1;
+    int32_t k = -1;
+    if (c >= 0 && (int64_t)c < n_cols_max) k = atomicAdd(&counts[c], 1);
+    rank[e] = k;
+    // only the few entries that land far down a long column report its length
+    if (longest != nullptr && k >= FGL_SHORT_ROW_ENTRIES) atomicMax(longest, k + 1);
+}
+
+__global__ __launch_bounds__(kBlock) void transpose_init_kernel(int32_t* __restrict__ counts, int64_t n, int32_t* __restrict__ longest)
+{
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) counts[i] = 0;
+    if (longest != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *longest = 0;
 }
 
 // sixteen lanes per row: the row's entries are read coalesced and scattered in parallel
@@ -351,16 +503,30 @@ size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int so
 }
 
 // ---- dispatch ----------------------------------------------------------------------
+// Workgroups of the long-row pass: each looks through an equal share of the row offsets.
+constexpr int kLongRowBlocks = 1024;
+
 template <typename T, int VEC, int LPR>
-static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const AggArgs& g)
+static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStream_t stream, AggArgs g)
 {
-#define FGL_LAUNCH_MODE(M) hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, g)
+    const bool second_pass = long_rows_possible && mode != FGL_AGG_EDGE;
+    g.skip_rows_longer_than = second_pass ? kLongRowEntries : 0x7FFFFFFF;
+#define FGL_LAUNCH_MODE(M)                                                                                         \
+    do {                                                                                                           \
+        hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, g);                  \
+        if (second_pass) {                                                                                         \
+            int64_t blocks = ceil_div(g.n_rows_max, kLongBlock);                                                   \
+            if (blocks > kLongRowBlocks) blocks = kLongRowBlocks;                                                  \
+            hipLaunchKernelGGL((aggregate_long_rows_kernel<T, VEC, LPR, M>), dim3((unsigned)blocks, grid.y),       \
+                               dim3(kLongBlock), 0, stream, g);                                                    \
+        }                                                                                                          \
+    } while (0)
     switch (mode) {
         case FGL_AGG_SUM: FGL_LAUNCH_MODE(FGL_AGG_SUM); break;
         case FGL_AGG_MEAN: FGL_LAUNCH_MODE(FGL_AGG_MEAN); break;
         case FGL_AGG_GCN: FGL_LAUNCH_MODE(FGL_AGG_GCN); break;
         case FGL_AGG_COLMEAN: FGL_LAUNCH_MODE(FGL_AGG_COLMEAN); break;
-        default: FGL_LAUNCH_MODE(FGL_AGG_EDGE); break;
+        default: hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, FGL_AGG_EDGE>), grid, dim3(kBlock), 0, stream, g); break;
     }
 #undef FGL_LAUNCH_MODE
     FGL_CHECK_LAUNCH("aggregate_kernel");
@@ -368,7 +534,7 @@ static int launch_agg_mode(int mode, dim3 grid, hipStream_t stream, const AggArg
 }
 
 template <typename T, int VEC>
-static int launch_agg_vec(int mode, hipStream_t stream, const AggArgs& g)
+static int launch_agg_vec(int mode, int64_t longest_row_max, hipStream_t stream, const AggArgs& g)
 {
     const int lanes_needed = (g.D + VEC - 1) / VEC;
     int lpr = 8;
@@ -381,11 +547,13 @@ static int launch_agg_vec(int mode, hipStream_t stream, const AggArgs& g)
         return FGL_ERR_UNSUPPORTED;
     }
     const dim3 grid((unsigned)gx, (unsigned)gy);
+    // a host-side bound that rules long rows out makes this exactly one launch of the plain kernel
+    const bool long_rows_possible = longest_row_max < 0 || longest_row_max > kLongRowEntries;
     switch (lpr) {
-        case 8: return launch_agg_mode<T, VEC, 8>(mode, grid, stream, g);
-        case 16: return launch_agg_mode<T, VEC, 16>(mode, grid, stream, g);
-        case 32: return launch_agg_mode<T, VEC, 32>(mode, grid, stream, g);
-        default: return launch_agg_mode<T, VEC, 64>(mode, grid, stream, g);
+        case 8: return launch_agg_mode<T, VEC, 8>(mode, long_rows_possible, grid, stream, g);
+        case 16: return launch_agg_mode<T, VEC, 16>(mode, long_rows_possible, grid, stream, g);
+        case 32: return launch_agg_mode<T, VEC, 32>(mode, long_rows_possible, grid, stream, g);
+        default: return launch_agg_mode<T, VEC, 64>(mode, long_rows_possible, grid, stream, g);
     }
 }
 
@@ -402,8 +570,9 @@ using namespace fgl;
 FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
                              const int32_t* d_n_rows, const void* d_x, int64_t ldx, int D, int dtype, int mode,
                              int zero_policy, const int32_t* d_row_norm, const int32_t* d_col_norm,
-                             const float* d_edge_w, int n_heads, const int32_t* d_edge_index, void* d_out,
-                             int64_t ldo, void* stream)
+                             const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
+                             int64_t longest_row_max, const int32_t* d_longest_row, void* d_out, int64_t ldo,
+                             void* stream)
 {
     FGL_REQUIRE(n_rows_max >= 0, "aggregate: negative row count");
     FGL_REQUIRE(D >= 1, "aggregate: feature length %d < 1", D);
@@ -421,12 +590,12 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     AggArgs g;
     g.indptr = d_indptr; g.indices = d_indices; g.n_rows_max = n_rows_max; g.d_n_rows = d_n_rows;
     g.x = d_x; g.ldx = ldx; g.D = D; g.zero_policy = zero_policy; g.row_norm = d_row_norm; g.col_norm = d_col_norm;
-    g.out = d_out; g.ldo = ldo; g.edge_w = d_edge_w; g.edge_index = d_edge_index;
+    g.out = d_out; g.ldo = ldo; g.edge_w = d_edge_w; g.edge_index = d_edge_index; g.longest_row = d_longest_row;
     g.n_heads = n_heads > 0 ? n_heads : 1; g.unit_dim = D / g.n_heads;
     hipStream_t s = as_stream(stream);
-    if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, s, g);
-    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, s, g);
-    return launch_agg_vec<uint16_t, 1>(mode, s, g);
+    if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, longest_row_max, s, g);
+    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, longest_row_max, s, g);
+    return launch_agg_vec<uint16_t, 1>(mode, longest_row_max, s, g);
 }
 
 FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)
@@ -438,7 +607,8 @@ FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_
 FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
                                    const int32_t* d_n_rows, int64_t n_cols_max, const int32_t* d_n_cols,
                                    int64_t n_edges_max, int32_t* d_t_indptr, int32_t* d_t_indices,
-                                   int32_t* d_t_edge, int sorted, void* d_ws, size_t ws_bytes, void* stream)
+                                   int32_t* d_t_edge, int32_t* d_t_longest_row, int sorted, void* d_ws, size_t ws_bytes,
+                                   void* stream)
 {
     FGL_REQUIRE(sorted == 0 || (d_n_rows == nullptr && d_n_cols == nullptr),
                 "block_transpose: the sorted variant needs exact sizes (no device-side counts)");
@@ -455,14 +625,20 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
     int32_t* rank = c.take<int32_t>((size_t)n_edges_max);
     char* scan_ws = c.take<char>(scan_workspace_bytes(n_cols_max));
     // the counts live in t_indptr and are scanned in place
-    int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(d_t_indptr), n_cols_max + 1, 0u, s);
-    if (rc != FGL_OK) return rc;
+    {
+        int64_t blocks = ceil_div(n_cols_max + 1, kBlock);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(transpose_init_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, d_t_indptr, n_cols_max + 1,
+                           d_t_longest_row);
+        FGL_CHECK_LAUNCH("transpose_init_kernel");
+    }
     if (n_edges_max > 0 && n_rows_max > 0) {
         hipLaunchKernelGGL(transpose_count_kernel, dim3((unsigned)ceil_div(n_edges_max, kBlock)), dim3(kBlock), 0, s,
-                           d_indptr, d_indices, n_rows_max, d_n_rows, n_edges_max, n_cols_max, d_t_indptr, rank);
+                           d_indptr, d_indices, n_rows_max, d_n_rows, n_edges_max, n_cols_max, d_t_indptr, rank,
+                           d_t_longest_row);
         FGL_CHECK_LAUNCH("transpose_count_kernel");
     }
-    rc = launch_exclusive_sum(d_t_indptr, n_cols_max, d_n_cols, d_t_indptr, nullptr, scan_ws, scan_workspace_bytes(n_cols_max), s);
+    int rc = launch_exclusive_sum(d_t_indptr, n_cols_max, d_n_cols, d_t_indptr, nullptr, scan_ws, scan_workspace_bytes(n_cols_max), s);
     if (rc != FGL_OK) return rc;
     if (sorted) {
         const size_t sort_bytes = sorted_transpose_workspace_bytes(n_cols_max, n_edges_max);

@@ -179,6 +179,15 @@ def exclusive_sum(in_degs):
     return out
 
 
+def _fanout_bound(edge_ptr, neighbor_num):
+    """``neighbor_num`` bounds the entries per row of a sampled block (the reference sizes its shared
+    staging by it, aggregate_acc_kernel.cu:238-247)."""
+    bound = getattr(edge_ptr, "fgl_longest_row", None)
+    if bound is None and int(neighbor_num) > 0:
+        bound = int(neighbor_num)
+    return bound
+
+
 def forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, weight, neighbor_num, dst_nodes):
     """fastgl.forward_gcn (aggregate_acc.cpp:133-160): ``[A_norm (X W)]`` with
     ``A_norm[d, s] = 1/sqrt(dst_norm[d]) * 1/sqrt(src_norm[s])``; a dst row without edges
@@ -190,7 +199,7 @@ def forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, w
     _check_input(weight, "weight", _FEAT)
     tmp = torch.mm(input_feat, weight)
     out = aggregate(edge_ptr, src_edges, tmp, mode="gcn", zero_policy="self", row_norm=dst_norm_degs,
-                    col_norm=src_norm_degs, n_rows=int(dst_nodes))
+                    col_norm=src_norm_degs, n_rows=int(dst_nodes), longest_row=_fanout_bound(edge_ptr, neighbor_num))
     return [out]
 
 
@@ -222,7 +231,8 @@ def forwaed_gin(edge_ptr, src_edges, input_feat, weight, neighbor_num, dst_nodes
     _check_input(src_edges, "src_edges", _I32)
     _check_input(input_feat, "input_feat", _FEAT)
     _check_input(weight, "weight", _FEAT)
-    tmp = aggregate(edge_ptr, src_edges, input_feat, mode="sum", zero_policy="self", n_rows=int(dst_nodes))
+    tmp = aggregate(edge_ptr, src_edges, input_feat, mode="sum", zero_policy="self", n_rows=int(dst_nodes),
+                    longest_row=_fanout_bound(edge_ptr, neighbor_num))
     return [torch.mm(tmp, weight), tmp]
 
 
@@ -276,10 +286,14 @@ _ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
 
 
 def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
-              out=None, edge_weight=None, n_heads=1, edge_index=None):
+              out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None):
     """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
     accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge;
     ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``.
+    ``longest_row``: what is known about the longest row's entry count -- an ``int`` bound (the fanout of a
+    sampled block) or a one-element int32 device tensor (as ``block_transpose`` makes).  Speed only: hub rows
+    of hundreds of entries get a second launch that a bound can save.  When not given it is taken from the
+    ``fgl_longest_row`` attribute that ``block_transpose`` and the sampler attach to their ``indptr`` tensors.
     ``mode="edge"``: ``edge_weight`` float32 [n_entries, n_heads], weight of entry e for column f is
     ``edge_weight[edge_index[e] if edge_index is not None else e, f // (D // n_heads)]``."""
     _check_input(indptr, "indptr", _I32)
@@ -304,7 +318,17 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
             raise RuntimeError("edge_index has fewer entries than indices")
     if mode == "edge" and (edge_weight is None or feat.size(1) % int(n_heads) != 0):
         raise RuntimeError("mode 'edge' needs edge_weight and a head count that divides the row length")
-    dev = _same_device(indptr, indices, feat, row_norm, col_norm, edge_weight, edge_index)
+    if longest_row is None:
+        longest_row = getattr(indptr, "fgl_longest_row", None)
+    longest_host, longest_dev = -1, None
+    if isinstance(longest_row, torch.Tensor):
+        _check_input(longest_row, "longest_row", _I32)
+        if longest_row.numel() != 1:
+            raise RuntimeError("longest_row must hold one int32")
+        longest_dev = longest_row
+    elif longest_row is not None:
+        longest_host = int(longest_row)
+    dev = _same_device(indptr, indices, feat, row_norm, col_norm, edge_weight, edge_index, longest_dev)
     n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
     if n < 0 or n > indptr.numel() - 1:
         raise RuntimeError("n_rows (%d) does not match indptr (%d entries)" % (n, indptr.numel()))
@@ -319,10 +343,13 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
         elif out.shape != (n, D) or out.dtype != feat.dtype or out.stride(1) != 1 or not out.is_cuda:
             raise RuntimeError("out has the wrong shape, dtype or layout")
         if n > 0:
-            L.check(L.lib().fgl_aggregate(L.ptr(indptr), L.ptr(indices), n, None, L.ptr(feat), int(feat.stride(0)), D,
+            # a block without entries has no index array to point at; the kernel then reads none
+            idx_ptr = L.ptr(indices) if indices.numel() else L.ptr(indptr)
+            L.check(L.lib().fgl_aggregate(L.ptr(indptr), idx_ptr, n, None, L.ptr(feat), int(feat.stride(0)), D,
                                           L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
-                                          L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index), L.ptr(out),
-                                          int(out.stride(0)), L.stream_handle()))
+                                          L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index),
+                                          longest_host, L.ptr(longest_dev), L.ptr(out), int(out.stride(0)),
+                                          L.stream_handle()))
     return out
 
 
@@ -341,10 +368,12 @@ def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False, sorted_rows
         t_ptr = torch.empty(n_cols + 1, dtype=torch.int32, device=dev)
         t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
         t_edge = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz] if edge_ids else None
+        longest = torch.empty(1, dtype=torch.int32, device=dev)
         ws = L.workspace(lib.fgl_block_transpose_workspace_bytes(n_cols, nnz, int(sorted_rows)), dev)
         L.check(lib.fgl_block_transpose(L.ptr(indptr), L.ptr(indices), n_rows, None, n_cols, None, nnz, L.ptr(t_ptr),
-                                        L.ptr(t_idx), L.ptr(t_edge), int(sorted_rows), L.ptr(ws), ws.numel(),
+                                        L.ptr(t_idx), L.ptr(t_edge), L.ptr(longest), int(sorted_rows), L.ptr(ws), ws.numel(),
                                         L.stream_handle()))
+    t_ptr.fgl_longest_row = longest  # read by aggregate()
     return (t_ptr, t_idx, t_edge) if edge_ids else (t_ptr, t_idx)
 
 

@@ -189,7 +189,9 @@ class FusedMapSampler:
         blocks = []
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]
-            blocks.insert(0, Block(bptr[h][:n_dst + 1], src_l[h][:n_e], n_src, n_dst,
+            block_ptr = bptr[h][:n_dst + 1]
+            block_ptr.fgl_longest_row = int(self.fanouts[H - 1 - h])  # no row exceeds the fanout (read by ops.aggregate)
+            blocks.insert(0, Block(block_ptr, src_l[h][:n_e], n_src, n_dst,
                                    None if src_g[h] is None else src_g[h][:n_e], sorted_transpose=self.deterministic))
         return uniq[:c[H]], pending["seeds"], blocks
 
@@ -270,6 +272,7 @@ class FusedMapSampler:
                 src_global = src_out.clone() if block_index == len(self.fanouts) - 1 else None
                 src_edges, _dst_edges, seed_nodes_acc = ops.transfer_edge_id(src_out, dst_out, dst_unique, dst_nodes,
                                                                              dst_nodes + edge_nums, max_src_num, edge_nums)
+                block_ptr.fgl_longest_row = int(fanout)
                 blocks.insert(0, Block(block_ptr, src_edges, int(seed_nodes_acc.size(0)), n_dst, src_global,
                                        sorted_transpose=self.deterministic))
                 dst_nodes = int(seed_nodes_acc.size(0))

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 1
+#define FGL_ABI_VERSION 2
 
 enum fgl_error {
     FGL_OK = 0,
@@ -194,12 +194,17 @@ int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_in
  * by ascending row (deterministic output, needs exact sizes: d_n_rows = d_n_cols = NULL, and
  * n_edges_max = the number of entries); sorted = 0 is faster and leaves the order within a
  * column to scheduling.
+ * d_t_longest_row (may be NULL) receives one int32 for fgl_aggregate's d_longest_row: the
+ * entry count of the transposed block's longest row if that exceeds FGL_SHORT_ROW_ENTRIES,
+ * else some value not above it.
  * ------------------------------------------------------------------------------- */
+#define FGL_SHORT_ROW_ENTRIES 32
 size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted);
 int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
                         int64_t n_rows_max, const int32_t* d_n_rows,
                         int64_t n_cols_max, const int32_t* d_n_cols, int64_t n_edges_max,
-                        int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge, int sorted,
+                        int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge,
+                        int32_t* d_t_longest_row, int sorted,
                         void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
@@ -213,12 +218,20 @@ int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
  * arrays as required by `mode` (else NULL).  FGL_AGG_EDGE: d_edge_w float[n_entries, n_heads],
  * n_heads divides D, d_edge_index (optional) maps a position in d_indices to its row of
  * d_edge_w (NULL: the position itself; the d_t_edge of a transposed block otherwise).
+ * (longest_row_max, d_longest_row): what the caller knows about the entry count of the
+ * longest row, in the library's usual (host bound, device value) form -- host: no row holds
+ * more entries than longest_row_max (the fanout for a sampled block; < 0: unknown); device:
+ * NULL, or one int32 as fgl_block_transpose writes it.  Rows of several hundred entries and
+ * more (hubs of a transposed block) are summed by a second launch in which a whole
+ * workgroup shares each such row; a host bound that rules them out saves that launch, a
+ * device value that does lets it end at once.  Speed only: wrong values still give correct sums.
  * ------------------------------------------------------------------------------- */
 int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
                   int64_t n_rows_max, const int32_t* d_n_rows,
                   const void* d_x, int64_t ldx, int D, int dtype, int mode, int zero_policy,
                   const int32_t* d_row_norm, const int32_t* d_col_norm,
                   const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
+                  int64_t longest_row_max, const int32_t* d_longest_row,
                   void* d_out, int64_t ldo, void* stream);
 
 /* ---------------------------------------------------------------------------------

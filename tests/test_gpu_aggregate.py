@@ -40,8 +40,8 @@ def run_modes(cuda, oracle, ptr, idx, deg, X_t, n_src, tol):
     d_ptr, d_idx, d_rn, d_cn = dev_i32(ptr, cuda), dev_i32(idx, cuda), dev_i32(rn, cuda), dev_i32(cn, cuda)
     for mode in ("sum", "mean", "gcn", "colmean"):
         for pol_name, pol in (("self", 0), ("zeros", 1)):
-            got = fastgl.aggregate(d_ptr, d_idx, X_t, mode=mode, zero_policy=pol_name, row_norm=d_rn, col_norm=d_cn)
             want = oracle.aggregate(ptr, idx, X_ref, mode, pol, rn, cn)
+            got = fastgl.aggregate(d_ptr, d_idx, X_t, mode=mode, zero_policy=pol_name, row_norm=d_rn, col_norm=d_cn)
             assert got.dtype == X_t.dtype and tuple(got.shape) == want.shape
             err = rel_err(got.float().cpu().numpy(), want)
             assert err < tol, (mode, pol_name, err)
@@ -56,6 +56,70 @@ def test_aggregate_vs_oracle(cuda, oracle, dtype, D):
     ptr, idx, deg = make_block(rng, n_dst, n_src, 12, hubs=[(3, 64), (4, 65), (100, 300)])
     X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
     run_modes(cuda, oracle, ptr, idx, deg, X, n_src, TOL[dtype])
+
+
+@pytest.mark.parametrize("n_dst", [1, 2, 3, 4, 5, 1023, 4096])
+@pytest.mark.parametrize("max_deg", [1, 2, 3, 9])
+def test_short_row_blocks(cuda, oracle, n_dst, max_deg):
+    """Blocks whose rows hold zero to a few entries (what a transposed block looks like; a block can also
+    have no entries at all), with a few longer lists in between and at the very end."""
+    print("short rows n_dst=%d max_deg=%d" % (n_dst, max_deg), flush=True)
+    rng = np.random.default_rng(n_dst * 16 + max_deg)
+    n_src = 300
+    hubs = [(n_dst - 1, 40)] if n_dst >= 1023 else []
+    if n_dst == 4096:
+        hubs += [(8, 7), (9, 1), (10, 0), (11, 1), (2001, 33), (2002, 31)]
+    ptr, idx, deg = make_block(rng, n_dst, max(n_src, n_dst), max_deg, hubs=hubs)
+    for dtype, D in ((torch.float32, 128), (torch.float32, 50), (torch.bfloat16, 256), (torch.bfloat16, 602)):
+        X = torch.from_numpy(rng.standard_normal((max(n_src, n_dst), D)).astype(np.float32)).to(cuda).to(dtype)
+        run_modes(cuda, oracle, ptr, idx, deg, X, max(n_src, n_dst), TOL[dtype])
+
+
+def test_long_rows_and_what_the_caller_knows_about_them(cuda, oracle):
+    """Rows beyond 128 entries are summed by a second launch (a workgroup per row).  Rows right at that
+    limit, hubs of thousands of entries next to each other and at the very end; and every form of the
+    caller's knowledge about the longest row -- none, a host bound, the device value that block_transpose
+    writes, and deliberately wrong values of both -- gives the same sums (the knowledge is for speed only)."""
+    import fastgl
+    rng = np.random.default_rng(77)
+    n_dst, n_src = 3001, 5000
+    hubs = [(0, 5000), (1, 129), (2, 128), (3, 127), (4, 2500), (5, 131), (1500, 640), (1501, 1), (1502, 0), (3000, 900)]
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 6, hubs=hubs)
+    rn = np.maximum(deg, 1).astype(np.int32)
+    cn = np.maximum(np.bincount(idx, minlength=n_src), 1).astype(np.int32)
+    d_ptr, d_idx, d_rn, d_cn = dev_i32(ptr, cuda), dev_i32(idx, cuda), dev_i32(rn, cuda), dev_i32(cn, cuda)
+    true_max = int(deg.max())
+    knowledge = [None, true_max, 4, 10 ** 9, dev_i32([true_max], cuda), dev_i32([7], cuda), dev_i32([0], cuda)]
+    for dtype, D in ((torch.float32, 128), (torch.float32, 20), (torch.float32, 602), (torch.bfloat16, 256), (torch.bfloat16, 31)):
+        print("long rows D=%d %s" % (D, dtype), flush=True)
+        X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
+        X_ref = X.float().cpu().numpy()
+        for mode in ("sum", "mean", "gcn", "colmean"):
+            want = oracle.aggregate(ptr, idx, X_ref, mode, 1, rn, cn)
+            for know in knowledge:
+                got = fastgl.aggregate(d_ptr, d_idx, X, mode=mode, zero_policy="zeros", row_norm=d_rn, col_norm=d_cn,
+                                       longest_row=know)
+                err = rel_err(got.float().cpu().numpy(), want)
+                assert err < TOL[dtype], (D, dtype, mode, know if not isinstance(know, torch.Tensor) else int(know), err)
+
+
+def test_block_transpose_reports_its_longest_row(cuda):
+    import fastgl
+    rng = np.random.default_rng(5)
+    for n_dst, n_src, hub_count in ((400, 50, 0), (4000, 300, 700), (2000, 2000, 33), (2000, 2000, 32)):
+        deg = rng.integers(0, 3, size=n_dst)
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+        idx = rng.integers(1, n_src, size=ptr[-1]).astype(np.int32)  # column 0 is filled below
+        rows = rng.choice(np.nonzero(deg)[0], size=hub_count, replace=False) if hub_count else []
+        for r in rows:
+            idx[ptr[r]] = 0  # hub_count rows mention column 0 once
+        counts = np.bincount(idx, minlength=n_src)
+        t_ptr, _ = fastgl.block_transpose(dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src)
+        reported = int(t_ptr.fgl_longest_row)
+        longest = int(counts.max())
+        print("transpose n_dst=%d longest=%d reported=%d" % (n_dst, longest, reported), flush=True)
+        # exact beyond 32 entries; below that only "not above 32" is promised
+        assert reported == longest if longest > 32 else reported <= 32
 
 
 def test_aggregate_golden(cuda):
