@@ -393,30 +393,64 @@ __global__ __launch_bounds__(kLongBlock) void aggregate_long_rows_kernel(const A
             for (int64_t base = (int64_t)a + (int64_t)grp * LPR; base < b; base += (int64_t)kGroups * LPR) {
                 const int cnt = (b - base) < LPR ? (int)(b - base) : LPR;
                 int my_col = 0;
-                float my_w = 0.0f;
+                int my_eid = 0;     // FGL_AGG_EDGE: which row of edge_w the entry uses
+                float my_w = 0.0f;  // the other modes: the entry's weight
                 if (gl < cnt) {
                     my_col = indices[base + gl];
-                    my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                    if (MODE == FGL_AGG_EDGE) my_eid = g.edge_index ? g.edge_index[base + gl] : (int)(base + gl);
+                    else my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
                 }
                 float part[VEC];  // two-level summation, as in gather_row
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) part[k] = 0.0f;
                 for (int t = 0; t < cnt; t += kInFlight) {
                     int c[kInFlight];
+                    int eid[kInFlight];
                     float w[kInFlight];
                     typename IO::Raw x[kInFlight];
 #pragma unroll
                     for (int j = 0; j < kInFlight; ++j) {
                         const int src = t + j < cnt ? t + j : t;  // lanes past the end repeat entry t and are not added
                         c[j] = __shfl(my_col, src, LPR);
-                        w[j] = __shfl(my_w, src, LPR);
+                        if (MODE == FGL_AGG_EDGE) eid[j] = __shfl(my_eid, src, LPR);
+                        else w[j] = __shfl(my_w, src, LPR);
                     }
                     if (ls.live) {
 #pragma unroll
                         for (int j = 0; j < kInFlight; ++j) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                        if constexpr (MODE == FGL_AGG_EDGE) {
+                            // one float per (entry, head); this lane's columns lie in one head when the head
+                            // width is a multiple of VEC, else each column looks its head up
+                            const float* __restrict__ ew = g.edge_w;
+                            const int H = g.n_heads, unit = g.unit_dim;
+                            if (unit % VEC == 0) {
+                                const int head = col0 / unit;
 #pragma unroll
-                        for (int j = 0; j < kInFlight; ++j)
-                            if (t + j < cnt) IO::fma(part, w[j], x[j]);
+                                for (int j = 0; j < kInFlight; ++j) w[j] = ew[(int64_t)eid[j] * H + head];
+#pragma unroll
+                                for (int j = 0; j < kInFlight; ++j)
+                                    if (t + j < cnt) IO::fma(part, w[j], x[j]);
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < kInFlight; ++j) {
+                                    if (t + j < cnt) {
+                                        float xf[VEC];
+#pragma unroll
+                                        for (int k = 0; k < VEC; ++k) xf[k] = 0.0f;
+                                        IO::fma(xf, 1.0f, x[j]);
+#pragma unroll
+                                        for (int k = 0; k < VEC; ++k) {
+                                            const int col = col0 + k < g.D ? col0 + k : g.D - 1;
+                                            part[k] += ew[(int64_t)eid[j] * H + col / unit] * xf[k];
+                                        }
+                                    }
+                                }
+                            }
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < kInFlight; ++j)
+                                if (t + j < cnt) IO::fma(part, w[j], x[j]);
+                        }
                     }
                 }
 #pragma unroll
@@ -509,7 +543,7 @@ constexpr int kLongRowBlocks = 1024;
 template <typename T, int VEC, int LPR>
 static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStream_t stream, AggArgs g)
 {
-    const bool second_pass = long_rows_possible && mode != FGL_AGG_EDGE;
+    const bool second_pass = long_rows_possible;
     g.skip_rows_longer_than = second_pass ? kLongRowEntries : 0x7FFFFFFF;
 #define FGL_LAUNCH_MODE(M)                                                                                         \
     do {                                                                                                           \
@@ -526,7 +560,7 @@ static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStre
         case FGL_AGG_MEAN: FGL_LAUNCH_MODE(FGL_AGG_MEAN); break;
         case FGL_AGG_GCN: FGL_LAUNCH_MODE(FGL_AGG_GCN); break;
         case FGL_AGG_COLMEAN: FGL_LAUNCH_MODE(FGL_AGG_COLMEAN); break;
-        default: hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, FGL_AGG_EDGE>), grid, dim3(kBlock), 0, stream, g); break;
+        default: FGL_LAUNCH_MODE(FGL_AGG_EDGE); break;
     }
 #undef FGL_LAUNCH_MODE
     FGL_CHECK_LAUNCH("aggregate_kernel");

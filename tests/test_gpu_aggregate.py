@@ -221,13 +221,17 @@ def test_edge_weighted_forward_backward(cuda, oracle, dtype, H, unit):
     print("aggregate edge mode H=%d unit=%d %s" % (H, unit, dtype), flush=True)
     rng = np.random.default_rng(H * 100 + unit)
     n_dst, n_src, D = 400, 1500, H * unit
-    ptr, idx, deg = make_block(rng, n_dst, n_src, 10, hubs=[(7, 130)])
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 10, hubs=[(7, 130), (8, 400)])
+    idx[rng.choice(idx.size, size=350, replace=False)] = 3  # a hub column: a long row of the transposed block
     X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
     alpha = rng.random((ptr[-1], H)).astype(np.float32)
     d_ptr, d_idx, d_alpha = dev_i32(ptr, cuda), dev_i32(idx, cuda), torch.from_numpy(alpha).to(cuda)
-    (out,) = fastgl.forward_gat(d_ptr, d_alpha, d_idx, X, 10, n_dst, H)
+    (out,) = fastgl.forward_gat(d_ptr, d_alpha, d_idx, X, 10, n_dst, H)  # (a bound that the hubs exceed: speed only)
     want = oracle.aggregate_edge(ptr, idx, X.float().cpu().numpy(), alpha, zero_policy=0)
     assert rel_err(out.float().cpu().numpy(), want) < TOL[dtype]
+    # nothing known about the rows: the two hub rows go through the long-row launch
+    out2 = fastgl.aggregate(d_ptr, d_idx, X, mode="edge", zero_policy="self", edge_weight=d_alpha, n_heads=H)
+    assert rel_err(out2.float().cpu().numpy(), want) < TOL[dtype]
     dO = torch.from_numpy(rng.standard_normal((n_dst, D)).astype(np.float32)).to(cuda).to(dtype)
     (d_x,) = fastgl.backward_gat(d_ptr, d_alpha, d_idx, dO, n_src, H)
     t_ptr, t_idx, t_edge = oracle.transpose_with_edges(ptr, idx, n_src)
