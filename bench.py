@@ -138,7 +138,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-batches", type=int, default=2, help="mini-batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu-batches", type=int, default=16, help="mini-batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
                     help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
     ap.add_argument("--overlap", action="store_true",
@@ -359,12 +359,15 @@ def main():
         t0 = time.time()
         h_ptr, h_src = edge_ptr.cpu().numpy(), edge_src.cpu().numpy()
         log("graph copied to the host in %.1fs; oracle threads: %d" % (time.time() - t0, O.num_threads()))
-        cpu_edges, cpu_t, agg_t, agg_bytes = 0, 0.0, 0.0, 0
+        cpu_edges, cpu_t, cpu_t_seq, agg_t, agg_bytes = 0, 0.0, 0.0, 0.0, 0
         for i in range(args.cpu_batches):
             seeds = train[i * B:(i + 1) * B].cpu().numpy()
             t0 = time.perf_counter()
-            inp, oblocks = O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, i * 64)
+            inp, oblocks = O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, i * 64, parallel_idmap=True)
             cpu_t += time.perf_counter() - t0
+            t0 = time.perf_counter()
+            O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, i * 64, parallel_idmap=False)
+            cpu_t_seq += time.perf_counter() - t0
             cpu_edges += sum(int(b["src_local"].size) for b in oblocks)
             ob = oblocks[0]
             xb = feat.index_select(0, torch.from_numpy(inp).to(dev).long()).float().cpu().numpy()  # rows of the input nodes
@@ -375,8 +378,10 @@ def main():
             agg_bytes += e_ * D * 4 + nd * D * 4 + 4 * e_ + 4 * (nd + 1)
         cpu = {"value": cpu_edges / cpu_t, "unit": "sampled edges/s", "cores": O.num_threads(), "kind": "port",
                "sample": "%d mini-batches of %d seeds of the same workload through the CPU oracle "
-                         "(OpenMP sampling, sequential first-occurrence id-map); aggregation = fp32 OpenMP row gather "
-                         "of the outermost block" % (args.cpu_batches, B),
+                         "(OpenMP sampling + OpenMP id-map: CAS insert, first-occurrence numbering by prefix sum; "
+                         "value_sequential_idmap = the same with a single-threaded hash-map id-map); "
+                         "aggregation = fp32 OpenMP row gather of the outermost block" % (args.cpu_batches, B),
+               "value_sequential_idmap": cpu_edges / cpu_t_seq,
                "aggregation_GBps": agg_bytes / agg_t / 1e9, "host_cpus": os.cpu_count()}
         log("cpu baseline: %.3g edges/s (%d threads), aggregation %.1f GB/s" % (cpu["value"], cpu["cores"], cpu["aggregation_GBps"]))
 

@@ -31,6 +31,7 @@
  *                       enumeration for tiny degrees
  *   orc_table_size      closed form / hand-evaluated values of the reference expression
  *   orc_idmap           numpy/python dict restatement, order-free invariants, hand cases
+ *   orc_idmap_parallel  (timing variant only) identical output to orc_idmap
  *   orc_cal_deg, orc_exclusive_sum   numpy.bincount / numpy.cumsum
  *   orc_aggregate_f64   scipy.sparse products, all-ones / one-hot closed forms
  *   orc_aggregate_edge_f64  scipy.sparse products per head; reduces to orc_aggregate_f64 for unit weights
@@ -229,6 +230,108 @@ ORC_API int64_t orc_idmap(int32_t* src, int32_t* dst, int64_t n_edges,
     }
     free(tab);
     return rc ? rc : n;
+}
+
+/* The same map built by all host threads (timing variant for the CPU baseline; its output is
+ * checked to be identical to orc_idmap's).  Keys are claimed with a compare-and-swap; a key that is new
+ * in this call carries, until it is numbered, the smallest index of an edge that mentions it (kept with
+ * an atomic minimum), so that new ids are numbered in first-occurrence order whatever the thread
+ * interleaving: flag the first mentions, prefix-sum the flags, number, relabel. */
+#define ORC_PENDING 0x80000000u
+
+static inline int64_t orc_claim(orc_slot* tab, int64_t mask, int shift, int32_t id)
+{
+    int64_t p = (int64_t)orc_hash((uint32_t)id, shift);
+    for (;;) {
+        int32_t k = __atomic_load_n(&tab[p].key, __ATOMIC_RELAXED);
+        if (k == -1) {
+            int32_t expected = -1;
+            if (__atomic_compare_exchange_n(&tab[p].key, &expected, id, 0, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) return p;
+            k = expected;
+        }
+        if (k == id) return p;
+        p = (p + 1) & mask;
+    }
+}
+
+static inline void orc_atomic_min_u32(uint32_t* addr, uint32_t v)
+{
+    uint32_t cur = __atomic_load_n(addr, __ATOMIC_RELAXED);
+    while (v < cur && !__atomic_compare_exchange_n(addr, &cur, v, 0, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) {}
+}
+
+ORC_API int64_t orc_idmap_parallel(int32_t* src, int64_t n_edges, const int32_t* dst_unique, int64_t n_dst,
+                                   int32_t* uniq, int64_t uniq_capacity)
+{
+    int64_t want = 2 * (n_dst + n_edges) + 2;
+    int lg = 1;
+    while (((int64_t)1 << lg) < want) ++lg;
+    if (lg > 31 || n_edges >= (int64_t)ORC_PENDING || n_dst > uniq_capacity) return -2;
+    int64_t slots = (int64_t)1 << lg, mask = slots - 1;
+    int shift = 32 - lg;
+    orc_slot* tab = (orc_slot*)malloc(sizeof(orc_slot) * (size_t)slots);
+    int64_t* slot_of = (int64_t*)malloc(sizeof(int64_t) * (size_t)(n_edges > 0 ? n_edges : 1));
+    int nt = 1;
+#ifdef _OPENMP
+    nt = omp_get_max_threads();
+#endif
+    int64_t* part = (int64_t*)calloc((size_t)nt + 1, sizeof(int64_t));
+    int64_t n_new = 0;
+#pragma omp parallel num_threads(nt)
+    {
+        int t = 0;
+#ifdef _OPENMP
+        t = omp_get_thread_num();
+#endif
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < slots; ++i) { tab[i].key = -1; tab[i].val = -1; }  /* val: all ones = larger than any index */
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < n_dst; ++i) {
+            uniq[i] = dst_unique[i];
+            int64_t p = orc_claim(tab, mask, shift, dst_unique[i]);
+            orc_atomic_min_u32((uint32_t*)&tab[p].val, (uint32_t)i);  /* a repeated id keeps its first position */
+        }
+#pragma omp for schedule(static)
+        for (int64_t e = 0; e < n_edges; ++e) {
+            int64_t p = orc_claim(tab, mask, shift, src[e]);
+            slot_of[e] = p;
+            orc_atomic_min_u32((uint32_t*)&tab[p].val, ORC_PENDING | (uint32_t)e);  /* no effect on numbered ids */
+        }
+        /* first mentions of new ids: count per thread (static schedule = contiguous, ordered ranges) */
+        int64_t lo = n_edges * t / nt, hi = n_edges * (t + 1) / nt, cnt = 0;
+        for (int64_t e = lo; e < hi; ++e) cnt += ((uint32_t)tab[slot_of[e]].val == (ORC_PENDING | (uint32_t)e));
+        part[t + 1] = cnt;
+#pragma omp barrier
+#pragma omp single
+        {
+            for (int i = 0; i < nt; ++i) part[i + 1] += part[i];
+            n_new = part[nt];
+        }
+        if (n_dst + n_new <= uniq_capacity) {
+            int64_t next = n_dst + part[t];
+            for (int64_t e = lo; e < hi; ++e) {
+                if ((uint32_t)tab[slot_of[e]].val == (ORC_PENDING | (uint32_t)e)) {
+                    uniq[next] = src[e];
+                    slot_of[e] = -1 - next;  /* the slot's val is replaced after the barrier: others still compare against it */
+                    ++next;
+                }
+            }
+#pragma omp barrier
+            for (int64_t e = lo; e < hi; ++e)
+                if (slot_of[e] < 0) {
+                    int64_t p = orc_claim(tab, mask, shift, src[e]);
+                    tab[p].val = (int32_t)(-1 - slot_of[e]);
+                    slot_of[e] = p;
+                }
+#pragma omp barrier
+            for (int64_t e = lo; e < hi; ++e) src[e] = tab[slot_of[e]].val;
+        }
+    }
+    int64_t rc = (n_dst + n_new <= uniq_capacity) ? n_dst + n_new : -2;
+    free(part);
+    free(slot_of);
+    free(tab);
+    return rc;
 }
 
 /* cal_deg (reference: utilis.cu:43-79): deg[ids[e]] += 1 over a zeroed array. */

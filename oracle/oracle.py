@@ -41,6 +41,8 @@ def lib():
         L.orc_table_size.restype = i64
         L.orc_idmap.argtypes = [vp, vp, i64, vp, i64, vp, i64]
         L.orc_idmap.restype = i64
+        L.orc_idmap_parallel.argtypes = [vp, i64, vp, i64, vp, i64]
+        L.orc_idmap_parallel.restype = i64
         L.orc_cal_deg.argtypes = [vp, i64, vp, i64]
         L.orc_cal_deg.restype = None
         L.orc_exclusive_sum.argtypes = [vp, i64, vp]
@@ -120,6 +122,18 @@ def idmap(src_global, dst_global, dst_unique):
     if n < 0:
         raise RuntimeError("orc_idmap failed: %d" % n)
     return src, dst, uniq[:n].copy()
+
+
+def idmap_parallel(src_global, dst_unique):
+    """``idmap`` on all host threads (the CPU baseline's timing variant): -> (src_local, uniq)."""
+    src = _i32(src_global).copy()
+    du = _i32(dst_unique)
+    cap = du.shape[0] + src.shape[0]
+    uniq = np.empty(max(cap, 1), dtype=np.int32)
+    n = lib().orc_idmap_parallel(_p(src), src.shape[0], _p(du), du.shape[0], _p(uniq), cap)
+    if n < 0:
+        raise RuntimeError("orc_idmap_parallel failed: %d" % n)
+    return src, uniq[:n].copy()
 
 
 def cal_deg(ids, n_nodes: int):
@@ -215,7 +229,7 @@ def rmat_csr(n_nodes: int, n_draws: int, seed: int = 0, indptr_dtype=np.int64):
     return indptr.astype(indptr_dtype), cols
 
 
-def sample_blocks(indptr, indices, seeds, fanouts, rng_seed=0, stream_base=0):
+def sample_blocks(indptr, indices, seeds, fanouts, rng_seed=0, stream_base=0, parallel_idmap=False):
     """Layer loop of the reference's sampler (FusedMapSampler.py:63-109): seeds are expanded
     with fanouts[-1] first; layer k's unique list is layer k+1's seed list.
     -> (input_nodes, blocks) where blocks[i] = dict(indptr, src_local, src_global, n_dst, n_src),
@@ -224,7 +238,10 @@ def sample_blocks(indptr, indices, seeds, fanouts, rng_seed=0, stream_base=0):
     blocks = []
     for li, fanout in enumerate(reversed(list(fanouts))):
         src_g, _dst_g, bptr = sample_node(indptr, indices, cur, fanout, rng_seed, stream_base + li)
-        src_l, _, uniq = idmap(src_g, None, cur)
+        if parallel_idmap:
+            src_l, uniq = idmap_parallel(src_g, cur)
+        else:
+            src_l, _, uniq = idmap(src_g, None, cur)
         blocks.insert(0, dict(indptr=bptr, src_local=src_l, src_global=src_g, n_dst=cur.shape[0], n_src=uniq.shape[0]))
         cur = uniq
     return cur, blocks

@@ -86,3 +86,21 @@ def test_transpose_matches_scipy(oracle):
     m = sp.csr_matrix((np.arange(1, indptr[-1] + 1), indices, indptr), shape=(n_rows, n_cols)).tocsc()
     assert np.array_equal(t_ptr, m.indptr)
     assert np.array_equal(t_idx, m.indices)
+
+
+def test_parallel_idmap_equals_the_sequential_one(oracle):
+    """The multi-threaded variant that the benchmark's CPU baseline times gives exactly the output of the
+    sequential oracle (which the python-dict restatement and the invariants above pin)."""
+    rng = np.random.default_rng(21)
+    for trial in range(25):
+        n_dst = int(rng.integers(0, 400))
+        n_edges = int(rng.integers(0, 30000))
+        pool = int(rng.integers(1, 5000))
+        dst_unique = rng.permutation(50000)[:n_dst].astype(np.int32)
+        if trial % 4 == 0 and n_dst > 5:
+            dst_unique[5] = dst_unique[1]  # a repeated destination keeps its first position
+        src = rng.integers(0, pool, size=n_edges).astype(np.int32)
+        want_src, _, want_uniq = oracle.idmap(src, None, dst_unique)
+        got_src, got_uniq = oracle.idmap_parallel(src, dst_unique)
+        assert np.array_equal(got_src, want_src), trial
+        assert np.array_equal(got_uniq, want_uniq), trial
