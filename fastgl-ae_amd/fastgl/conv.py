@@ -22,6 +22,14 @@ from . import ops
 from .sampler import Block
 
 
+def _transposed(t, edge_ids=False):
+    """The transposed block behind the ``transposed`` argument of the autograd functions: either the tuple
+    itself or a ``Block``, whose transpose is built here, on first use in a backward pass."""
+    if isinstance(t, Block):
+        return t.transposed(edge_ids=True) if edge_ids else t.transposed()
+    return t
+
+
 def _block_csr(graph):
     """(edge_ptr, src_edges, raw_dst_degs) of a block.  A ``Block`` carries its CSR; any other
     object with ``edges()`` goes through cal_deg + exclusive_sum like GraphConv.py:93-98."""
@@ -47,8 +55,15 @@ class MA_Function(torch.autograd.Function):
         d_input = d_input.contiguous()
         if ctx.transposed is None:
             d_x, d_w = ops.backward_gcn(edge_ptr, src_edges, dst_norm_degs, src_norm_degs, d_input, weight, input_feat)
-        else:  # same arithmetic, with the block's cached transpose
-            t_ptr, t_idx = ctx.transposed
+        elif not ctx.needs_input_grad[5]:
+            # the first layer: nobody wants d_x, and d_w = X^T (A^T d_out) = (A X)^T d_out needs no transposed
+            # block -- one more forward-direction gather (rows without edges contribute nothing, as in the
+            # reference's backward kernel, aggregate_acc_kernel.cu:498-500)
+            ax = ops.aggregate(edge_ptr, src_edges, input_feat, mode="gcn", zero_policy="zeros", row_norm=dst_norm_degs,
+                               col_norm=src_norm_degs, n_rows=int(d_input.size(0)))
+            d_x, d_w = None, torch.mm(ax.transpose(0, 1), d_input)
+        else:  # same arithmetic as backward_gcn, with the block's cached transpose
+            t_ptr, t_idx = _transposed(ctx.transposed)
             g = ops.aggregate(t_ptr, t_idx, d_input, mode="gcn", zero_policy="zeros", row_norm=src_norm_degs,
                               col_norm=dst_norm_degs, n_rows=int(input_feat.size(0)))
             d_x = torch.mm(g, weight.transpose(0, 1))
@@ -108,7 +123,7 @@ class GCN(nn.Module):
             edge_ptr, src_edges, raw_dst_norm_degs = _block_csr(graph)
             if isinstance(graph, Block):
                 src_norm_degs = graph.out_degrees().clamp(min=1)
-                transposed = graph.transposed() if torch.is_grad_enabled() else None
+                transposed = graph if torch.is_grad_enabled() else None  # transposed on demand, in backward
             else:
                 src_norm_degs = ops.cal_deg(src_edges, graph.num_src_nodes()).clamp(min=1)
                 transposed = None
@@ -134,10 +149,12 @@ class MA_Function_GIN(torch.autograd.Function):
         if ctx.transposed is None:
             d_x, d_w = ops.backward_gin(edge_ptr, src_edges, d_input, weight, tmp, ctx.src_nodes)
         else:
-            t_ptr, t_idx = ctx.transposed
-            d_tmp = torch.mm(d_input, weight.transpose(0, 1))
             d_w = torch.mm(tmp.transpose(0, 1), d_input)
-            d_x = ops.aggregate(t_ptr, t_idx, d_tmp, mode="sum", zero_policy="zeros", n_rows=int(ctx.src_nodes))
+            d_x = None
+            if ctx.needs_input_grad[3]:  # not for the first layer: its transposed block is never built
+                t_ptr, t_idx = _transposed(ctx.transposed)
+                d_tmp = torch.mm(d_input, weight.transpose(0, 1))
+                d_x = ops.aggregate(t_ptr, t_idx, d_tmp, mode="sum", zero_policy="zeros", n_rows=int(ctx.src_nodes))
         return None, None, None, d_x, d_w, None, None
 
 
@@ -160,7 +177,7 @@ class GIN(nn.Module):
             graph = blocks[i]
             dst_nodes = graph.num_dst_nodes()
             edge_ptr, src_edges, _ = _block_csr(graph)
-            transposed = graph.transposed() if isinstance(graph, Block) and torch.is_grad_enabled() else None
+            transposed = graph if isinstance(graph, Block) and torch.is_grad_enabled() else None
             h = layer(edge_ptr, src_edges, dst_nodes, h, neighbor_list[i], transposed)
         return h
 
@@ -186,8 +203,10 @@ class MA_Function_GAT(torch.autograd.Function):
         d_input = d_input.contiguous()
         if ctx.transposed is None:
             d_x = ops.backward_gat(edge_ptr, edge_data, src_edges, d_input, ctx.src_nodes, ctx.num_heads)[0]
+        elif not ctx.needs_input_grad[5]:
+            d_x = None
         else:
-            t_ptr, t_idx, t_edge = ctx.transposed
+            t_ptr, t_idx, t_edge = _transposed(ctx.transposed, edge_ids=True)
             d_x = ops.aggregate(t_ptr, t_idx, d_input, mode="edge", zero_policy="zeros", n_rows=int(ctx.src_nodes),
                                 edge_weight=edge_data, n_heads=int(ctx.num_heads), edge_index=t_edge)
         # as in the reference (GraphConv.py:227) the attention weights receive no gradient from here
@@ -236,9 +255,7 @@ class GATConv(nn.Module):
         e = self.leaky_relu(el.index_select(0, src_edges.long()) + er.index_select(0, dst_edges.long()))
         edge_data = self.attn_drop(edge_softmax(edge_ptr, dst_edges, e, dst_nodes)).contiguous()
         feat_src = feat_src.reshape(-1, self.out_feats * self.num_heads)
-        transposed = None
-        if isinstance(graph, Block) and torch.is_grad_enabled():
-            transposed = graph.transposed(edge_ids=True)
+        transposed = graph if isinstance(graph, Block) and torch.is_grad_enabled() else None
         return MA_Function_GAT.apply(edge_ptr, edge_data.detach(), src_edges, dst_edges, dst_nodes, feat_src, self.num_heads,
                                      neighbor_num, transposed)
 

@@ -36,15 +36,18 @@ def dense_adj(block, kind):
     return A, passthrough
 
 
+@pytest.mark.parametrize("input_grad", [True, False])
 @pytest.mark.parametrize("model_name", ["gcn", "gin"])
-def test_gcn_gin_forward_backward(cuda, oracle, small_graph, model_name):
+def test_gcn_gin_forward_backward(cuda, oracle, small_graph, model_name, input_grad):
+    """input_grad=False is the training case (raw features): the first layer then computes only the weight
+    gradient, without ever building the outermost block's transpose."""
     import fastgl
-    print("conv %s" % model_name, flush=True)
+    print("conv %s input_grad=%s" % (model_name, input_grad), flush=True)
     input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
     torch.manual_seed(0)
     cls = fastgl.GCN if model_name == "gcn" else fastgl.GIN
     model = cls(20, 16, 5, 2, None, True, 0.0).to(cuda)
-    x = torch.randn(input_nodes.numel(), 20, device=cuda, requires_grad=True)
+    x = torch.randn(input_nodes.numel(), 20, device=cuda, requires_grad=input_grad)
     out = model(blocks, x, neighbor_list=[4, 3])
     gout = torch.randn_like(out)
     out.backward(gout)
@@ -63,7 +66,10 @@ def test_gcn_gin_forward_backward(cuda, oracle, small_graph, model_name):
             cur = (A @ cur + passthrough[:, None] * cur[:n_dst].detach()) @ w
     cur.backward(gout.cpu().double())
     assert torch.allclose(out.detach().cpu().double(), cur.detach(), rtol=1e-4, atol=1e-5)
-    assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
+    if input_grad:
+        assert torch.allclose(x.grad.cpu().double(), h.grad, rtol=1e-4, atol=1e-5)
+    else:
+        assert x.grad is None and blocks[0]._transposed is None and blocks[1]._transposed is not None
     for l, w in zip(model.layers, ws):
         assert torch.allclose(l.weights.grad.cpu().double(), w.grad, rtol=1e-4, atol=1e-5)
 
