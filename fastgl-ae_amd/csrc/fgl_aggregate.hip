@@ -164,6 +164,14 @@ struct LaneSlice {
         full = nvalid >= VEC;
     }
     __device__ __forceinline__ typename IO::Raw load(const T* p) const { return full ? IO::load(p) : IO::load_partial(p, nvalid); }
+    // ALL_FULL: the row length is a multiple of VEC, so every live lane moves a whole vector -- the caller
+    // has tested that once for the launch, and the loads carry no per-lane branch
+    template <bool ALL_FULL>
+    __device__ __forceinline__ typename IO::Raw load_row(const T* p) const
+    {
+        if (ALL_FULL) return IO::load(p);
+        return load(p);
+    }
     __device__ __forceinline__ void store(T* p, const float (&a)[VEC]) const
     {
         if (full) IO::store(p, a);
@@ -172,7 +180,7 @@ struct LaneSlice {
 };
 
 // acc += sum over the entries [a, b) of one row (a < b), all modes except FGL_AGG_EDGE.
-template <typename T, int VEC, int LPR, int MODE>
+template <typename T, int VEC, int LPR, int MODE, bool ALL_FULL>
 __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, VEC>& ls, int gl, int64_t row, int a, int b,
                                            float (&acc)[VEC])
 {
@@ -211,10 +219,10 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
             const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
             const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
             if (live) {
-                const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
-                const typename IO::Raw r1 = ls.load(X + (int64_t)c1 * ldx + col0);
-                const typename IO::Raw r2 = ls.load(X + (int64_t)c2 * ldx + col0);
-                const typename IO::Raw r3 = ls.load(X + (int64_t)c3 * ldx + col0);
+                const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
+                const typename IO::Raw r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
+                const typename IO::Raw r3 = ls.template load_row<ALL_FULL>(X + (int64_t)c3 * ldx + col0);
                 IO::fma(part, w0, r0);
                 IO::fma(part, w1, r1);
                 IO::fma(part, w2, r2);
@@ -232,10 +240,10 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
             const float w1 = __shfl(my_w, rem > 1 ? t + 1 : t, LPR);
             const float w2 = __shfl(my_w, rem > 2 ? t + 2 : t, LPR);
             if (live) {
-                const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
                 typename IO::Raw r1 = r0, r2 = r0;
-                if (rem > 1) r1 = ls.load(X + (int64_t)c1 * ldx + col0);
-                if (rem > 2) r2 = ls.load(X + (int64_t)c2 * ldx + col0);
+                if (rem > 1) r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
+                if (rem > 2) r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
                 IO::fma(part, w0, r0);
                 if (rem > 1) IO::fma(part, w1, r1);
                 if (rem > 2) IO::fma(part, w2, r2);
@@ -331,7 +339,9 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
             for (int i = 0; i < VEC; ++i) acc[i] += part[i];
         }
     } else {
-        gather_row<T, VEC, LPR, MODE>(g, ls, gl, row, a, b, acc);
+        // one test per launch instead of one per load: is every live lane's vector whole?
+        if (D % VEC == 0) gather_row<T, VEC, LPR, MODE, true>(g, ls, gl, row, a, b, acc);
+        else gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc);
     }
     if (live) ls.store(out + row * ldo + col0, acc);
 }
@@ -363,6 +373,7 @@ __global__ __launch_bounds__(kLongBlock) void aggregate_long_rows_kernel(const A
     const int grp = (int)threadIdx.x / LPR;
     const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, g.D);
     const int col0 = ls.col0;
+    const bool all_full = g.D % VEC == 0;  // every live lane moves a whole vector: loads without a per-lane branch
 
     __shared__ int found[kLongBlock];  // the lanes that met a long row in the current pass
     __shared__ int n_found;
@@ -416,8 +427,13 @@ __global__ __launch_bounds__(kLongBlock) void aggregate_long_rows_kernel(const A
                         else w[j] = __shfl(my_w, src, LPR);
                     }
                     if (ls.live) {
+                        if (all_full) {
 #pragma unroll
-                        for (int j = 0; j < kInFlight; ++j) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                            for (int j = 0; j < kInFlight; ++j) x[j] = IO::load(X + (int64_t)c[j] * ldx + col0);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < kInFlight; ++j) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                        }
                         if constexpr (MODE == FGL_AGG_EDGE) {
                             // one float per (entry, head); this lane's columns lie in one head when the head
                             // width is a multiple of VEC, else each column looks its head up
@@ -538,7 +554,8 @@ size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int so
 
 // ---- dispatch ----------------------------------------------------------------------
 // Workgroups of the long-row pass: each looks through an equal share of the row offsets.
-constexpr int kLongRowBlocks = 1024;
+constexpr int kLongRowBlocks = 1021;  // a prime: rows are dealt round robin, and ids that agree in their low bits are
+                                       // alike in synthetic (R-MAT) graphs -- a power of two would hand all hubs to a few workgroups
 
 template <typename T, int VEC, int LPR>
 static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStream_t stream, AggArgs g)
