@@ -74,6 +74,38 @@ def test_mid_shape_properties(cuda):
     assert abs(a - b) <= 1e-6 * scale
 
 
+def test_whole_graph_as_one_block(cuda):
+    """Aggregation over the whole 2.4M-node graph as one block: tens of thousands of rows beyond 128 entries
+    (the longest holds ~85 K), so the long-row launch carries most of the work.  Closed forms (exact in fp32:
+    sums of ones stay below 2^24), the same result whatever the caller says about the longest row, and
+    linearity."""
+    import fastgl
+    print("full-size: whole graph as one block", flush=True)
+    n = 2_400_000
+    ptr, src = fastgl.graph.rmat_csr(n, 36_000_000, seed=0, device=cuda)
+    ptr32 = ptr.int()
+    deg = ptr32[1:] - ptr32[:-1]
+    assert int((deg > 128).sum()) > 10_000 and int(deg.max()) > 50_000
+    ones = torch.ones(n, 8, device=cuda)
+    total = fastgl.aggregate(ptr32, src, ones, mode="sum", zero_policy="zeros")
+    assert torch.equal(total, deg.float()[:, None].expand(-1, 8))
+    mean = fastgl.aggregate(ptr32, src, ones, mode="mean", zero_policy="zeros")
+    # n terms of fl(1/n), summed in fp32 per chunk and then across chunks: not exactly 1 for the longest rows
+    mean_err = float((mean - (deg > 0).float()[:, None]).abs().max())
+    print("mean of ones: max deviation %.2e" % mean_err, flush=True)
+    assert mean_err <= 2e-5
+    gen = torch.Generator(device=cuda).manual_seed(3)
+    x = torch.randn(n, 32, device=cuda, generator=gen)
+    y = torch.randn(n, 32, device=cuda, generator=gen)
+    two = fastgl.aggregate(ptr32, src, x, mode="mean", zero_policy="zeros")                  # nothing known: two launches
+    one = fastgl.aggregate(ptr32, src, x, mode="mean", zero_policy="zeros", longest_row=1)    # (wrong) bound: one launch
+    scale = float(two.abs().max())
+    assert float((two - one).abs().max()) <= 1e-5 * scale
+    both = fastgl.aggregate(ptr32, src, 2.0 * x - y, mode="mean", zero_policy="zeros")
+    ay = fastgl.aggregate(ptr32, src, y, mode="mean", zero_policy="zeros")
+    assert float((both - (2.0 * two - ay)).abs().max()) <= 1e-5 * max(scale, float(ay.abs().max())) * 3
+
+
 def test_offsets_beyond_int32(cuda):
     """A CSR with more than 2^31 edges (int64 row offsets): rows at the far end are sampled from the
     right place.  Closed form: indices[e] = e mod 2^20, so a full-neighbourhood row is a known range."""
