@@ -493,7 +493,8 @@ __global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* 
                                                                  const int32_t* __restrict__ indices, int64_t n_rows_max,
                                                                  const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
                                                                  int64_t n_cols_max, int32_t* __restrict__ counts,
-                                                                 int32_t* __restrict__ rank, int32_t* __restrict__ longest)
+                                                                 int split, int32_t* __restrict__ rank,
+                                                                 int32_t* __restrict__ longest)
 {
     const int64_t n_rows = actual_count(n_rows_max, d_n_rows);
     int64_t n_e = n_rows > 0 ? (int64_t)indptr[n_rows] : 0;
@@ -502,10 +503,29 @@ __global__ __launch_bounds__(kBlock) void transpose_count_kernel(const int32_t* 
     if (e >= n_e) return;
     const int32_t c = indices[e];
     int32_t k = -1;
-    if (c >= 0 && (int64_t)c < n_cols_max) k = atomicAdd(&counts[c], 1);
+    // split > 1: every column has `split` counters and entry e uses number e % split -- a returning atomic
+    // on one address completes before the next one starts, and a hub column is mentioned thousands of times
+    if (c >= 0 && (int64_t)c < n_cols_max) k = atomicAdd(&counts[(int64_t)c * split + (int)(e & (split - 1))], 1);
     rank[e] = k;
-    // only the few entries that land far down a long column report its length
-    if (longest != nullptr && k >= FGL_SHORT_ROW_ENTRIES) atomicMax(longest, k + 1);
+    // only the few entries that land far down a long column report its length (split counters: see
+    // transpose_offsets_kernel)
+    if (split == 1 && longest != nullptr && k >= FGL_SHORT_ROW_ENTRIES) atomicMax(longest, k + 1);
+}
+
+// split counters, after their scan: the column offsets are every split-th prefix
+__global__ __launch_bounds__(kBlock) void transpose_offsets_kernel(const int32_t* __restrict__ scanned, int split,
+                                                                   int64_t n_cols_max, int32_t* __restrict__ t_indptr,
+                                                                   int32_t* __restrict__ longest)
+{
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c <= n_cols_max; c += stride) {
+        const int32_t begin = scanned[c * split];
+        t_indptr[c] = begin;
+        if (longest != nullptr && c < n_cols_max) {
+            const int32_t len = scanned[(c + 1) * split] - begin;
+            if (len > FGL_SHORT_ROW_ENTRIES) atomicMax(longest, len);
+        }
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void transpose_init_kernel(int32_t* __restrict__ counts, int64_t n, int32_t* __restrict__ longest)
@@ -519,7 +539,7 @@ __global__ __launch_bounds__(kBlock) void transpose_init_kernel(int32_t* __restr
 __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* __restrict__ indptr,
                                                                 const int32_t* __restrict__ indices, int64_t n_rows_max,
                                                                 const int32_t* __restrict__ d_n_rows, int64_t n_edges_max,
-                                                                const int32_t* __restrict__ t_indptr,
+                                                                const int32_t* __restrict__ t_indptr, int split,
                                                                 const int32_t* __restrict__ rank,
                                                                 int32_t* __restrict__ t_indices,
                                                                 int32_t* __restrict__ t_edge)
@@ -535,7 +555,8 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
         for (int64_t e = a + lane; e < b; e += kLanes) {
             const int32_t k = rank[e];
             if (k >= 0) {
-                const int64_t pos = (int64_t)t_indptr[indices[e]] + k;
+                // t_indptr: the column offsets, or (split > 1) the scanned split counters
+                const int64_t pos = (int64_t)t_indptr[(int64_t)indices[e] * split + (int)(e & (split - 1))] + k;
                 t_indices[pos] = (int32_t)r;
                 if (t_edge) t_edge[pos] = (int32_t)e;
             }
@@ -543,11 +564,19 @@ __global__ __launch_bounds__(kBlock) void transpose_fill_kernel(const int32_t* _
     }
 }
 
+// Blocks of at least this many entries count with kCountSplit counters per column (the extra scan and the
+// offsets pass cost a few microseconds; below, the contention they remove costs less than that).
+constexpr int64_t kCountSplitMinEdges = (int64_t)1 << 20;
+constexpr int kCountSplit = 8;
+static inline int count_split(int64_t n_edges_max, int sorted) { return (!sorted && n_edges_max >= kCountSplitMinEdges) ? kCountSplit : 1; }
+
 size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)
 {
+    const int split = count_split(n_edges_max, sorted);
     Carver c(nullptr);
     c.take<int32_t>((size_t)n_edges_max);
-    c.take<char>(scan_workspace_bytes(n_cols_max));
+    c.take<char>(scan_workspace_bytes(n_cols_max * split));
+    if (split > 1) c.take<int32_t>((size_t)(n_cols_max * split + 1));
     if (sorted) c.take<char>(sorted_transpose_workspace_bytes(n_cols_max, n_edges_max));
     return c.used();
 }
@@ -672,25 +701,37 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
         return FGL_ERR_WORKSPACE;
     }
     hipStream_t s = as_stream(stream);
+    const int split = count_split(n_edges_max, sorted);
     Carver c(d_ws);
     int32_t* rank = c.take<int32_t>((size_t)n_edges_max);
-    char* scan_ws = c.take<char>(scan_workspace_bytes(n_cols_max));
-    // the counts live in t_indptr and are scanned in place
+    char* scan_ws = c.take<char>(scan_workspace_bytes(n_cols_max * split));
+    // the counts live in t_indptr and are scanned in place; with split counters they live in the workspace
+    int32_t* counts = split > 1 ? c.take<int32_t>((size_t)(n_cols_max * split + 1)) : d_t_indptr;
+    const int64_t n_counts = n_cols_max * split;
     {
-        int64_t blocks = ceil_div(n_cols_max + 1, kBlock);
+        int64_t blocks = ceil_div(n_counts + 1, kBlock);
         if (blocks > 4096) blocks = 4096;
-        hipLaunchKernelGGL(transpose_init_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, d_t_indptr, n_cols_max + 1,
+        hipLaunchKernelGGL(transpose_init_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, counts, n_counts + 1,
                            d_t_longest_row);
         FGL_CHECK_LAUNCH("transpose_init_kernel");
     }
     if (n_edges_max > 0 && n_rows_max > 0) {
         hipLaunchKernelGGL(transpose_count_kernel, dim3((unsigned)ceil_div(n_edges_max, kBlock)), dim3(kBlock), 0, s,
-                           d_indptr, d_indices, n_rows_max, d_n_rows, n_edges_max, n_cols_max, d_t_indptr, rank,
+                           d_indptr, d_indices, n_rows_max, d_n_rows, n_edges_max, n_cols_max, counts, split, rank,
                            d_t_longest_row);
         FGL_CHECK_LAUNCH("transpose_count_kernel");
     }
-    int rc = launch_exclusive_sum(d_t_indptr, n_cols_max, d_n_cols, d_t_indptr, nullptr, scan_ws, scan_workspace_bytes(n_cols_max), s);
+    // (split counters are scanned up to the host bound: counters of columns past a device-side count are zero)
+    int rc = launch_exclusive_sum(counts, n_counts, split > 1 ? nullptr : d_n_cols, counts, nullptr, scan_ws,
+                                  scan_workspace_bytes(n_counts), s);
     if (rc != FGL_OK) return rc;
+    if (split > 1) {
+        int64_t blocks = ceil_div(n_cols_max + 1, kBlock);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(transpose_offsets_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, counts, split, n_cols_max,
+                           d_t_indptr, d_t_longest_row);
+        FGL_CHECK_LAUNCH("transpose_offsets_kernel");
+    }
     if (sorted) {
         const size_t sort_bytes = sorted_transpose_workspace_bytes(n_cols_max, n_edges_max);
         char* sort_ws = c.take<char>(sort_bytes);
@@ -701,7 +742,7 @@ FGL_EXPORT int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_ind
         int64_t fill_blocks = ceil_div(n_rows_max, kBlock / 16);
         if (fill_blocks > 16384) fill_blocks = 16384;
         hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)fill_blocks), dim3(kBlock), 0, s, d_indptr,
-                           d_indices, n_rows_max, d_n_rows, n_edges_max, d_t_indptr, rank, d_t_indices, d_t_edge);
+                           d_indices, n_rows_max, d_n_rows, n_edges_max, counts, split, rank, d_t_indices, d_t_edge);
         FGL_CHECK_LAUNCH("transpose_fill_kernel");
     }
     return FGL_OK;

@@ -122,6 +122,30 @@ def test_block_transpose_reports_its_longest_row(cuda):
         assert reported == longest if longest > 32 else reported <= 32
 
 
+def test_transpose_of_a_large_block(cuda):
+    """Blocks of 2M+ entries count with several counters per column: offsets, the permutation of the entries
+    and the reported longest row against device-side recomputation (the transposition is the same multiset of
+    (row, column) pairs, t_edge names the entry each one came from)."""
+    import fastgl
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    n_dst, n_src, k = 150_000, 400_000, 15
+    ptr = (torch.arange(n_dst + 1, device=cuda, dtype=torch.int32) * k)
+    idx = torch.randint(0, n_src, (n_dst * k,), generator=gen, device=cuda, dtype=torch.int32)
+    hub = torch.randint(0, n_dst * k, (60_000,), generator=gen, device=cuda)
+    idx[hub[:40_000]] = 7          # one column mentioned ~40 K times
+    idx[hub[40_000:]] = 123_456    # another ~20 K times
+    print("large transpose: %d entries" % idx.numel(), flush=True)
+    t_ptr, t_idx, t_edge = fastgl.block_transpose(ptr, idx, n_dst, n_src, edge_ids=True)
+    counts = torch.bincount(idx.long(), minlength=n_src)
+    want_ptr = torch.cat([torch.zeros(1, dtype=torch.long, device=cuda), counts.cumsum(0)])
+    assert torch.equal(t_ptr.long(), want_ptr)
+    assert int(t_ptr.fgl_longest_row) == int(counts.max())
+    assert torch.equal(torch.sort(t_edge.long()).values, torch.arange(idx.numel(), device=cuda))   # a permutation
+    col_of_t = torch.repeat_interleave(torch.arange(n_src, device=cuda), counts)
+    assert torch.equal(idx.long()[t_edge.long()], col_of_t)                    # every entry sits in its column's list
+    assert torch.equal((t_edge // k).int(), t_idx)                             # and names the row it came from
+
+
 def test_aggregate_golden(cuda):
     import fastgl
     print("aggregate golden", flush=True)
