@@ -101,3 +101,13 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libfastgl_hip.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         L.lib()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message that says so (no GPU is touched)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "--gpus 1" in (r.stdout + r.stderr)
