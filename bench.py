@@ -138,6 +138,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--sampler", choices=["graph", "eager"], default="eager",
+                    help="eager: launch the fused sampler's kernels (default); graph: replay them from a captured HIP graph "
+                         "(pays off when the GPU would wait for the host: small batches, one batch at a time)")
     ap.add_argument("--cpu-batches", type=int, default=16, help="mini-batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
                     help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
@@ -188,7 +191,29 @@ def main():
     torch.cuda.synchronize()
     log("features %s x %d %s and %d training seeds in %.1fs" % (N, D, w["dtype"], w["train"], time.time() - t0))
 
-    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
+    def make_sampler(graph_slots):
+        return fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order,
+                                      graph_slots=graph_slots).set_graph(edge_ptr, edge_src)
+
+    # --sampler graph: the fused path's launch sequence is replayed from a captured HIP graph.  The mode is
+    # checked here against the eager path on a few mini-batches and abandoned, loudly, if capture fails or
+    # any result differs.
+    sampler_mode = args.sampler
+    sampler = make_sampler(2 if sampler_mode == "graph" else 0)
+    if sampler_mode == "graph":
+        try:
+            check = make_sampler(0)
+            for i in range(4):
+                got, want = sampler.sample_blocks(None, train[i * B:i * B + B]), check.sample_blocks(None, train[i * B:i * B + B])
+                same = torch.equal(got[0], want[0]) and all(torch.equal(a.edge_ptr, b.edge_ptr) and torch.equal(a.src_local, b.src_local)
+                                                            for a, b in zip(got[2], want[2]))
+                if not same:
+                    raise RuntimeError("graph replay differs from the eager path on mini-batch %d" % i)
+            del check, got, want
+        except Exception as exc:  # noqa: BLE001 -- any failure of the optional mode falls back to the eager path
+            log("graph-replay sampler abandoned: %s" % exc)
+            sampler_mode = "eager (graph replay abandoned: %s)" % exc
+            sampler = make_sampler(0)
     L = len(w["fanouts"])
     # hidden activations / upstream gradients of the inner layers: synthetic; sized from a probe
     # batch with head-room (the worst-case bound would be tens of GB for deep fanouts) and grown on demand
@@ -228,7 +253,7 @@ def main():
         e4.record()
         if rec is not None:
             rec.append(((sum(b.num_edges() for b in blocks), b0.num_edges(), b0.num_dst_nodes()), (e0, e1, e2, e3, e4)))
-            keep.append(b0)
+            keep.append(b0.clone() if sampler.graph_slots else b0)  # (a graph-replay slot is overwritten two batches on)
             del keep[:-4]  # a few outermost blocks are kept for the kernel-time replay below
         return blocks
 
@@ -284,6 +309,27 @@ def main():
     rb.record()
     torch.cuda.synchronize()
     t_kernel0 = ra.elapsed_time(rb)
+
+    # ---- the same sampling without graph replay (context for `value`) -----------------------
+    value_eager = None
+    if sampler.graph_slots:
+        eager = make_sampler(0)
+        for i in range(3):
+            eager.sample_blocks(None, train[i * B:i * B + B])
+        ea, eb = ev(), ev()
+        eager_edges, eager_ms = 0, 0.0
+        for i in range(args.steps):
+            seeds = train[((args.warmup + i) % n_batches) * B:((args.warmup + i) % n_batches) * B + B]
+            torch.cuda.synchronize()
+            ea.record()
+            _, _, blocks = eager.sample_blocks(None, seeds)
+            eb.record()
+            torch.cuda.synchronize()
+            eager_ms += ea.elapsed_time(eb)
+            eager_edges += sum(b.num_edges() for b in blocks)
+        value_eager = eager_edges / (eager_ms * 1e-3)
+        del eager, blocks
+        log("sampling without graph replay: %.3g edges/s" % value_eager)
 
     # ---- context: what a plain streaming copy reaches on this box ---------------------------
     cp_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -400,7 +446,7 @@ def main():
         "dtype": w["dtype"],
         "data": "synthetic",
         "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
-                   "sampled_edges_per_step": tot_edges / K, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
+                   "sampled_edges_per_step": tot_edges / K, "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
                    "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
                            "feature table); block transpose + bwd gather on the inner blocks; no dense layers"},
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
@@ -408,6 +454,7 @@ def main():
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,
                         "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
         "random_read_Gps": random_read_gps,
+        "value_eager_launch": value_eager,
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,

@@ -114,7 +114,8 @@ FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const in
 
 FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                                  const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                                 const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base, int idmap_flags, void* d_table,
+                                 const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base,
+                                 const uint32_t* d_stream_offset, int idmap_flags, void* d_table,
                                  int64_t table_slots,
                                  int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
                                  int32_t* const* src_local, int32_t* const* src_global, int32_t* d_counts, void* d_ws,
@@ -154,7 +155,8 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         char* ws = static_cast<char*>(d_ws);
         const size_t ws_sample = sample_workspace_bytes(p.cap_dst[h], fanouts[h]);
         rc = launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], rng_seed,
-                           stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s);
+                           stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s,
+                           d_stream_offset);
         if (rc != FGL_OK) return rc;
         // the node count this hop may grow to: what the next hop's buffers (or the unique list) hold;
         // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped

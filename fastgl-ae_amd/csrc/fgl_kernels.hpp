@@ -22,7 +22,7 @@ int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indice
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                   int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws, size_t ws_bytes,
-                  hipStream_t stream);
+                  hipStream_t stream, const uint32_t* d_stream_add = nullptr);
 
 // id-map (fgl_idmap.hip)
 size_t idmap_map_src_workspace_bytes(int64_t n_edges_max);

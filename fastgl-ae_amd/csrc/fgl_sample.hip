@@ -69,6 +69,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                                                           const int32_t* __restrict__ deg_arr,
                                                           const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
                                                           uint32_t seed_hi, uint32_t stream_id,
+                                                          const uint32_t* __restrict__ d_stream_add,
                                                           int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
                                                           int32_t* __restrict__ block_ptr)
 {
@@ -80,6 +81,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
     __shared__ int s_seed[TS];
 
     const int tid = (int)threadIdx.x;
+    if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -164,6 +166,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
                                                               const int32_t* __restrict__ deg_arr,
                                                               const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
                                                               uint32_t seed_hi, uint32_t stream_id,
+                                                              const uint32_t* __restrict__ d_stream_add,
                                                               int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
                                                               int32_t* __restrict__ block_ptr)
 {
@@ -173,6 +176,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
     int32_t* s_dst = s_stage + TS * fanout;
 
     const int tid = (int)threadIdx.x;
+    if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -247,7 +251,7 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
                             const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                             uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                             int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws,
-                            hipStream_t stream)
+                            hipStream_t stream, const uint32_t* d_stream_add)
 {
     const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, TS);
     Carver c(d_ws);
@@ -270,7 +274,7 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
 #define FGL_LAUNCH_REG(F)                                                                                           \
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr)
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr)
         if (fanout <= 8) FGL_LAUNCH_REG(8);
         else if (fanout <= 16) FGL_LAUNCH_REG(16);
         else FGL_LAUNCH_REG(32);
@@ -282,7 +286,7 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
 #define FGL_LAUNCH_EDGES(U)                                                                                        \
     hipLaunchKernelGGL((sample_edges_kernel<TS, U>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,          \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_src_out, d_dst_out, d_block_ptr)
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr)
     FGL_LAUNCH_EDGES(16);
 #undef FGL_LAUNCH_EDGES
     FGL_CHECK_LAUNCH("sample_edges_kernel");
@@ -293,7 +297,7 @@ int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indice
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                   int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws, size_t ws_bytes,
-                  hipStream_t stream)
+                  hipStream_t stream, const uint32_t* d_stream_add)
 {
     FGL_REQUIRE(n_seeds_max >= 0 && n_nodes >= 0, "sample_node: negative size");
     FGL_REQUIRE(fanout >= 1 && fanout <= FGL_MAX_FANOUT, "sample_node: fanout %d outside [1, %d]", fanout, FGL_MAX_FANOUT);
@@ -308,10 +312,10 @@ int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indice
     if (tile_seeds_for(fanout) == 256)
         return launch_sample_ts<256>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
                                      rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status,
-                                     d_ws, stream);
+                                     d_ws, stream, d_stream_add);
     return launch_sample_ts<64>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
                                 rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws,
-                                stream);
+                                stream, d_stream_add);
 }
 
 }  // namespace fgl

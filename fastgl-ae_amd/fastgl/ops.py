@@ -408,7 +408,7 @@ class BlocksPlan:
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
-                        keep_global=(0,), table_slots=None, id_order="first"):
+                        keep_global=(0,), table_slots=None, id_order="first", stream_offset=None):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
@@ -419,11 +419,15 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     ``table_slots`` (a power of two, default the plan's worst case) uses only that much of the
     hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL).
     ``id_order``: ``"first"`` numbers new ids by first occurrence (deterministic), ``"arrival"`` as
-    their inserts land (faster; any run is a valid map, equal to every other after sorting the new ids)."""
+    their inserts land (faster; any run is a valid map, equal to every other after sorting the new ids).
+    ``stream_offset``: one-element int32 device tensor added to ``stream_base`` when the kernels run (for
+    callers that capture this call in a graph and advance the random stream between replays)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
     _check_input(indices, "indices", _I32)
     _check_input(seeds, "seeds", _I32)
-    dev = _same_device(edge_ptr, indices, seeds)
+    if stream_offset is not None:
+        _check_input(stream_offset, "stream_offset", _I32)
+    dev = _same_device(edge_ptr, indices, seeds, stream_offset)
     if int(seeds.numel()) != plan.n_seeds:
         raise RuntimeError("plan was made for %d seeds, got %d" % (plan.n_seeds, seeds.numel()))
     H = plan.n_hops
@@ -440,7 +444,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         arr = lambda ts: (C.c_void_p * H)(*[L.ptr(t) for t in ts])
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,
-                                      int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF,
+                                      int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF, L.ptr(stream_offset),
                                       {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order], L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
                                       L.stream_handle()))

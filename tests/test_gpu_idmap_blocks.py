@@ -218,6 +218,37 @@ def test_pipelined_iterator_equals_batch_by_batch(cuda, oracle, small_graph):
     assert list(sampler.iter_batches([])) == []
 
 
+@pytest.mark.parametrize("pipelined", [False, True])
+def test_graph_replay_equals_the_oracle_batch_after_batch(cuda, oracle, small_graph, pipelined):
+    """graph_slots=2: the launch sequence is captured per slot and replayed.  Twelve mini-batches -- so every
+    graph is replayed several times, with eager work of this test and of the consumer between the replays --
+    each checked against the oracle (seeds and random stream change from replay to replay); one batch outgrows
+    the buffers sized by experience and is redone eagerly, after which the plan changes and the graphs are
+    captured anew."""
+    import fastgl
+    print("sample_blocks graph replay pipelined=%s" % pipelined, flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    rng = np.random.default_rng(5)
+    batches = [rng.permutation(indptr.size - 1)[:700].astype(np.int32) for _ in range(12)]
+    batches[7] = np.argsort(-np.diff(indptr))[:700].astype(np.int32)
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=33, graph_slots=2).set_graph(ptr, idx)
+    feat = torch.randn(indptr.size - 1, 32, device=cuda)
+    seeds_dev = [dev_i32(b, cuda) for b in batches]
+    results = sampler.iter_batches(iter(seeds_dev)) if pipelined else (sampler.sample_blocks(None, s) for s in seeds_dev)
+    captures = set()
+    for i, got in enumerate(results):
+        check_blocks(oracle, indptr, indices, batches[i], [15, 10, 5], got, 33, i * 64)
+        b0 = got[2][0]
+        out = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")  # eager work between replays
+        want = oracle.aggregate(b0.edge_ptr.cpu().numpy(), b0.src_global.cpu().numpy(), feat.cpu().numpy(), "mean", 1)
+        assert np.abs(out.cpu().numpy() - want).max() < 1e-5
+        if sampler._graphs is not None:
+            captures.add(sampler._graphs[0])
+    assert sampler._graphs is not None and all(slot is not None for slot in sampler._graphs[2])  # graphs were used
+    assert len(captures) >= 2  # ... and captured anew after the plan changed
+
+
 @pytest.mark.parametrize("fused", [True, False])
 def test_sample_blocks_degenerate_batches(cuda, oracle, small_graph, fused):
     """no seeds, repeated seeds, seeds without neighbours: same answers as the oracle"""
