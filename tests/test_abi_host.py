@@ -94,6 +94,15 @@ def test_sampler_front_end_without_gpu():
     src, dst = b.edges()
     assert dst.tolist() == [0, 0, 2, 2, 2] and b.num_src_nodes() == 5 and b.num_dst_nodes() == 3 and b.num_edges() == 5
     assert b.in_degrees().tolist() == [2, 0, 3]
+    b.edge_ptr.fgl_longest_row = 3
+    c = b.clone()
+    assert c.edge_ptr.data_ptr() != b.edge_ptr.data_ptr() and c.edge_ptr.fgl_longest_row == 3
+    assert c.edges()[0].tolist() == src.tolist() and c.num_src_nodes() == 5
+    for bad in (1, -2):
+        with pytest.raises(ValueError):
+            fastgl.FusedMapSampler([5], graph_slots=bad)
+    with pytest.raises(ValueError):
+        fastgl.FusedMapSampler([5], id_order="arrival", deterministic=True)
 
 
 def test_missing_library_fails_loudly(monkeypatch):
