@@ -39,6 +39,7 @@ WORKLOADS = {
     "c5deep": dict(nodes=269_000_000, draws=3_320_000_000, dim=128, dtype="bf16", hidden=256, batch=8192, train=1_200_000,
                    fanouts=[10, 10, 10, 10, 10]),
     "c4": None,  # aggregation-only microbench, see run_c4
+    "ceiling": None,  # random row gathers from a 48 GB table, see run_ceiling
 }
 DESCRIPTIONS = {
     "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
@@ -49,6 +50,8 @@ DESCRIPTIONS = {
           "batch 8192, fanout [15,10,5]",
     "c5deep": "R-MAT 269M nodes / ~4.0B edges (int64 indptr, int32 indices), feat 269Mx128 bf16 resident, hidden 256, "
               "batch 8192, fanout [10,10,10,10,10]",
+    "ceiling": "random row gathers from a 48 GB table: 2^20 output rows x 1 or 13 uniformly random source rows of 256 B - 2 KB, "
+               "fp32 and bf16, through the aggregation kernel and through torch.index_select; streaming copy and add",
     "c4": "aggregation microbench: 8192 dst x exactly 25 src out of 200K rows (int32 CSR), D in {64,128,256,602}, fp32 and bf16, "
           "sum and mean, forward and backward",
 }
@@ -128,6 +131,81 @@ def run_c4(args):
 
 
 
+def run_ceiling(args):
+    """What the box gives to row gathers, whatever kernel asks: the aggregation kernel as a pure random
+    gather (one random source row per output row: no reuse, no arithmetic to speak of) and with 13 random
+    rows per output row (the outer block's shape), for several row sizes, from a table far larger than the
+    caches; next to it torch's own row gather, a streaming add and a device-to-device copy."""
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def timed(fn, reps=20):
+        for _ in range(3):
+            fn()
+        a, b = ev(), ev()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e-3  # seconds
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    table_bytes = 48 << 30
+    n_out = 1 << 20
+    rows_out = []
+    for dtype, esz in ((torch.float32, 4), (torch.bfloat16, 2)):
+        for row_bytes in (256, 512, 1024, 2048):
+            D = row_bytes // esz
+            n_rows = table_bytes // row_bytes
+            table = torch.empty((n_rows, D), dtype=dtype, device=dev)
+            table.view(torch.int32).fill_(0)  # the values do not matter (zeros in either format), the addresses do
+            out = torch.empty((n_out, D), dtype=dtype, device=dev)
+            case = {"dtype": "f32" if esz == 4 else "bf16", "row_bytes": row_bytes, "table_GB": table_bytes / 2 ** 30}
+            for k in (1, 13):
+                ptr = torch.arange(n_out + 1, dtype=torch.int32, device=dev) * k
+                idx = torch.randint(0, n_rows, (n_out * k,), generator=gen, device=dev, dtype=torch.int32)
+                t = timed(lambda: fastgl.aggregate(ptr, idx, table, mode="sum", zero_policy="zeros", out=out, longest_row=k))
+                moved = n_out * k * row_bytes + n_out * row_bytes + 4 * n_out * k + 4 * (n_out + 1)
+                case["k%d_GBps" % k] = moved / t / 1e9
+                case["k%d_Grows_per_s" % k] = n_out * k / t / 1e9
+                if k == 1:
+                    idx64 = idx.long()
+                    t = timed(lambda: torch.index_select(table, 0, idx64, out=out))
+                    case["torch_index_select_GBps"] = 2 * n_out * row_bytes / t / 1e9
+            rows_out.append(case)
+            log("%-4s rows of %4d B: 1 source per row %5.0f GB/s (%.1f G rows/s; torch.index_select %5.0f GB/s) | "
+                "13 sources per row %5.0f GB/s (%.1f G rows/s)"
+                % (case["dtype"], row_bytes, case["k1_GBps"], case["k1_Grows_per_s"], case["torch_index_select_GBps"],
+                   case["k13_GBps"], case["k13_Grows_per_s"]))
+            del table, out
+            torch.cuda.empty_cache()
+    a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    b = torch.empty_like(a)
+    t = timed(lambda: b.copy_(a))
+    copy_gbps = 2 * (1 << 30) / t / 1e9
+    x = a.view(torch.float32)
+    y = b.view(torch.float32)
+    t = timed(lambda: torch.add(x, 1.0, out=y))
+    add_gbps = 2 * (1 << 30) / t / 1e9
+    log("streaming: device copy %.0f GB/s, elementwise add %.0f GB/s (read + write)" % (copy_gbps, add_gbps))
+    head = [r for r in rows_out if r["dtype"] == "f32" and r["row_bytes"] == 512][0]
+    print(json.dumps({
+        "metric": "random row gather GB/s (context for the aggregation roofline), 1 MI355X", "value": head["k13_GBps"],
+        "unit": "GB/s", "n_gpus": 1, "steps": 20, "warmup": 3, "ms_per_step": None, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": DESCRIPTIONS["ceiling"]},
+        "roofline": {"bound": "hbm", "achieved": head["k13_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": head["k13_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "aggregate_kernel<float,4,32,SUM> (13 random 512-byte rows per output row, 48 GB table)"},
+        "cpu_baseline": None, "stream_copy_GBps": copy_gbps, "stream_add_GBps": add_gbps, "cases": rows_out}), flush=True)
+
+
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
@@ -168,6 +246,8 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "c4":
         return run_c4(args)
+    if args.workload == "ceiling":
+        return run_ceiling(args)
     w = WORKLOADS[args.workload]
     N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
     fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16
