@@ -12,6 +12,10 @@
 // time before the first FMA so that each lane keeps several 16-byte loads in flight.
 // Accumulation is fp32, in CSR order, in registers: no shared-memory read-modify-write
 // and no redundant staging of the id list as in the reference kernel.
+//
+// Rows of more than 128 entries (hubs of a transposed block; none in a sampled block) are left to a
+// second launch, aggregate_long_rows_kernel, in which a whole 512-lane workgroup sums one row; the
+// caller's knowledge of the longest row decides whether that launch is enqueued at all.
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
