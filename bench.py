@@ -26,9 +26,9 @@ for _p in (ROOT, os.path.join(ROOT, "fastgl-ae_amd")):
 
 HBM_PEAK_GBPS = 8000.0
 # HBM traffic per launch of the dominant kernel on workload c3, from two `rocprofv3 --pmc` runs
-# (FETCH_SIZE 369838 KiB x 1.898 + WRITE_SIZE 55671 KiB x 1.000, the factors being what the same
+# (FETCH_SIZE 370030 KiB x 1.898 + WRITE_SIZE 55671 KiB x 1.000, the factors being what the same
 # counters read for this kernel run as a plain copy of known size: 1064960 KiB read -> 561177)
-TRAFFIC_BYTES_C3 = 369838 * 1024 * 1.898 + 55671 * 1024 * 1.0
+TRAFFIC_BYTES_C3 = 370030 * 1024 * 1.898 + 55671 * 1024 * 1.0
 
 WORKLOADS = {
     # name: nodes, R-MAT draws, feature dim, feature dtype, hidden, batch, training seeds, fanouts (reference order)
