@@ -302,3 +302,28 @@ def test_hash_collisions_and_probe_limit(cuda, oracle):
         else:
             with pytest.raises(RuntimeError, match="hash table full"):
                 run_transfer(cuda, src, dst, dst_unique, 1 << 31)
+
+
+def test_random_configurations_against_the_oracle(cuda, oracle):
+    """Thirty seeded random configurations -- graph size and density, 1 to 4 hops, fanouts 1 to 192 (all three
+    sampling kernels), int32 and int64 offsets, repeated seeds, plain launches and graph replay, three
+    mini-batches each -- every output bit for bit against the oracle."""
+    import fastgl
+    rng = np.random.default_rng(123)
+    for case in range(30):
+        n = int(rng.integers(50, 20000))
+        indptr, indices = oracle.rmat_csr(n, int(n * rng.uniform(0.5, 20)), seed=int(rng.integers(0, 1000)),
+                                          indptr_dtype=np.int64 if case % 2 else np.int32)
+        hops = int(rng.integers(1, 5))
+        fanouts = [int(rng.integers(1, 41)) if rng.random() < 0.8 else int(rng.integers(41, 193)) for _ in range(hops)]
+        n_seeds = int(rng.integers(1, min(n, 2000) + 1))
+        seeds = rng.permutation(n)[:n_seeds].astype(np.int32)
+        if case % 7 == 0:
+            seeds[rng.integers(0, n_seeds)] = seeds[0]
+        rng_seed = int(rng.integers(0, 2 ** 40))
+        print("random configuration %d: n=%d fanouts=%s seeds=%d" % (case, n, fanouts, n_seeds), flush=True)
+        ptr, idx = load_graph(cuda, indptr, indices)
+        sampler = fastgl.FusedMapSampler(fanouts, rng_seed=rng_seed, graph_slots=2 if case % 3 == 0 else 0).set_graph(ptr, idx)
+        for batch in range(3):
+            got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+            check_blocks(oracle, indptr, indices, seeds, fanouts, got, rng_seed, batch * 64)
