@@ -306,3 +306,30 @@ def test_deterministic_sampler_gives_bitwise_reproducible_gradients(cuda, oracle
         t_ptr, t_idx = b.transposed()
         grads.append(fastgl.aggregate(t_ptr, t_idx, g, mode="sum", zero_policy="zeros"))
     assert torch.equal(grads[0], grads[1])
+
+
+def test_random_blocks_all_modes_against_the_oracle(cuda, oracle):
+    """Thirty seeded random blocks -- row counts, row lengths from empty to beyond the long-row limit, feature
+    lengths from 1 to 700 (whole and partial vectors, one to several column slices), both element types, all
+    modes and both policies for empty rows, forward and over the transposed block."""
+    import fastgl
+    rng = np.random.default_rng(2024)
+    for case in range(30):
+        n_dst = int(rng.integers(1, 3000))
+        n_src = max(n_dst, int(rng.integers(1, 6000)))
+        max_deg = int(rng.choice([0, 1, 2, 5, 20, 70]))
+        hubs = [(int(rng.integers(0, n_dst)), int(rng.integers(100, 900))) for _ in range(int(rng.integers(0, 4)))]
+        ptr, idx, deg = make_block(rng, n_dst, n_src, max_deg, hubs=hubs)
+        D = int(rng.choice([1, 2, 5, 8, 31, 32, 64, 100, 128, 200, 256, 602, 700]))
+        dtype = torch.float32 if case % 3 else torch.bfloat16
+        print("random block %d: %d x %d, %d entries, D=%d %s" % (case, n_dst, n_src, idx.size, D, dtype), flush=True)
+        X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
+        run_modes(cuda, oracle, ptr, idx, deg, X, n_src, TOL[dtype])
+        # the transposed block: every source row sums the destination rows it feeds
+        G = torch.from_numpy(rng.standard_normal((n_dst, D)).astype(np.float32)).to(cuda).to(dtype)
+        t_ptr, t_idx = fastgl.block_transpose(dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src)
+        got = fastgl.aggregate(t_ptr, t_idx, G, mode="sum", zero_policy="zeros")
+        want_ptr, want_idx = oracle.transpose(ptr, idx, n_src)
+        want = oracle.aggregate(want_ptr, want_idx, G.float().cpu().numpy(), "sum", 1)
+        assert np.array_equal(t_ptr.cpu().numpy(), want_ptr)
+        assert rel_err(got.float().cpu().numpy(), want) < TOL[dtype], case
