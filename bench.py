@@ -219,7 +219,7 @@ def main():
     ap.add_argument("--sampler", choices=["graph", "eager"], default="eager",
                     help="eager: launch the fused sampler's kernels (default); graph: replay them from a captured HIP graph "
                          "(pays off when the GPU would wait for the host: small batches, one batch at a time)")
-    ap.add_argument("--cpu-batches", type=int, default=16, help="mini-batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu-batches", type=int, default=128, help="mini-batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
                     help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
     ap.add_argument("--overlap", action="store_true",
