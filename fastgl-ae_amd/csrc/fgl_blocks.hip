@@ -11,10 +11,15 @@
 
 namespace fgl {
 
-__global__ void blocks_init_counts_kernel(int32_t* __restrict__ counts, int n_entries, int32_t n_seeds)
+// Start of a mini-batch in one launch: every table slot back to empty (all ones), node count of
+// hop 0 = the seed count, the other counts and the status word zero.
+__global__ __launch_bounds__(kBlock) void blocks_reset_kernel(uint32_t* __restrict__ table_words, int64_t n_words,
+                                                              int32_t* __restrict__ counts, int n_entries, int32_t n_seeds)
 {
-    const int i = (int)threadIdx.x;
-    if (i < n_entries) counts[i] = (i == 0) ? n_seeds : 0;
+    const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (first < n_entries) counts[first] = (first == 0) ? n_seeds : 0;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = first; i < n_words; i += stride) table_words[i] = 0xFFFFFFFFu;
 }
 
 struct BlocksPlan {
@@ -140,10 +145,16 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     hipStream_t s = as_stream(stream);
     const int n_counts = 2 * n_hops + 2;
     uint32_t* d_status = reinterpret_cast<uint32_t*>(d_counts + 2 * n_hops + 1);
-    hipLaunchKernelGGL(blocks_init_counts_kernel, dim3(1), dim3(128), 0, s, d_counts, n_counts, (int32_t)n_seeds);
-    FGL_CHECK_LAUNCH("blocks_init_counts_kernel");
-    rc = launch_idmap_reset(d_table, table_slots, s);
-    if (rc != FGL_OK) return rc;
+    FGL_REQUIRE(table_slots >= 64 && table_slots <= ((int64_t)1 << 31) && (table_slots & (table_slots - 1)) == 0,
+                "sample_blocks: slot count %lld is not a power of two in [64, 2^31]", (long long)table_slots);
+    {
+        const int64_t n_words = table_slots * 2;
+        int64_t blocks = ceil_div(n_words, (int64_t)kBlock * 4);
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(blocks_reset_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, static_cast<uint32_t*>(d_table),
+                           n_words, d_counts, n_counts, (int32_t)n_seeds);
+        FGL_CHECK_LAUNCH("blocks_reset_kernel");
+    }
     rc = launch_idmap_insert_dst(d_table, table_slots, d_seeds, n_seeds, nullptr, d_uniq, d_status, s);
     if (rc != FGL_OK) return rc;
 

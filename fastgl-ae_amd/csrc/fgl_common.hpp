@@ -105,6 +105,27 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* smem, int* total
     return wave_prefix + incl - v;
 }
 
+// Sum of v[0..count) over a workgroup of NT threads, the same value in every thread.  `smem` needs
+// NT/64 ints.  Contains two barriers: every thread of the block must call it.  Lets the workgroup
+// of tile t derive its own exclusive prefix from the per-tile sums of an earlier launch, which
+// saves the single-workgroup scan launch in between while the tile count is small.
+template <int NT>
+__device__ __forceinline__ int block_sum_before(const int32_t* __restrict__ v, int64_t count, int* smem)
+{
+    constexpr int NW = NT / kWave;
+    int s = 0;
+    for (int64_t i = threadIdx.x; i < count; i += NT) s += v[i];
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) s += __shfl_xor(s, d, kWave);
+    if (lane_id() == 0) smem[threadIdx.x / kWave] = s;
+    __syncthreads();
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += smem[w];
+    __syncthreads();
+    return sum;
+}
+
 // Philox4x32-10 (Salmon et al., SC'11): the counter-based generator the reference uses
 // through cuRAND (sample.cu:69-70).
 __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,

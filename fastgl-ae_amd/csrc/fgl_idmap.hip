@@ -9,7 +9,7 @@
 // new ids are numbered in first-occurrence order -- deterministic, and the order DGL's
 // to_block gives -- instead of the reference's race on one global counter (id_map.cu:317-320).
 //
-// map_src = four launches:
+// map_src = four launches (three for small inputs):
 //   1. insert     per edge: probe (one 8-byte load per slot), install {key, pending first-edge index}
 //                 with one 64-bit CAS if new, else atomicMin the first-edge index; remember the slot.
 //                 An id that was numbered before this call is relabelled on the spot from the val
@@ -19,7 +19,9 @@
 //                 of 2048 edges, and per-tile counts
 //   3. prefix     single workgroup over the tile counts; publishes the new node total
 //                 (the edge-parallel launches are grid-stride loops over the actual count,
-//                 so a bound much larger than the batch costs nothing)
+//                 so a bound much larger than the batch costs nothing).  Skipped while the bound
+//                 is at most 1024 tiles (2 M edges): the number pass then scans the tile counts
+//                 itself in every workgroup, and its first workgroup publishes the total
 //   4. number     per edge, coalesced: a first edge computes its id's local id from the three
 //                 counts, stores it in the slot, appends the id to the unique list and relabels
 //                 itself without reading the table; a later mention reads the slot and, if the
@@ -185,6 +187,18 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
     }
 }
 
+// n_total = n_base + (number of new ids), clamped to the capacity of the unique list.
+__device__ __forceinline__ void publish_node_total(int64_t n_base, int n_new, int64_t capacity,
+                                                   int32_t* __restrict__ d_n_total_out, uint32_t* __restrict__ d_status)
+{
+    int64_t total = n_base + (int64_t)n_new;
+    if (total > capacity) {
+        if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
+        total = capacity;
+    }
+    if (d_n_total_out) *d_n_total_out = (int32_t)total;
+}
+
 // One workgroup: exclusive scan of the per-tile counts of new ids, then
 // n_total = n_base + (number of new ids), clamped to the capacity of the unique list.
 __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_t* __restrict__ tile_sums,
@@ -205,38 +219,62 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
         if (i < n_tiles) tile_prefix[i] = carry + ex;
         carry += total;
     }
-    if (threadIdx.x == 0) {
-        const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-        int64_t total = n_base + (int64_t)carry;
-        if (total > capacity) {
-            if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
-            total = capacity;
-        }
-        if (d_n_total_out) *d_n_total_out = (int32_t)total;
-    }
+    if (threadIdx.x == 0)
+        publish_node_total(d_n_base ? (int64_t)(*d_n_base) : n_base_h, carry, capacity, d_n_total_out, d_status);
 }
 
-// Local id of the new node whose first mention is edge e (an edge that the mark pass flagged).
-__device__ __forceinline__ int64_t local_of_first_edge(int64_t n_base, int64_t e, uint32_t byte_flags,
-                                                       const uint16_t* __restrict__ before8,
-                                                       const int32_t* __restrict__ tile_prefix)
-{
-    return n_base + tile_prefix[e / kTile] + before8[e >> 3] + __popc(byte_flags & ((1u << (e & 7)) - 1u));
-}
+// Up to this many tiles the number pass scans the tile counts itself (every workgroup, into LDS) and
+// its first workgroup publishes the node total: one launch less per call where launches, not
+// edges, set the time.  Above it the single-workgroup prefix launch prepares the array once.
+constexpr int kSelfTilesPerLane = 4;
+constexpr int kSelfPrefixTiles = kBlock * kSelfTilesPerLane;
 
 // Lane per edge.  `src` and `out` may be the same array: an entry is read and written by one lane only.
 // (Edges whose id was numbered before this call were relabelled by the insert pass.)
+// SELF: no prefix launch ran; tile_prefix is unused, the tile counts are scanned here.
+template <bool SELF>
 __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const int32_t* src, int64_t e_max,
                                                               const int32_t* __restrict__ d_e, int64_t n_base_h,
                                                               const int32_t* __restrict__ d_n_base,
                                                               const uint32_t* __restrict__ slot_of,
                                                               const uint8_t* __restrict__ flags8,
                                                               const uint16_t* __restrict__ before8,
+                                                              const int32_t* __restrict__ tile_sums,
                                                               const int32_t* __restrict__ tile_prefix,
-                                                              int32_t* __restrict__ uniq, int64_t capacity, int32_t* out)
+                                                              int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
+                                                              int32_t* __restrict__ d_n_total_out,
+                                                              uint32_t* __restrict__ d_status)
 {
+    __shared__ int s_prefix[SELF ? kSelfPrefixTiles : 1];
+    __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
+    if constexpr (SELF) {
+        const int n_tiles = (int)tiles_of(n_e);  // <= kSelfPrefixTiles: the launcher checks the bound
+        int v[kSelfTilesPerLane];
+        int s = 0;
+#pragma unroll
+        for (int j = 0; j < kSelfTilesPerLane; ++j) {
+            const int i = (int)threadIdx.x * kSelfTilesPerLane + j;
+            v[j] = i < n_tiles ? tile_sums[i] : 0;
+            s += v[j];
+        }
+        int total;
+        int run = block_exclusive_scan<kBlock>(s, smem, &total);
+#pragma unroll
+        for (int j = 0; j < kSelfTilesPerLane; ++j) {
+            s_prefix[(int)threadIdx.x * kSelfTilesPerLane + j] = run;
+            run += v[j];
+        }
+        __syncthreads();
+        if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status);
+    }
+    // local id of the new node whose first mention is edge x (an edge that the mark pass flagged)
+    auto local_of_first_edge = [&](int64_t x, uint32_t byte_flags) -> int64_t {
+        const int64_t tile = x / kTile;
+        const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
+        return n_base + before_tile + before8[x >> 3] + __popc(byte_flags & ((1u << (x & 7)) - 1u));
+    };
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
@@ -245,7 +283,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
         if (p != kEmpty) {
             const uint32_t f = flags8[e >> 3];
             if ((f >> (e & 7)) & 1u) {
-                local = local_of_first_edge(n_base, e, f, before8, tile_prefix);
+                local = local_of_first_edge(e, f);
                 if (local < capacity) {
                     t.words[2 * (size_t)p + 1] = (uint32_t)local;
                     uniq[local] = src[e];
@@ -258,10 +296,10 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                     // the first edge's lane has not stored the local id yet (or this lane's cache has
                     // not seen it): derive it the way that lane does
                     const int64_t ef = (int64_t)(v & ~kPending);
-                    if (ef < n_e) local = local_of_first_edge(n_base, ef, flags8[ef >> 3], before8, tile_prefix);
+                    if (ef < n_e) local = local_of_first_edge(ef, flags8[ef >> 3]);
                 }
             }
-            if (local >= capacity) local = -1;  // the unique list is full (reported by the prefix pass)
+            if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
         }
         out[e] = (int32_t)local;
     }
@@ -449,11 +487,18 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
                        slot_of, flags8, before8, sums);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
-    hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max, d_n_edges,
-                       n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
-    FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
-    hipLaunchKernelGGL(idmap_number_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
-                       d_n_edges, n_base, d_n_base, slot_of, flags8, before8, prefix, d_uniq, uniq_capacity, d_src_out);
+    if (tiles <= kSelfPrefixTiles) {
+        hipLaunchKernelGGL(idmap_number_kernel<true>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
+                           d_n_edges, n_base, d_n_base, slot_of, flags8, before8, sums, nullptr, d_uniq, uniq_capacity,
+                           d_src_out, d_n_total_out, d_status);
+    } else {
+        hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max,
+                           d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
+        FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
+        hipLaunchKernelGGL(idmap_number_kernel<false>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
+                           d_n_edges, n_base, d_n_base, slot_of, flags8, before8, sums, prefix, d_uniq, uniq_capacity,
+                           d_src_out, nullptr, nullptr);
+    }
     FGL_CHECK_LAUNCH("idmap_number_kernel");
     return FGL_OK;
 }

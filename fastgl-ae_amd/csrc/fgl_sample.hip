@@ -61,17 +61,46 @@ __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restric
     }
 }
 
+// Output offset of a tile of seeds.  With a prefix array (from the single-workgroup scan launch) it
+// is one load.  Without one (tile_prefix == nullptr: the launcher skips that launch while the tile
+// count is small) the workgroup sums the earlier tiles' sums itself, and the workgroup of the last
+// tile also publishes the edge total: block_ptr[n] and *n_edges_out.
+template <int TS>
+__device__ __forceinline__ int tile_base(const int32_t* __restrict__ tile_sums, const int32_t* __restrict__ tile_prefix,
+                                         int64_t tile, int64_t n_tiles, int64_t n, int tile_total, int* smem,
+                                         int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+{
+    if (tile_prefix) return tile_prefix[tile];
+    const int base = block_sum_before<TS>(tile_sums, tile, smem);
+    if (tile == n_tiles - 1 && threadIdx.x == 0) {
+        block_ptr[n] = base + tile_total;
+        if (n_edges_out) *n_edges_out = base + tile_total;
+    }
+    return base;
+}
+
+// The launch for zero seeds still has to publish the (empty) totals when no scan launch does.
+__device__ __forceinline__ void publish_empty(const int32_t* __restrict__ tile_prefix, int64_t n_tiles,
+                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+{
+    if (tile_prefix == nullptr && n_tiles == 0 && blockIdx.x == 0 && threadIdx.x == 0) {
+        block_ptr[0] = 0;
+        if (n_edges_out) *n_edges_out = 0;
+    }
+}
+
 template <int TS, int U>
 __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restrict__ indices,
                                                           const int32_t* __restrict__ seeds, int64_t n_max,
                                                           const int32_t* __restrict__ d_n, int fanout,
                                                           const int64_t* __restrict__ row_start,
                                                           const int32_t* __restrict__ deg_arr,
+                                                          const int32_t* __restrict__ tile_sums,
                                                           const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
                                                           uint32_t seed_hi, uint32_t stream_id,
                                                           const uint32_t* __restrict__ d_stream_add,
                                                           int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
-                                                          int32_t* __restrict__ block_ptr)
+                                                          int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
 {
     extern __shared__ uint32_t s_sel[];  // [fanout][TS] picked positions
     __shared__ int s_scan[TS / kWave + 1];
@@ -84,6 +113,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
     if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
+    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i = tile * TS + tid;
         int deg = 0, seed = 0;
@@ -96,7 +126,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_prefix[tile];
+        const int base = tile_base<TS>(tile_sums, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
         s_off[tid] = ex;
         if (tid == 0) s_off[TS] = total;
         s_row[tid] = row;
@@ -164,11 +194,12 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
                                                               const int32_t* __restrict__ d_n, int fanout,
                                                               const int64_t* __restrict__ row_start,
                                                               const int32_t* __restrict__ deg_arr,
+                                                              const int32_t* __restrict__ tile_sums,
                                                               const int32_t* __restrict__ tile_prefix, uint32_t seed_lo,
                                                               uint32_t seed_hi, uint32_t stream_id,
                                                               const uint32_t* __restrict__ d_stream_add,
                                                               int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
-                                                              int32_t* __restrict__ block_ptr)
+                                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
 {
     extern __shared__ int32_t s_stage[];  // [TS*fanout] sampled ids (+ [TS*fanout] seed ids when dst_out is wanted)
     __shared__ int s_scan[TS / kWave + 1];
@@ -179,6 +210,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
     if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
+    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i = tile * TS + tid;
         int deg = 0, seed = 0;
@@ -191,7 +223,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_prefix[tile];
+        const int base = tile_base<TS>(tile_sums, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
         if (i < n) block_ptr[i] = base + ex;
 
         uint32_t sel[F];
@@ -234,6 +266,10 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
 
 static inline int tile_seeds_for(int fanout) { return fanout <= 48 ? 256 : 64; }
 
+// Up to this many tiles of seeds the edges kernel derives its tile offsets itself (at most 16 KiB of
+// tile sums per workgroup, read from L2); above it a scan launch prepares them.
+constexpr int64_t kSelfPrefixTiles = 4096;
+
 size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
 {
     const int ts = tile_seeds_for(fanout);
@@ -264,17 +300,23 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     hipLaunchKernelGGL(sample_degree_kernel<TS>, dim3(grid), dim3(TS), 0, stream, d_indptr, indptr_is64,
                        n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
     FGL_CHECK_LAUNCH("sample_degree_kernel");
-    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds, TS,
-                                stream);
-    if (rc != FGL_OK) return rc;
+    // few tiles: each workgroup of the edges kernel sums the earlier tile sums itself (the last one
+    // publishes the totals), which saves the scan launch in between
+    if (tiles > kSelfPrefixTiles) {
+        int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds,
+                                    TS, stream);
+        if (rc != FGL_OK) return rc;
+    } else {
+        prefix = nullptr;
+    }
     // the register variant stages the tile's output (and, if wanted, the seed ids) in LDS: it is used
     // while that fits comfortably in the 64 KiB a workgroup may take
     const size_t lds_reg = (size_t)fanout * TS * sizeof(int32_t) * (d_dst_out ? 2 : 1);
     if constexpr (TS == 256) if (fanout <= 32 && lds_reg <= 60 * 1024) {
 #define FGL_LAUNCH_REG(F)                                                                                           \
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
-                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr)
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out)
         if (fanout <= 8) FGL_LAUNCH_REG(8);
         else if (fanout <= 16) FGL_LAUNCH_REG(16);
         else FGL_LAUNCH_REG(32);
@@ -285,8 +327,8 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
 #define FGL_LAUNCH_EDGES(U)                                                                                        \
     hipLaunchKernelGGL((sample_edges_kernel<TS, U>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,          \
-                       n_seeds_max, d_n_seeds, fanout, row_start, deg, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr)
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out)
     FGL_LAUNCH_EDGES(16);
 #undef FGL_LAUNCH_EDGES
     FGL_CHECK_LAUNCH("sample_edges_kernel");

@@ -82,9 +82,13 @@ int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_pref
 
 // `in` and `out` may be the same buffer: every lane reads its items before the barrier and
 // writes only its own positions after it (hence no __restrict__ on them).
+// tile_prefix == nullptr: no prefix launch ran; the workgroup sums the earlier tiles' sums itself
+// (tile 0 needs none), and the lane that holds index n also stores the grand total in *total_extra.
 __global__ __launch_bounds__(kBlock) void scan_apply_kernel(const int32_t* in, int64_t n_max,
                                                             const int32_t* __restrict__ d_n,
-                                                            const int32_t* __restrict__ tile_prefix, int32_t* out)
+                                                            const int32_t* __restrict__ tile_sums,
+                                                            const int32_t* __restrict__ tile_prefix, int32_t* out,
+                                                            int32_t* __restrict__ total_extra)
 {
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n = actual_count(n_max, d_n);
@@ -96,14 +100,19 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(const int32_t* in, i
         v[j] = (base + j < n) ? in[base + j] : 0;
         s += v[j];
     }
+    const int before = tile_prefix ? tile_prefix[blockIdx.x] : block_sum_before<kBlock>(tile_sums, blockIdx.x, smem);
     int total;
-    int run = block_exclusive_scan<kBlock>(s, smem, &total) + tile_prefix[blockIdx.x];
+    int run = block_exclusive_scan<kBlock>(s, smem, &total) + before;
 #pragma unroll
     for (int j = 0; j < kScanItems; ++j) {
         if (base + j <= n) out[base + j] = run;  // index n receives the grand total
+        if (base + j == n && tile_prefix == nullptr && total_extra) *total_extra = run;
         run += v[j];
     }
 }
+
+// Up to this many tiles the apply pass derives its tile offsets itself (no prefix launch).
+constexpr int64_t kSelfPrefixTiles = 4096;
 
 size_t scan_workspace_bytes(int64_t n_max)
 {
@@ -130,12 +139,20 @@ int launch_exclusive_sum(const int32_t* d_in, int64_t n_max, const int32_t* d_n,
     Carver c(d_ws);
     int32_t* sums = c.take<int32_t>((size_t)tiles);
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
-    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, sums);
-    FGL_CHECK_LAUNCH("scan_tile_sums_kernel");
-    int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_total_extra, nullptr, nullptr, 0, nullptr, 0, stream);
-    if (rc != FGL_OK) return rc;
-    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, prefix,
-                       d_out);
+    // one tile: its offset is zero, the apply pass alone does the job; few tiles: the apply pass sums the
+    // tile sums before its own; many: a single-workgroup launch turns the sums into offsets first
+    if (tiles > 1) {
+        hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, sums);
+        FGL_CHECK_LAUNCH("scan_tile_sums_kernel");
+    }
+    if (tiles > kSelfPrefixTiles) {
+        int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_total_extra, nullptr, nullptr, 0, nullptr, 0, stream);
+        if (rc != FGL_OK) return rc;
+    } else {
+        prefix = nullptr;
+    }
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, sums, prefix,
+                       d_out, d_total_extra);
     FGL_CHECK_LAUNCH("scan_apply_kernel");
     return FGL_OK;
 }

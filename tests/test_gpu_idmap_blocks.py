@@ -43,7 +43,11 @@ def test_hand_fixture(cuda):
 
 
 @pytest.mark.parametrize("n_ids,n_dst,n_edges", [(50, 10, 4000), (100_000, 1000, 15_000), (2**31 - 1, 64, 50_000),
-                                                 (3_000_000, 8192, 1_000_000), (7, 7, 0), (1000, 1, 2049)])
+                                                 (3_000_000, 8192, 1_000_000), (7, 7, 0), (1000, 1, 2049),
+                                                 # 1024 tiles of 2048 edges: up to there the numbering pass scans the
+                                                 # tile counts itself, beyond a scan launch does
+                                                 (5_000_000, 4096, 2_097_152), (5_000_000, 4096, 2_097_153),
+                                                 (40_000_000, 100, 2_500_000)])
 def test_transfer_edge_id_vs_oracle(cuda, oracle, n_ids, n_dst, n_edges):
     print("idmap %d %d %d" % (n_ids, n_dst, n_edges), flush=True)
     rng = np.random.default_rng(n_edges + n_dst)

@@ -11,7 +11,8 @@ def dev_i32(a, cuda):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(cuda)
 
 
-@pytest.mark.parametrize("n", [0, 1, 63, 2047, 2048, 2049, 100_000, 3_000_001])
+# one tile (a single launch), a few tiles (offsets summed by each workgroup), beyond 4096 tiles (scan launch in between)
+@pytest.mark.parametrize("n", [0, 1, 63, 2047, 2048, 2049, 100_000, 3_000_001, 8_388_607, 8_388_608, 9_000_001])
 def test_exclusive_sum(cuda, oracle, n):
     import fastgl
     print("exclusive_sum n=%d" % n, flush=True)
@@ -53,6 +54,18 @@ def test_sample_bit_exact_vs_oracle(cuda, oracle, small_graph, ptr_dtype, fanout
     assert np.array_equal(bptr, wptr)
     assert np.array_equal(dst, wdst)
     assert np.array_equal(src, wsrc)
+
+
+@pytest.mark.parametrize("n_seeds", [1_048_576, 1_048_577, 1_300_000])
+def test_sample_many_seeds_vs_oracle(cuda, oracle, small_graph, n_seeds):
+    """Around 4096 tiles of 256 seeds the way the tile offsets are derived changes (summed by each
+    workgroup below, a scan launch above): same bits either way."""
+    print("sample %d seeds" % n_seeds, flush=True)
+    indptr, indices = small_graph
+    seeds = np.random.default_rng(n_seeds).integers(0, indptr.size - 1, size=n_seeds).astype(np.int32)
+    src, dst, bptr = _sample(cuda, indptr, indices, seeds, 5, seed=3, stream=1)
+    wsrc, wdst, wptr = oracle.sample_node(indptr, indices, seeds, 5, rng_seed=3, stream_id=1)
+    assert np.array_equal(bptr, wptr) and np.array_equal(dst, wdst) and np.array_equal(src, wsrc)
 
 
 def test_sample_full_neighbourhood_closed_form(cuda, small_graph):
