@@ -324,8 +324,8 @@ __global__ __launch_bounds__(kBlock) void idmap_lookup_kernel(TableRef t, int32_
 // ---- arrival-order numbering (FGL_IDMAP_ARRIVAL) ---------------------------------------
 // The lane whose CAS installs a key numbers it at once from a global counter, as the
 // reference does (id_map.cu:314-321) -- but with one counter update per workgroup instead
-// of one per new id.  Two launches instead of four and about half the table traffic; the
-// numbering of new ids then depends on scheduling (any run is a valid map, and equal to
+// of one per new id.  Fewer launches and about half the table traffic (though the two barriers
+// per round cost about what that saves); the numbering of new ids then depends on scheduling (any run is a valid map, and equal to
 // every other after sorting the new ids).
 __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t, const int32_t* __restrict__ src,
                                                                       int64_t e_max, const int32_t* __restrict__ d_e,
