@@ -48,7 +48,9 @@ def run_modes(cuda, oracle, ptr, idx, deg, X_t, n_src, tol):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("D", [1, 7, 30, 64, 100, 128, 256, 602, 1030])
+# 602, 1030, 300 (and 514 in bf16): rows that fill 64-lane groups badly take the flat-mapped kernel; 7, 30, 50, 130:
+# the last lane of a row overlaps its neighbour instead of moving a cut-off vector
+@pytest.mark.parametrize("D", [1, 3, 7, 30, 50, 64, 100, 128, 130, 256, 300, 514, 602, 1030])
 def test_aggregate_vs_oracle(cuda, oracle, dtype, D):
     print("aggregate D=%d %s" % (D, dtype), flush=True)
     rng = np.random.default_rng(D)
@@ -171,6 +173,25 @@ def test_strided_rows_and_narrow_vectors(cuda, oracle):
         got = fastgl.aggregate(dev_i32(ptr, cuda), dev_i32(idx, cuda), X, mode="mean", zero_policy="zeros")
         want = oracle.aggregate(ptr, idx, X.cpu().numpy(), "mean", 1)
         assert rel_err(got.cpu().numpy(), want) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_strided_wide_rows(cuda, oracle, dtype):
+    """Column slices of a 700-column table: wide rows (flat-mapped kernel) whose stride differs from their
+    length, even and odd lengths, bases that are only 4-byte (fp32) or 2-byte (bf16) aligned; one block with
+    rows of several hundred entries, so that the long-row launch sees the same layouts."""
+    import fastgl
+    print("aggregate strided wide %s" % dtype, flush=True)
+    rng = np.random.default_rng(9)
+    n_dst, n_src = 150, 700
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 10, hubs=[(5, 200), (6, 129)])
+    wide = torch.from_numpy(rng.standard_normal((n_src, 700)).astype(np.float32)).to(cuda).to(dtype)
+    for lo, hi in ((0, 602), (1, 603), (2, 603), (3, 700), (0, 301), (5, 38), (4, 37)):
+        X = wide[:, lo:hi]
+        for mode in ("sum", "mean"):
+            got = fastgl.aggregate(dev_i32(ptr, cuda), dev_i32(idx, cuda), X, mode=mode, zero_policy="self")
+            want = oracle.aggregate(ptr, idx, X.float().cpu().numpy(), mode, 0)
+            assert rel_err(got.float().cpu().numpy(), want) < TOL[dtype], (lo, hi, mode)
 
 
 def test_closed_forms_on_device(cuda):
