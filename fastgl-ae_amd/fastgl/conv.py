@@ -40,19 +40,62 @@ def _block_csr(graph):
     return ops.exclusive_sum(raw), graph.edges()[0].int(), raw
 
 
+def _aggregate_first_is_cheaper(n_src, n_dst, n_edges, d_in, d_out):
+    """(A X) W against A (X W): the product runs over n_dst rows instead of n_src, the gather moves rows of
+    d_in instead of d_out columns.  Priced with round figures for this GPU (fp32 matrix product ~50 TFLOP/s,
+    random row gather ~5 TB/s); the two orders agree up to fp32 rounding."""
+    flop_s, byte_s = 50e12, 5e12
+    product_first = 2.0 * n_src * d_in * d_out / flop_s + 4.0 * n_edges * d_out / byte_s
+    gather_first = 2.0 * n_dst * d_in * d_out / flop_s + 4.0 * n_edges * d_in / byte_s
+    return gather_first < product_first
+
+
 class MA_Function(torch.autograd.Function):
+    """GCN layer ``A_norm X W``.  The reference multiplies first and gathers rows of ``X W``
+    (aggregate_acc.cpp:133-160); a sampled block has several times more source than destination rows, so
+    for most layers it is cheaper to gather rows of ``X`` and multiply the (fewer) gathered rows --
+    ``order="auto"`` (default) prices both and picks; ``"product_first"`` is the reference's order.  Either
+    way a destination row without edges passes ``(X W)[d]`` through and sends no gradient back
+    (aggregate_acc_kernel.cu:307-309,498-500)."""
+
     @staticmethod
     def forward(ctx, edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat, weight, neighbor_num,
-                transposed=None):
-        ctx.save_for_backward(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat)
+                transposed=None, order="auto"):
         ctx.transposed = transposed
-        return ops.forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, weight, neighbor_num,
-                               dst_nodes)[0]
+        n_dst = int(dst_nodes)
+        gather_first = order == "gather_first" or (order == "auto" and _aggregate_first_is_cheaper(
+            input_feat.size(0), n_dst, src_edges.numel(), weight.size(0), weight.size(1)))
+        ctx.gather_first = gather_first
+        if not gather_first:
+            ctx.save_for_backward(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat)
+            return ops.forward_gcn(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, input_feat, weight, neighbor_num,
+                                   dst_nodes)[0]
+        ax = ops.aggregate(edge_ptr, src_edges, input_feat, mode="gcn", zero_policy="self", row_norm=dst_norm_degs,
+                           col_norm=src_norm_degs, n_rows=n_dst, longest_row=ops._fanout_bound(edge_ptr, neighbor_num))
+        ctx.n_src = int(input_feat.size(0))
+        ctx.save_for_backward(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, ax)
+        return torch.mm(ax, weight)
 
     @staticmethod
     def backward(ctx, d_input):
-        edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat = ctx.saved_tensors
         d_input = d_input.contiguous()
+        if ctx.gather_first:
+            edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, ax = ctx.saved_tensors
+            # rows without edges took no part in the sum: no gradient through them (as in the reference)
+            has_edges = (edge_ptr[1:] != edge_ptr[:-1]).to(d_input.dtype)[:, None]
+            d_out = d_input * has_edges
+            d_w = torch.mm(ax.transpose(0, 1), d_out)
+            d_x = None
+            if ctx.needs_input_grad[5]:
+                d_ax = torch.mm(d_out, weight.transpose(0, 1))
+                if ctx.transposed is None:
+                    t_ptr, t_idx = ops.block_transpose(edge_ptr, src_edges, int(d_input.size(0)), ctx.n_src)
+                else:
+                    t_ptr, t_idx = _transposed(ctx.transposed)
+                d_x = ops.aggregate(t_ptr, t_idx, d_ax, mode="gcn", zero_policy="zeros", row_norm=src_norm_degs,
+                                    col_norm=dst_norm_degs, n_rows=ctx.n_src)
+            return None, None, None, None, None, d_x, d_w, None, None, None
+        edge_ptr, src_edges, src_norm_degs, dst_norm_degs, weight, input_feat = ctx.saved_tensors
         if ctx.transposed is None:
             d_x, d_w = ops.backward_gcn(edge_ptr, src_edges, dst_norm_degs, src_norm_degs, d_input, weight, input_feat)
         elif not ctx.needs_input_grad[5]:
@@ -68,7 +111,7 @@ class MA_Function(torch.autograd.Function):
                               col_norm=dst_norm_degs, n_rows=int(input_feat.size(0)))
             d_x = torch.mm(g, weight.transpose(0, 1))
             d_w = torch.mm(input_feat.transpose(0, 1), g)
-        return None, None, None, None, None, d_x, d_w, None, None
+        return None, None, None, None, None, d_x, d_w, None, None, None
 
 
 class _Conv(nn.Module):
@@ -92,10 +135,12 @@ class _Conv(nn.Module):
 
 
 class GCNConv(_Conv):
+    order = "auto"  # "product_first": the reference's order of product and gather in every layer (see MA_Function)
+
     def forward(self, edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat, neighbor_num,
                 transposed=None):
         return MA_Function.apply(edge_ptr, src_edges, src_norm_degs, dst_norm_degs, dst_nodes, input_feat,
-                                 self._weight(), neighbor_num, transposed)
+                                 self._weight(), neighbor_num, transposed, self.order)
 
 
 def _stack(conv, in_feats, n_hidden, n_classes, n_layers, weight):

@@ -37,16 +37,21 @@ def dense_adj(block, kind):
 
 
 @pytest.mark.parametrize("input_grad", [True, False])
-@pytest.mark.parametrize("model_name", ["gcn", "gin"])
+@pytest.mark.parametrize("model_name", ["gcn", "gcn:product_first", "gcn:gather_first", "gin"])
 def test_gcn_gin_forward_backward(cuda, oracle, small_graph, model_name, input_grad):
     """input_grad=False is the training case (raw features): the first layer then computes only the weight
-    gradient, without ever building the outermost block's transpose."""
+    gradient, without ever building the outermost block's transpose.  GCN in both orders of product and
+    gather (the reference's, and gather first) and with the layer's own choice."""
     import fastgl
     print("conv %s input_grad=%s" % (model_name, input_grad), flush=True)
     input_nodes, _, blocks = small_blocks(cuda, oracle, small_graph)
     torch.manual_seed(0)
+    model_name, _, order = model_name.partition(":")
     cls = fastgl.GCN if model_name == "gcn" else fastgl.GIN
     model = cls(20, 16, 5, 2, None, True, 0.0).to(cuda)
+    for layer in model.layers:
+        if order:
+            layer.order = order
     x = torch.randn(input_nodes.numel(), 20, device=cuda, requires_grad=input_grad)
     out = model(blocks, x, neighbor_list=[4, 3])
     gout = torch.randn_like(out)
