@@ -16,6 +16,7 @@ from .ops import (  # noqa: F401
     backward_gin,
     block_transpose,
     cal_deg,
+    edge_softmax,
     exclusive_sum,
     forwaed_gin,
     forward_gat,
@@ -41,6 +42,6 @@ from .conv import (  # noqa: F401
     MA_Function_GIN,
     MA_Function_Mean,
     SAGEConv,
-    edge_softmax,
+    edge_softmax_torch,
 )
 from . import graph  # noqa: F401

@@ -258,9 +258,10 @@ class MA_Function_GAT(torch.autograd.Function):
         return None, None, None, None, None, d_x, None, None, None
 
 
-def edge_softmax(edge_ptr, dst_edges, e, n_dst):
+def edge_softmax_torch(edge_ptr, dst_edges, e, n_dst):
     """softmax of the edge scores ``e`` [E, H] over the edges of each destination (what the reference
-    takes from dgl.nn.functional.edge_softmax, GraphConv.py:272)"""
+    takes from dgl.nn.functional.edge_softmax, GraphConv.py:272), written with torch operators: the plain
+    fp32 restatement that ``ops.edge_softmax`` (one HIP launch, used by ``GATConv``) is tested against."""
     idx = dst_edges.long()
     top = torch.full((n_dst, e.size(1)), float("-inf"), dtype=e.dtype, device=e.device)
     top = top.scatter_reduce(0, idx[:, None].expand(-1, e.size(1)), e, reduce="amax", include_self=True)
@@ -295,13 +296,16 @@ class GATConv(nn.Module):
         el = (feat_src * self.attn_l).sum(dim=-1)  # [n_src, H]
         er = (feat_dst * self.attn_r).sum(dim=-1)  # [n_dst, H]
         edge_ptr, src_edges, _ = _block_csr(graph)
-        dst_edges = graph.edges()[1].int()
-        # u_add_v + leaky_relu + edge_softmax (DGL calls in the reference, GraphConv.py:265-272)
-        e = self.leaky_relu(el.index_select(0, src_edges.long()) + er.index_select(0, dst_edges.long()))
-        edge_data = self.attn_drop(edge_softmax(edge_ptr, dst_edges, e, dst_nodes)).contiguous()
+        # u_add_v + leaky_relu + edge_softmax (DGL calls in the reference, GraphConv.py:265-272) in one launch.
+        # No gradient reaches the coefficients (the aggregation's backward returns none for them, as in the
+        # reference, GraphConv.py:227), so they are computed outside the autograd graph.
+        with torch.no_grad():
+            alpha = ops.edge_softmax(edge_ptr, src_edges, el.detach().contiguous(), er.detach().contiguous(),
+                                     self.leaky_relu.negative_slope, n_rows=dst_nodes)
+            edge_data = self.attn_drop(alpha).contiguous()
         feat_src = feat_src.reshape(-1, self.out_feats * self.num_heads)
         transposed = graph if isinstance(graph, Block) and torch.is_grad_enabled() else None
-        return MA_Function_GAT.apply(edge_ptr, edge_data.detach(), src_edges, dst_edges, dst_nodes, feat_src, self.num_heads,
+        return MA_Function_GAT.apply(edge_ptr, edge_data, src_edges, None, dst_nodes, feat_src, self.num_heads,
                                      neighbor_num, transposed)
 
 

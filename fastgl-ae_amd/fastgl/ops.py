@@ -353,6 +353,30 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     return out
 
 
+def edge_softmax(indptr, indices, el, er, negative_slope=0.2, n_rows=None):
+    """Attention coefficients of a GAT layer over a block CSR, ``float32 [n_entries, n_heads]``:
+    ``softmax`` over the entries of each row of ``leaky_relu(el[indices[e]] + er[row])`` -- the reference's
+    ``u_add_v`` + ``leaky_relu`` + ``edge_softmax`` (GraphConv.py:265-272) in one launch.  ``el``: float32
+    [n_cols, n_heads], ``er``: float32 [n_rows, n_heads]."""
+    _check_input(indptr, "indptr", _I32)
+    _check_input(indices, "indices", _I32)
+    _check_input(el, "el", (torch.float32,))
+    _check_input(er, "er", (torch.float32,))
+    if el.dim() != 2 or er.dim() != 2 or el.size(1) != er.size(1):
+        raise RuntimeError("el and er must be [n, n_heads] with the same head count")
+    dev = _same_device(indptr, indices, el, er)
+    n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
+    if n < 0 or n > indptr.numel() - 1 or n > er.size(0):
+        raise RuntimeError("n_rows (%d) does not match indptr (%d entries) / er (%d rows)" % (n, indptr.numel(), er.size(0)))
+    H = int(el.size(1))
+    with torch.cuda.device(dev):
+        alpha = torch.empty((int(indices.numel()), H), dtype=torch.float32, device=dev)
+        if n > 0 and indices.numel() > 0:
+            L.check(L.lib().fgl_edge_softmax(L.ptr(indptr), L.ptr(indices), n, None, L.ptr(el), L.ptr(er), H,
+                                             float(negative_slope), L.ptr(alpha), L.stream_handle()))
+    return alpha
+
+
 def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False, sorted_rows=False):
     """Column-major companion ``(t_indptr[n_cols+1], t_indices[nnz])`` of a block CSR; with
     ``edge_ids=True`` also ``t_edge[nnz]``, the position in ``indices`` of every transposed entry.

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 3
+#define FGL_ABI_VERSION 4
 
 enum fgl_error {
     FGL_OK = 0,
@@ -240,6 +240,19 @@ int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
                   const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
                   int64_t longest_row_max, const int32_t* d_longest_row,
                   void* d_out, int64_t ldo, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * Attention coefficients of a GAT layer over a block CSR -- replaces the three DGL calls of
+ * the reference's GATConv.forward (GraphConv.py:265-272: apply_edges(u_add_v('el','er')),
+ * leaky_relu, edge_softmax).  d_el float[n_cols, n_heads] (per source node), d_er
+ * float[n_rows, n_heads] (per destination row); for entry e of row r and head h
+ *   s = leaky_relu(el[indices[e], h] + er[r, h]),  alpha[e, h] = softmax of s over the row's entries.
+ * d_alpha float[n_entries, n_heads] is what fgl_aggregate(FGL_AGG_EDGE) takes as d_edge_w.
+ * A row without entries writes nothing.
+ * ------------------------------------------------------------------------------- */
+int fgl_edge_softmax(const int32_t* d_indptr, const int32_t* d_indices, int64_t n_rows_max,
+                     const int32_t* d_n_rows, const float* d_el, const float* d_er, int n_heads,
+                     float negative_slope, float* d_alpha, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * Seeded R-MAT key generator for the synthetic graphs (a=.57 b=.19 c=.19 d=.05).

@@ -14,6 +14,8 @@
  *   cuda_operators/aggregate_acc_kernel.cu:270-331,375-427,467-517,554-596
  *                                             GCN / GIN forward and backward, zero-degree rule
  *   cuda_operators/aggregate_acc_kernel.cu:835-886,924-979   GAT forward and backward
+ *   GraphConv.py:265-272                      GAT attention coefficients (DGL u_add_v, leaky_relu,
+ *                                             edge_softmax: third-party, restated from their definitions)
  *
  * Deliberate departures from the reference (each one is also what the HIP library does):
  *   - random picks are WITHOUT replacement (Floyd's subset algorithm) from a
@@ -35,6 +37,8 @@
  *   orc_cal_deg, orc_exclusive_sum   numpy.bincount / numpy.cumsum
  *   orc_aggregate_f64   scipy.sparse products, all-ones / one-hot closed forms
  *   orc_aggregate_edge_f64  scipy.sparse products per head; reduces to orc_aggregate_f64 for unit weights
+ *   orc_edge_softmax_f64  scipy.special.softmax per row and head; rows sum to one; invariance to a
+ *                       shift of er; uniform 1/deg for equal scores; the leaky-relu slope by hand values
  *   orc_transpose       scipy.sparse transpose (stable order)
  *   orc_rmat_keys       quadrant frequencies against (a,b,c,d); symmetry; determinism
  *   orc_aggregate_f32   (timing variant only) compared with orc_aggregate_f64
@@ -424,6 +428,34 @@ ORC_API void orc_aggregate_edge_f64(const int32_t* indptr, const int32_t* indice
             const float* x = X + (int64_t)indices[e] * ldx;
             const float* w = edge_w + (int64_t)(edge_index ? edge_index[e] : e) * n_heads;
             for (int f = 0; f < D; ++f) o[f] += (double)w[f / unit] * (double)x[f];
+        }
+    }
+}
+
+/* GAT attention coefficients (reference: GraphConv.py:265-272, which calls DGL 1.0's
+ * apply_edges(fn.u_add_v), torch's LeakyReLU and dgl.nn.functional.edge_softmax; DGL is not
+ * part of the reference checkout, so their published definitions are restated):
+ *   s(e, h)     = leaky_relu(el[indices[e], h] + er[r, h])   for entry e of destination row r
+ *   alpha(e, h) = exp(s(e, h)) / sum over the entries e' of row r of exp(s(e', h))
+ * computed in fp64 with the row maximum subtracted. */
+ORC_API void orc_edge_softmax_f64(const int32_t* indptr, const int32_t* indices, int64_t n_rows, const float* el,
+                                  const float* er, int n_heads, double negative_slope, double* alpha)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        for (int h = 0; h < n_heads; ++h) {
+            double top = -INFINITY, sum = 0.0;
+            for (int64_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+                double s = (double)el[(int64_t)indices[e] * n_heads + h] + (double)er[r * n_heads + h];
+                if (s < 0.0) s *= negative_slope;
+                alpha[e * n_heads + h] = s;
+                if (s > top) top = s;
+            }
+            for (int64_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+                alpha[e * n_heads + h] = exp(alpha[e * n_heads + h] - top);
+                sum += alpha[e * n_heads + h];
+            }
+            for (int64_t e = indptr[r]; e < indptr[r + 1]; ++e) alpha[e * n_heads + h] /= sum;
         }
     }
 }

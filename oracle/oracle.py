@@ -54,6 +54,8 @@ def lib():
             f.restype = None
         L.orc_aggregate_edge_f64.argtypes = [vp, vp, i64, vp, i64, i32, i32, vp, i32, vp, vp]
         L.orc_aggregate_edge_f64.restype = None
+        L.orc_edge_softmax_f64.argtypes = [vp, vp, i64, vp, vp, i32, C.c_double, vp]
+        L.orc_edge_softmax_f64.restype = None
         L.orc_rmat_keys.argtypes = [i64, i64, i32, i64, u64, vp]
         L.orc_rmat_keys.restype = None
         L.orc_num_threads.argtypes = []
@@ -197,6 +199,20 @@ def aggregate_edge(indptr, indices, X, edge_w, zero_policy=0, edge_index=None):
     lib().orc_aggregate_edge_f64(_p(indptr), _p(indices), n_rows, _p(X), X.shape[1], D, zero_policy, _p(edge_w),
                                  edge_w.shape[1], _p(ei), _p(out))
     return out
+
+
+def edge_softmax(indptr, indices, el, er, negative_slope=0.2):
+    """fp64 GAT attention coefficients [n_entries, n_heads]; el float32 [n_cols, H], er float32 [n_rows, H]."""
+    indptr = _i32(indptr)
+    indices = _i32(indices)
+    el = np.ascontiguousarray(el, dtype=np.float32)
+    er = np.ascontiguousarray(er, dtype=np.float32)
+    n_rows = indptr.shape[0] - 1
+    H = el.shape[1]
+    assert er.shape == (n_rows, H)
+    alpha = np.zeros((indices.shape[0], H), dtype=np.float64)
+    lib().orc_edge_softmax_f64(_p(indptr), _p(indices), n_rows, _p(el), _p(er), H, float(negative_slope), _p(alpha))
+    return alpha
 
 
 def transpose_with_edges(indptr, indices, n_cols: int):

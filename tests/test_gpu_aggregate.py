@@ -354,3 +354,35 @@ def test_random_blocks_all_modes_against_the_oracle(cuda, oracle):
         want = oracle.aggregate(want_ptr, want_idx, G.float().cpu().numpy(), "sum", 1)
         assert np.array_equal(t_ptr.cpu().numpy(), want_ptr)
         assert rel_err(got.float().cpu().numpy(), want) < TOL[dtype], case
+
+
+@pytest.mark.parametrize("H", [1, 3, 4, 8])
+def test_edge_softmax_vs_oracle_and_torch(cuda, oracle, H):
+    """GAT attention coefficients in one launch against the fp64 oracle and against the plain torch fp32
+    restatement (gather, leaky_relu, scatter-max, exp, scatter-add, divide); tolerance 1e-5 relative to the
+    largest coefficient (fp32 exp and division).  Rows without entries, one-entry rows (coefficient 1), a row
+    of several hundred entries, scores large enough that exp would overflow without the maximum subtracted."""
+    import fastgl
+    print("edge_softmax H=%d" % H, flush=True)
+    rng = np.random.default_rng(40 + H)
+    n_dst, n_src = 700, 2500
+    ptr, idx, deg = make_block(rng, n_dst, n_src, 12, hubs=[(5, 300), (6, 1), (7, 0)])
+    el = (rng.standard_normal((n_src, H)) * 3).astype(np.float32)
+    er = (rng.standard_normal((n_dst, H)) * 3).astype(np.float32)
+    el[:10] += 95.0  # exp(95) overflows fp32
+    d_ptr, d_idx = dev_i32(ptr, cuda), dev_i32(idx, cuda)
+    d_el, d_er = torch.from_numpy(el).to(cuda), torch.from_numpy(er).to(cuda)
+    got = fastgl.edge_softmax(d_ptr, d_idx, d_el, d_er, 0.2)
+    want = oracle.edge_softmax(ptr, idx, el, er, 0.2)
+    assert tuple(got.shape) == want.shape and got.dtype == torch.float32
+    assert rel_err(got.cpu().numpy(), want) < 1e-5
+    assert torch.isfinite(got).all()
+    one = ptr[6]
+    assert np.array_equal(got[one].cpu().numpy(), np.ones(H, np.float32))
+    dst = torch.repeat_interleave(torch.arange(n_dst, device=cuda), torch.from_numpy(deg).to(cuda)).int()
+    e = torch.nn.functional.leaky_relu(d_el.index_select(0, d_idx.long()) + d_er.index_select(0, dst.long()), 0.2)
+    ref = fastgl.edge_softmax_torch(d_ptr, dst, e, n_dst)
+    assert rel_err(got.cpu().numpy(), ref.double().cpu().numpy()) < 1e-5
+    # an empty block
+    empty = fastgl.edge_softmax(dev_i32(np.zeros(4, np.int32), cuda), dev_i32(np.zeros(0, np.int32), cuda), d_el, d_er[:3], 0.2)
+    assert tuple(empty.shape) == (0, H)

@@ -129,3 +129,38 @@ def test_edge_weighted_aggregation(oracle):
     y = rng.standard_normal((n_dst, D)).astype(np.float32)
     aty = oracle.aggregate_edge(t_ptr, t_idx, y, alpha, 1, edge_index=t_edge)
     assert np.isclose((want * y).sum(), (X * aty).sum(), rtol=1e-9)
+
+
+def test_edge_softmax_pins(oracle):
+    """The attention coefficients against scipy's softmax row by row and head by head, plus what the
+    mathematics fixes: rows sum to one, a shift of er changes nothing where no score changes sign, equal
+    scores give 1/deg, and hand values for the leaky-relu slope."""
+    from scipy.special import softmax
+    rng = np.random.default_rng(21)
+    n_dst, n_src, H = 150, 400, 3
+    indptr, indices, deg = _block(rng, n_dst, n_src, 11)
+    el = rng.standard_normal((n_src, H)).astype(np.float32)
+    er = rng.standard_normal((n_dst, H)).astype(np.float32)
+    got = oracle.edge_softmax(indptr, indices, el, er, 0.2)
+    assert got.shape == (indptr[-1], H)
+    for r in range(n_dst):
+        a, b = indptr[r], indptr[r + 1]
+        if a == b:
+            continue
+        s = el[indices[a:b]].astype(np.float64) + er[r].astype(np.float64)
+        s = np.where(s > 0, s, 0.2 * s)
+        assert np.allclose(got[a:b], softmax(s, axis=0), rtol=1e-12, atol=1e-15)
+        assert np.allclose(got[a:b].sum(0), 1.0, rtol=1e-12)
+    # all scores positive: leaky_relu is the identity and a shift of er cancels in the softmax
+    el_pos = np.abs(el) + 1.0
+    a1 = oracle.edge_softmax(indptr, indices, el_pos, np.full((n_dst, H), 0.5, np.float32), 0.2)
+    a2 = oracle.edge_softmax(indptr, indices, el_pos, np.full((n_dst, H), 3.0, np.float32), 0.2)
+    assert np.allclose(a1, a2, rtol=1e-6)
+    # equal scores: 1/deg
+    a3 = oracle.edge_softmax(indptr, indices, np.zeros((n_src, H), np.float32), er, 0.2)
+    assert np.allclose(a3, np.repeat(1.0 / np.maximum(deg, 1), deg)[:, None], rtol=1e-12)
+    # by hand: one row, two entries, scores +1 and -1 with slope 0.5 -> exp(1), exp(-0.5)
+    a4 = oracle.edge_softmax(np.array([0, 2], np.int32), np.array([0, 1], np.int32),
+                             np.array([[1.0], [-1.0]], np.float32), np.zeros((1, 1), np.float32), 0.5)
+    want = np.exp([1.0, -0.5]) / np.exp([1.0, -0.5]).sum()
+    assert np.allclose(a4[:, 0], want, rtol=1e-12)
