@@ -129,6 +129,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     BlocksPlan p;
     int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
     if (rc != FGL_OK) return rc;
+    FGL_REQUIRE(idmap_flags == FGL_IDMAP_ORDERED || idmap_flags == FGL_IDMAP_ARRIVAL, "sample_blocks: unknown id-map flags %d", idmap_flags);
     FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
     FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
     // A table smaller than the plan's worst case is accepted (batches are usually far below the
@@ -173,7 +174,8 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped
         const int64_t grow_to = (h + 1 < n_hops && p.cap_dst[h + 1] < p.cap_uniq) ? p.cap_dst[h + 1] : p.cap_uniq;
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
-                                  d_counts + h + 1, d_uniq, grow_to, idmap_flags, d_status, ws + ws_sample,
+                                  d_counts + h + 1, d_uniq, grow_to,
+                                  idmap_flags | (h == n_hops - 1 ? FGL_IDMAP_FINAL : 0), d_status, ws + ws_sample,
                                   ws_bytes - ws_sample, s);
         if (rc != FGL_OK) return rc;
     }

@@ -22,11 +22,11 @@
 //                 so a bound much larger than the batch costs nothing).  Skipped while the bound
 //                 is at most 1024 tiles (2 M edges): the number pass then scans the tile counts
 //                 itself in every workgroup, and its first workgroup publishes the total
-//   4. number     per edge, coalesced: a first edge computes its id's local id from the three
-//                 counts, stores it in the slot, appends the id to the unique list and relabels
-//                 itself without reading the table; a later mention reads the slot and, if the
-//                 val there is still the pending first-edge index, computes the same local id
-//                 from that edge's counts -- either way the same number, so the race is benign.
+//   4. number     per edge, coalesced: the local id follows from the first-edge index that the mark
+//                 pass left for the edge and the three counts (cache-resident arrays): no table read.
+//                 The first edge of a new id appends the id to the unique list and stores the local id
+//                 in the id's slot for later calls -- skipped with FGL_IDMAP_FINAL, when the caller
+//                 will not consult the table again (the last hop of a mini-batch: most of its edges).
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
@@ -158,9 +158,11 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
 __device__ __forceinline__ int64_t tiles_of(int64_t n) { return (n + kTile - 1) / kTile; }
 
 // flags8[tile*256 + lane] bit j  <=>  edge (tile*2048 + lane*8 + j) is the first edge of a new id;
-// before8[tile*256 + lane] = number of flagged edges of the tile before edge tile*2048 + lane*8
+// before8[tile*256 + lane] = number of flagged edges of the tile before edge tile*2048 + lane*8;
+// first_of[e] = pending | index of the first edge that mentions e's id (edges that take part only)
 __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
                                                             const uint32_t* __restrict__ slot_of,
+                                                            uint32_t* __restrict__ first_of,
                                                             uint8_t* __restrict__ flags8, uint16_t* __restrict__ before8,
                                                             int32_t* __restrict__ tile_sums)
 {
@@ -169,9 +171,17 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
     const int64_t n_tiles = tiles_of(n_e);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t first = tile * kTile + (int64_t)threadIdx.x * kItems;
+        const bool whole = first + kItems <= n_e;  // the lane's eight edges all exist: 32-byte vector accesses
         uint32_t p[kItems];
+        if (whole) {
+            const uint4 lo = *reinterpret_cast<const uint4*>(slot_of + first);
+            const uint4 hi = *reinterpret_cast<const uint4*>(slot_of + first + 4);
+            p[0] = lo.x; p[1] = lo.y; p[2] = lo.z; p[3] = lo.w;
+            p[4] = hi.x; p[5] = hi.y; p[6] = hi.z; p[7] = hi.w;
+        } else {
 #pragma unroll
-        for (int j = 0; j < kItems; ++j) p[j] = (first + j < n_e) ? slot_of[first + j] : kEmpty;
+            for (int j = 0; j < kItems; ++j) p[j] = (first + j < n_e) ? slot_of[first + j] : kEmpty;
+        }
         uint32_t v[kItems];
 #pragma unroll
         for (int j = 0; j < kItems; ++j) v[j] = (p[j] < kDone) ? t.words[2 * (size_t)p[j] + 1] : 0u;
@@ -179,6 +189,16 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
 #pragma unroll
         for (int j = 0; j < kItems; ++j)
             if (p[j] < kDone && v[j] == (kPending | (uint32_t)(first + j))) bits |= 1u << j;
+        // what the slot holds now -- pending | index of the id's first edge -- is all the number pass
+        // needs to know about the edge: it never goes back to the table for it
+        if (whole) {
+            *reinterpret_cast<uint4*>(first_of + first) = make_uint4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<uint4*>(first_of + first + 4) = make_uint4(v[4], v[5], v[6], v[7]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kItems; ++j)
+                if (first + j < n_e) first_of[first + j] = v[j];
+        }
         flags8[tile * kBlock + threadIdx.x] = (uint8_t)bits;
         int total;
         const int before = block_exclusive_scan<kBlock>(__popc(bits), smem, &total);
@@ -229,14 +249,19 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
 constexpr int kSelfTilesPerLane = 4;
 constexpr int kSelfPrefixTiles = kBlock * kSelfTilesPerLane;
 
-// Lane per edge.  `src` and `out` may be the same array: an entry is read and written by one lane only.
-// (Edges whose id was numbered before this call were relabelled by the insert pass.)
+// Lane per edge, coalesced.  `src` and `out` may be the same array: an entry is read and written by one lane only.
+// (Edges whose id was numbered before this call were relabelled by the insert pass.)  The local id of an
+// edge's node follows from the index of the node's first edge (first_of, from the mark pass) and the three
+// counts -- small arrays that stay in cache -- so no lane reads the table; the first edge of a new id also
+// appends the id to the unique list and, unless the caller has said that the table will not be consulted
+// again (WRITE_BACK = false), stores the local id in the id's slot.
 // SELF: no prefix launch ran; tile_prefix is unused, the tile counts are scanned here.
-template <bool SELF>
+template <bool SELF, bool WRITE_BACK>
 __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const int32_t* src, int64_t e_max,
                                                               const int32_t* __restrict__ d_e, int64_t n_base_h,
                                                               const int32_t* __restrict__ d_n_base,
                                                               const uint32_t* __restrict__ slot_of,
+                                                              const uint32_t* __restrict__ first_of,
                                                               const uint8_t* __restrict__ flags8,
                                                               const uint16_t* __restrict__ before8,
                                                               const int32_t* __restrict__ tile_sums,
@@ -269,37 +294,23 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
         __syncthreads();
         if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status);
     }
-    // local id of the new node whose first mention is edge x (an edge that the mark pass flagged)
-    auto local_of_first_edge = [&](int64_t x, uint32_t byte_flags) -> int64_t {
-        const int64_t tile = x / kTile;
-        const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
-        return n_base + before_tile + before8[x >> 3] + __popc(byte_flags & ((1u << (x & 7)) - 1u));
-    };
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
         if (p == kDone) continue;
         int64_t local = -1;
         if (p != kEmpty) {
-            const uint32_t f = flags8[e >> 3];
-            if ((f >> (e & 7)) & 1u) {
-                local = local_of_first_edge(e, f);
-                if (local < capacity) {
-                    t.words[2 * (size_t)p + 1] = (uint32_t)local;
-                    uniq[local] = src[e];
-                }
-            } else {
-                const uint32_t v = t.words[2 * (size_t)p + 1];
-                if (!(v & kPending)) {
-                    local = (int64_t)v;
-                } else {
-                    // the first edge's lane has not stored the local id yet (or this lane's cache has
-                    // not seen it): derive it the way that lane does
-                    const int64_t ef = (int64_t)(v & ~kPending);
-                    if (ef < n_e) local = local_of_first_edge(ef, flags8[ef >> 3]);
-                }
+            const int64_t ef = (int64_t)(first_of[e] & ~kPending);  // first edge of this edge's id (ef <= e)
+            if (ef < n_e) {
+                const int64_t tile = ef / kTile;
+                const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
+                local = n_base + before_tile + before8[ef >> 3] + __popc((uint32_t)flags8[ef >> 3] & ((1u << (ef & 7)) - 1u));
             }
             if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
+            if (ef == e && local >= 0) {
+                uniq[local] = src[e];
+                if (WRITE_BACK) t.words[2 * (size_t)p + 1] = (uint32_t)local;
+            }
         }
         out[e] = (int32_t)local;
     }
@@ -435,6 +446,7 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
     const int64_t tiles = ceil_div(n_edges_max > 0 ? n_edges_max : 1, kTile);
     Carver c(nullptr);
     c.take<uint32_t>((size_t)n_edges_max);      // slot_of
+    c.take<uint32_t>((size_t)n_edges_max);      // first_of
     c.take<uint8_t>((size_t)tiles * kBlock);    // flags8
     c.take<uint16_t>((size_t)tiles * kBlock);   // before8
     c.take<int32_t>((size_t)tiles);             // tile sums
@@ -448,18 +460,21 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          size_t ws_bytes, hipStream_t stream)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
-    FGL_REQUIRE(flags == FGL_IDMAP_ORDERED || flags == FGL_IDMAP_ARRIVAL, "idmap_map_src: unknown flags %d", flags);
+    FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
+    const bool final_call = (flags & FGL_IDMAP_FINAL) != 0;
     FGL_REQUIRE(n_edges_max >= 0 && n_base >= 0 && uniq_capacity >= 0, "idmap_map_src: negative size");
-    FGL_REQUIRE(n_base + n_edges_max <= 0x7FFFFFFFll, "idmap_map_src: n_base + n_edges exceeds 31 bits");
+    FGL_REQUIRE(n_base + n_edges_max <= 0x7FFFFFFDll, "idmap_map_src: n_base + n_edges exceeds 31 bits");
     FGL_REQUIRE(n_edges_max == 0 || (d_src_in && d_src_out && d_uniq), "idmap_map_src: null pointer");
     FGL_REQUIRE(d_n_total_out == nullptr || d_n_total_out != d_n_base, "idmap_map_src: n_total_out must not alias n_base");
     if (d_ws == nullptr || ws_bytes < idmap_map_src_workspace_bytes(n_edges_max)) {
         set_error("idmap_map_src: workspace too small (%zu < %zu)", ws_bytes, idmap_map_src_workspace_bytes(n_edges_max));
         return FGL_ERR_WORKSPACE;
     }
+    FGL_REQUIRE(((uintptr_t)d_ws & 15) == 0, "idmap_map_src: the workspace must be 16-byte aligned");
     const int64_t tiles = ceil_div(n_edges_max > 0 ? n_edges_max : 1, kTile);
     Carver c(d_ws);
     uint32_t* slot_of = c.take<uint32_t>((size_t)n_edges_max);
+    uint32_t* first_of = c.take<uint32_t>((size_t)n_edges_max);
     uint8_t* flags8 = c.take<uint8_t>((size_t)tiles * kBlock);
     uint16_t* before8 = c.take<uint16_t>((size_t)tiles * kBlock);
     int32_t* sums = c.take<int32_t>((size_t)tiles);
@@ -468,7 +483,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     const unsigned edge_blocks = stride_grid(n_edges_max, kBlock);
     const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
 
-    if (flags == FGL_IDMAP_ARRIVAL) {
+    if (flags & FGL_IDMAP_ARRIVAL) {
         int32_t* counter = sums;  // one int of the (otherwise unused) tile-sum array
         int rc0 = launch_fill_u32(reinterpret_cast<uint32_t*>(counter), 1, 0u, stream);
         if (rc0 != FGL_OK) return rc0;
@@ -485,20 +500,23 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                        n_edges_max, d_n_edges, slot_of, d_src_out, d_status);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                       slot_of, flags8, before8, sums);
+                       slot_of, first_of, flags8, before8, sums);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
+#define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS)                                                              \
+    hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
+                       n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
+                       uniq_capacity, d_src_out, TOTAL, STATUS)
     if (tiles <= kSelfPrefixTiles) {
-        hipLaunchKernelGGL(idmap_number_kernel<true>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
-                           d_n_edges, n_base, d_n_base, slot_of, flags8, before8, sums, nullptr, d_uniq, uniq_capacity,
-                           d_src_out, d_n_total_out, d_status);
+        if (final_call) FGL_LAUNCH_NUMBER(true, false, nullptr, d_n_total_out, d_status);
+        else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status);
     } else {
         hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max,
                            d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
         FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
-        hipLaunchKernelGGL(idmap_number_kernel<false>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
-                           d_n_edges, n_base, d_n_base, slot_of, flags8, before8, sums, prefix, d_uniq, uniq_capacity,
-                           d_src_out, nullptr, nullptr);
+        if (final_call) FGL_LAUNCH_NUMBER(false, false, prefix, nullptr, nullptr);
+        else FGL_LAUNCH_NUMBER(false, true, prefix, nullptr, nullptr);
     }
+#undef FGL_LAUNCH_NUMBER
     FGL_CHECK_LAUNCH("idmap_number_kernel");
     return FGL_OK;
 }

@@ -21,7 +21,7 @@ AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE = 0, 1, 2, 3, 4
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
 ABI_VERSION = 4  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED = 1, 2, 4, 8
-IDMAP_ORDERED, IDMAP_ARRIVAL = 0, 1
+IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL = 0, 1, 2
 MAX_FANOUT = 192
 
 _i64, _i32, _u64, _u32, _vp, _sz = C.c_int64, C.c_int, C.c_uint64, C.c_uint32, C.c_void_p, C.c_size_t

@@ -68,6 +68,8 @@ enum fgl_zero_policy {
 #define FGL_IDMAP_ORDERED 0 /* new ids numbered by first occurrence (deterministic) */
 #define FGL_IDMAP_ARRIVAL 1 /* new ids numbered as their inserts land (the reference's rule,
                                id_map.cu:314-321): fewer passes, order depends on scheduling */
+#define FGL_IDMAP_FINAL 2   /* (or'ed in) the table is not consulted after this call: the local ids of the
+                               new ids go to the edges and the unique list, not back into the table */
 #define FGL_MAX_FANOUT 192
 
 int fgl_abi_version(void);
@@ -129,10 +131,11 @@ int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids,
 /* number the new source ids and relabel the edges (id_map.cu:290-383 for the src half).
  * n_base ids are already numbered (host value n_base, or *d_n_base when non-NULL).
  * New ids get n_base, n_base+1, ... and are appended to d_uniq -- in order of first
- * occurrence in d_src_in (flags = FGL_IDMAP_ORDERED) or of arrival (FGL_IDMAP_ARRIVAL);
+ * occurrence in d_src_in (flags = FGL_IDMAP_ORDERED) or of arrival (FGL_IDMAP_ARRIVAL), either
+ * optionally or'ed with FGL_IDMAP_FINAL when no later call will look these ids up in the table;
  * d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
  * *d_n_total_out = n_base + number of new ids (must not alias d_n_base).
- * n_base + n_edges_max must stay below 2^31. */
+ * n_base + n_edges_max must stay below 2^31 - 2. */
 size_t fgl_idmap_map_src_workspace_bytes(int64_t n_edges_max);
 int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
                       int64_t n_edges_max, const int32_t* d_n_edges,
@@ -151,7 +154,7 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * in one call with no host synchronisation: per hop sample_node -> id-map, the table and
  * the numbering persisting across hops (hop h's unique list is hop h+1's seed list).
  * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0];
- * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL.
+ * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL (the last hop adds FGL_IDMAP_FINAL by itself).
  * (The reference lists fanouts the other way round and iterates reversed(); the caller
  * passes them already reversed.)
  *
