@@ -182,6 +182,8 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * src_global[h] int32[cap_edges[h]] or NULL; d_uniq int32[cap_uniq];
  * d_counts int32[2*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
  * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word.
+ * The table is scratch: after the call it holds the local ids of the nodes of every hop but the
+ * last (whose new nodes keep a transient value there); d_uniq is the complete map local -> global.
  * ------------------------------------------------------------------------------- */
 int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
                            const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,
