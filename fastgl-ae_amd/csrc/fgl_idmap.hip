@@ -247,7 +247,7 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
 // its first workgroup publishes the node total: one launch less per call where launches, not
 // edges, set the time.  Above it the single-workgroup prefix launch prepares the array once.
 constexpr int kSelfTilesPerLane = 4;
-constexpr int kSelfPrefixTiles = kBlock * kSelfTilesPerLane;
+constexpr int kIdmapSelfPrefixTiles = kBlock * kSelfTilesPerLane;
 
 // Lane per edge, coalesced.  `src` and `out` may be the same array: an entry is read and written by one lane only.
 // (Edges whose id was numbered before this call were relabelled by the insert pass.)  The local id of an
@@ -270,12 +270,12 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                                                               int32_t* __restrict__ d_n_total_out,
                                                               uint32_t* __restrict__ d_status)
 {
-    __shared__ int s_prefix[SELF ? kSelfPrefixTiles : 1];
+    __shared__ int s_prefix[SELF ? kIdmapSelfPrefixTiles : 1];
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
     if constexpr (SELF) {
-        const int n_tiles = (int)tiles_of(n_e);  // <= kSelfPrefixTiles: the launcher checks the bound
+        const int n_tiles = (int)tiles_of(n_e);  // <= kIdmapSelfPrefixTiles: the launcher checks the bound
         int v[kSelfTilesPerLane];
         int s = 0;
 #pragma unroll
@@ -506,7 +506,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
                        uniq_capacity, d_src_out, TOTAL, STATUS)
-    if (tiles <= kSelfPrefixTiles) {
+    if (tiles <= kIdmapSelfPrefixTiles) {
         if (final_call) FGL_LAUNCH_NUMBER(true, false, nullptr, d_n_total_out, d_status);
         else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status);
     } else {

@@ -268,7 +268,7 @@ static inline int tile_seeds_for(int fanout) { return fanout <= 48 ? 256 : 64; }
 
 // Up to this many tiles of seeds the edges kernel derives its tile offsets itself (at most 16 KiB of
 // tile sums per workgroup, read from L2); above it a scan launch prepares them.
-constexpr int64_t kSelfPrefixTiles = 4096;
+constexpr int64_t kSampleSelfPrefixTiles = 4096;
 
 size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
 {
@@ -302,7 +302,7 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     FGL_CHECK_LAUNCH("sample_degree_kernel");
     // few tiles: each workgroup of the edges kernel sums the earlier tile sums itself (the last one
     // publishes the totals), which saves the scan launch in between
-    if (tiles > kSelfPrefixTiles) {
+    if (tiles > kSampleSelfPrefixTiles) {
         int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds,
                                     TS, stream);
         if (rc != FGL_OK) return rc;

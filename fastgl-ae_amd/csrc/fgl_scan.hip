@@ -112,7 +112,7 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(const int32_t* in, i
 }
 
 // Up to this many tiles the apply pass derives its tile offsets itself (no prefix launch).
-constexpr int64_t kSelfPrefixTiles = 4096;
+constexpr int64_t kScanSelfPrefixTiles = 4096;
 
 size_t scan_workspace_bytes(int64_t n_max)
 {
@@ -145,7 +145,7 @@ int launch_exclusive_sum(const int32_t* d_in, int64_t n_max, const int32_t* d_n,
         hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kBlock), 0, stream, d_in, n_max, d_n, sums);
         FGL_CHECK_LAUNCH("scan_tile_sums_kernel");
     }
-    if (tiles > kSelfPrefixTiles) {
+    if (tiles > kScanSelfPrefixTiles) {
         int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_total_extra, nullptr, nullptr, 0, nullptr, 0, stream);
         if (rc != FGL_OK) return rc;
     } else {
