@@ -33,6 +33,7 @@ class Block:
         self._dst_local = None
         self._transposed = None
         self._src_deg = None
+        self._in_deg = None
 
     # -- the part of the DGLBlock interface that the reference's model code uses -------------
     def num_src_nodes(self):
@@ -62,7 +63,9 @@ class Block:
 
     # -- what this library adds ---------------------------------------------------------
     def in_degrees(self):
-        return self.edge_ptr[1:] - self.edge_ptr[:-1]
+        if self._in_deg is None:
+            self._in_deg = self.edge_ptr[1:] - self.edge_ptr[:-1]
+        return self._in_deg
 
     def out_degrees(self):
         if self._src_deg is None:
