@@ -222,6 +222,9 @@ def main():
     ap.add_argument("--cpu-batches", type=int, default=128, help="mini-batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--id-order", default="first", choices=["first", "arrival"],
                     help="numbering of new node ids: first occurrence (deterministic, default) or arrival (the reference's rule)")
+    ap.add_argument("--readback", choices=["hidden", "first"], default="hidden",
+                    help="hidden: enqueue the outermost aggregation before waiting for the batch's sizes (default); "
+                         "first: read the sizes back right after sampling, as sample_blocks() does")
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
@@ -316,11 +319,25 @@ def main():
         seeds = train[(i % n_batches) * B:(i % n_batches) * B + B]
         e0, e1, e2, e3, e4 = ev(), ev(), ev(), ev(), ev()
         e0.record()
-        input_nodes, _, blocks = sampler.sample_blocks(None, seeds)  # includes the one count read-back
-        e1.record()
-        b0 = blocks[0]
-        out0 = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
-        e2.record()
+        if args.readback == "hidden":
+            # the outermost aggregation is enqueued on the bound-sized block with its row count on the device,
+            # and the host's wait for the batch's sizes hides behind it
+            pend = sampler.begin_sample(seeds)
+            e1.record()
+            out0 = fastgl.aggregate(pend.outer_edge_ptr, pend.outer_src_global, feat, mode="mean", zero_policy="zeros",
+                                    n_rows=pend.outer_n_dst_bound, n_rows_dev=pend.outer_n_dst, longest_row=pend.outer_fanout)
+            e2.record()
+            input_nodes, _, blocks = pend.finish()
+            b0 = blocks[0]
+            if pend.redone:  # the batch outgrew its buffers and was sampled again: aggregate again
+                out0 = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
+            out0 = out0[:b0.num_dst_nodes()]
+        else:
+            input_nodes, _, blocks = sampler.sample_blocks(None, seeds)  # includes the one count read-back
+            e1.record()
+            b0 = blocks[0]
+            out0 = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
+            e2.record()
         outs = [out0]
         hid, grad = inner_buffers(max([b.num_src_nodes() for b in blocks[1:]] + [1]))
         for b in blocks[1:]:
@@ -528,7 +545,10 @@ def main():
         "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
                    "sampled_edges_per_step": tot_edges / K, "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
                    "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
-                           "feature table); block transpose + bwd gather on the inner blocks; no dense layers"},
+                           "feature table); block transpose + bwd gather on the inner blocks; no dense layers",
+                   "readback": ("the batch's sizes reach the host on a second stream while the outermost aggregation runs "
+                                "(sample_idmap = the sampling kernels' own time)") if args.readback == "hidden" else
+                               "the batch's sizes are read back before anything else is enqueued (inside sample_idmap)"},
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
                       "transpose_agg_bwd_inner": t_bwd / K},
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,

@@ -28,7 +28,7 @@ from .ops import (  # noqa: F401
     table_size,
     transfer_edge_id,
 )
-from .sampler import Block, FusedMapSampler  # noqa: F401
+from .sampler import Block, FusedMapSampler, PendingBatch  # noqa: F401
 from .conv import (  # noqa: F401
     GAT,
     GCN,

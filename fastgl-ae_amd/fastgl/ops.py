@@ -286,7 +286,7 @@ _ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
 
 
 def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
-              out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None):
+              out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None, n_rows_dev=None):
     """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
     accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge;
     ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``.
@@ -295,7 +295,9 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     of hundreds of entries get a second launch that a bound can save.  When not given it is taken from the
     ``fgl_longest_row`` attribute that ``block_transpose`` and the sampler attach to their ``indptr`` tensors.
     ``mode="edge"``: ``edge_weight`` float32 [n_entries, n_heads], weight of entry e for column f is
-    ``edge_weight[edge_index[e] if edge_index is not None else e, f // (D // n_heads)]``."""
+    ``edge_weight[edge_index[e] if edge_index is not None else e, f // (D // n_heads)]``.
+    ``n_rows_dev``: one-element int32 device tensor with the actual row count when the host only knows the
+    bound ``n_rows`` (a block whose sizes have not been read back yet): rows past it are left unwritten."""
     _check_input(indptr, "indptr", _I32)
     _check_input(indices, "indices", _I32)
     if not isinstance(feat, torch.Tensor) or not feat.is_cuda:
@@ -328,7 +330,11 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
         longest_dev = longest_row
     elif longest_row is not None:
         longest_host = int(longest_row)
-    dev = _same_device(indptr, indices, feat, row_norm, col_norm, edge_weight, edge_index, longest_dev)
+    if n_rows_dev is not None:
+        _check_input(n_rows_dev, "n_rows_dev", _I32)
+        if n_rows_dev.numel() != 1:
+            raise RuntimeError("n_rows_dev must hold one int32")
+    dev = _same_device(indptr, indices, feat, row_norm, col_norm, edge_weight, edge_index, longest_dev, n_rows_dev)
     n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
     if n < 0 or n > indptr.numel() - 1:
         raise RuntimeError("n_rows (%d) does not match indptr (%d entries)" % (n, indptr.numel()))
@@ -345,7 +351,7 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
         if n > 0:
             # a block without entries has no index array to point at; the kernel then reads none
             idx_ptr = L.ptr(indices) if indices.numel() else L.ptr(indptr)
-            L.check(L.lib().fgl_aggregate(L.ptr(indptr), idx_ptr, n, None, L.ptr(feat), int(feat.stride(0)), D,
+            L.check(L.lib().fgl_aggregate(L.ptr(indptr), idx_ptr, n, L.ptr(n_rows_dev), L.ptr(feat), int(feat.stride(0)), D,
                                           L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
                                           L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index),
                                           longest_host, L.ptr(longest_dev), L.ptr(out), int(out.stride(0)),

@@ -94,6 +94,45 @@ class Block:
         return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())
 
 
+class PendingBatch:
+    """A mini-batch whose kernels are enqueued and whose sizes are still on the device
+    (``FusedMapSampler.begin_sample``).  The sizes travel to a pinned host buffer on a second stream as soon as
+    the sampling kernels are done, whatever the caller enqueues behind them in the meantime."""
+
+    def __init__(self, sampler, pending):
+        self._sampler, self._pending = sampler, pending
+        _, bptr, _, src_g, counts = pending["out"]
+        H = len(sampler.fanouts)
+        self.outer_edge_ptr = bptr[H - 1]        # int32[bound + 1]: row offsets of the outermost block
+        self.outer_src_global = src_g[H - 1]     # int32[edge bound]: its neighbour lists in graph ids
+        self.outer_n_dst = counts[H - 1:H]       # int32[1] on the device: its actual row count
+        self.outer_n_dst_bound = int(bptr[H - 1].numel()) - 1
+        self.outer_fanout = int(sampler.fanouts[0])
+        self.redone = False
+        dev = counts.device
+        main = torch.cuda.current_stream(dev)
+        side = sampler._side_stream(dev)
+        sampled = torch.cuda.Event()
+        sampled.record(main)
+        side.wait_event(sampled)
+        self._host = torch.empty(counts.numel(), dtype=torch.int32, pin_memory=True)
+        with torch.cuda.stream(side):
+            self._host.copy_(counts, non_blocking=True)
+            self._arrived = torch.cuda.Event()
+            self._arrived.record(side)
+
+    def finish(self):
+        """The second half: wait for the sizes, then ``(input_nodes, output_nodes, blocks)`` as ``sample_blocks``
+        returns them.  ``redone`` is set if the batch outgrew its buffers and was sampled again with larger
+        ones -- anything computed from the ``outer_*`` arrays before is then void (it read valid memory, the
+        kernels never leave their bounds)."""
+        outer_ptr = self.outer_edge_ptr.data_ptr()
+        self._arrived.synchronize()
+        result = self._sampler._finish_fused(self._pending, self._host.tolist())
+        self.redone = result[2][0].edge_ptr.data_ptr() != outer_ptr
+        return result
+
+
 class FusedMapSampler:
     def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
                  prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0,
@@ -266,9 +305,29 @@ class FusedMapSampler:
                                    None if src_g[h] is None else src_g[h][:n_e], sorted_transpose=self.deterministic))
         return uniq[:c[H]], pending["seeds"], blocks
 
+    def begin_sample(self, seed_nodes):
+        """First half of ``sample_blocks`` (fused path): enqueue every hop and return at once, without the host
+        read-back.  The ``PendingBatch`` exposes the outermost block with bound-sized arrays and its row count on
+        the device, so that the first layer's aggregation -- the largest kernel of a step -- can be enqueued
+        before ``finish()`` waits for the sizes; the host's wake-up then hides behind that kernel."""
+        if not self.fused:
+            raise RuntimeError("begin_sample needs the fused path")
+        if self.edge_ptr is None or self.edge_src is None:
+            raise RuntimeError("FusedMapSampler: edge_ptr / edge_src are not set")
+        self.output_nodes = seed_nodes
+        seeds = seed_nodes.to(device=self.edge_src.device, dtype=torch.int32).contiguous()
+        stream_base = (self.batches * 64) & 0xFFFFFFFF
+        self.batches += 1
+        return PendingBatch(self, self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel()))))
+
     def _sample_fused(self, seeds, stream_base):
         pending = self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel())))
         return self._finish_fused(pending, pending["out"][4].tolist())  # the one host synchronisation of the mini-batch
+
+    def _side_stream(self, dev):
+        if self._side is None:
+            self._side = torch.cuda.Stream(device=dev)  # default priority
+        return self._side
 
     def iter_batches(self, seed_batches):
         """Yields ``(input_nodes, output_nodes, blocks)`` for every seed batch, sampling batch i+1 on
@@ -281,9 +340,7 @@ class FusedMapSampler:
             return
         dev = self.edge_src.device
         main = torch.cuda.current_stream(dev)
-        if self._side is None:
-            self._side = torch.cuda.Stream(device=dev)  # default priority
-        side = self._side
+        side = self._side_stream(dev)
         H = len(self.fanouts)
 
         def launch(seed_nodes):

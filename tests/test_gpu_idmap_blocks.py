@@ -137,6 +137,39 @@ def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     check_blocks(oracle, indptr, indices, seeds, [4, 4], got, 1, 0)
 
 
+def test_begin_sample_then_finish(cuda, oracle, small_graph):
+    """The two-phase form of sample_blocks: the outermost block is usable (bound-sized, row count on the
+    device) before the sizes are read back; finish() then returns exactly what sample_blocks returns.  A batch
+    that outgrows its buffers is redone inside finish() and says so."""
+    import fastgl
+    print("begin_sample / finish", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    n = indptr.size - 1
+    feat = torch.randn(n, 24, device=cuda)
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=4).set_graph(ptr, idx)
+    rng = np.random.default_rng(2)
+    for batch in range(3):  # first batch: worst-case buffers; then sized by experience
+        seeds = rng.permutation(n)[:700].astype(np.int32)
+        pend = sampler.begin_sample(dev_i32(seeds, cuda))
+        early = fastgl.aggregate(pend.outer_edge_ptr, pend.outer_src_global, feat, mode="mean", zero_policy="zeros",
+                                 n_rows=pend.outer_n_dst_bound, n_rows_dev=pend.outer_n_dst, longest_row=pend.outer_fanout)
+        got = pend.finish()
+        assert not pend.redone
+        check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], got, 4, 64 * batch)
+        b0 = got[2][0]
+        late = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
+        assert torch.equal(early[:b0.num_dst_nodes()], late)
+    sampler._nodes_seen = [700, 800, 900, 1000]                             # (pretend the batches stayed tiny)
+    hubs = np.argsort(-np.diff(indptr))[:700].astype(np.int32)
+    pend = sampler.begin_sample(dev_i32(hubs, cuda))
+    fastgl.aggregate(pend.outer_edge_ptr, pend.outer_src_global, feat, mode="mean", zero_policy="zeros",
+                     n_rows=pend.outer_n_dst_bound, n_rows_dev=pend.outer_n_dst)  # on an overflowed batch: stays in bounds
+    got = pend.finish()
+    assert pend.redone
+    check_blocks(oracle, indptr, indices, hubs, [15, 10, 5], got, 4, 64 * 3)
+
+
 def test_undersized_buffers_are_detected_and_redone(cuda, oracle, small_graph):
     """The sampler sizes its hash table and output buffers from earlier batches; a batch that outgrows
     them must be caught by the kernels (status word) and repeated with the worst-case plan, same result."""
