@@ -103,6 +103,10 @@ def test_sampler_front_end_without_gpu():
             fastgl.FusedMapSampler([5], graph_slots=bad)
     with pytest.raises(ValueError):
         fastgl.FusedMapSampler([5], id_order="arrival", deterministic=True)
+    with pytest.raises(RuntimeError, match="fused"):
+        fastgl.FusedMapSampler([5], fused=False).begin_sample(torch.arange(4))
+    with pytest.raises(RuntimeError, match="not set"):
+        fastgl.FusedMapSampler([5]).begin_sample(torch.arange(4))
 
 
 def test_missing_library_fails_loudly(monkeypatch):
