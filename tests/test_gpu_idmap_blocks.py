@@ -364,3 +364,48 @@ def test_random_configurations_against_the_oracle(cuda, oracle):
         for batch in range(3):
             got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
             check_blocks(oracle, indptr, indices, seeds, fanouts, got, rng_seed, batch * 64)
+
+
+@pytest.mark.parametrize("n_edges", [5000, 2_200_000])
+def test_final_call_leaves_the_table_alone_and_the_results_unchanged(cuda, oracle, n_edges):
+    """FGL_IDMAP_FINAL (the caller will not consult the table again): same relabelled edges, same unique list,
+    same count as without it -- on both sides of the tile count where the number pass changes form -- and the new
+    ids' slots keep their transient value, so a later lookup of a new id reports it (top bit set = not a local id)."""
+    import ctypes as C
+    import fastgl
+    from fastgl import _lib as L
+    print("idmap final n_edges=%d" % n_edges, flush=True)
+    rng = np.random.default_rng(n_edges)
+    n_dst = 300
+    dst_unique = rng.choice(10**6, size=n_dst, replace=False).astype(np.int32)
+    src = rng.integers(0, 3 * 10**6, size=n_edges).astype(np.int32)
+    src[::5] = dst_unique[rng.integers(0, n_dst, size=src[::5].size)]     # ids that are numbered already
+    lib = fastgl.lib()
+    capacity = n_dst + n_edges
+    slots = lib.fgl_idmap_slots(capacity)
+    results = []
+    for flags in (L.IDMAP_ORDERED, L.IDMAP_ORDERED | L.IDMAP_FINAL):
+        table = torch.empty(slots, dtype=torch.int64, device=cuda)
+        uniq = torch.empty(capacity, dtype=torch.int32, device=cuda)
+        meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+        d_src, d_out = dev_i32(src, cuda), torch.empty(n_edges, dtype=torch.int32, device=cuda)
+        ws = torch.empty(lib.fgl_idmap_map_src_workspace_bytes(n_edges), dtype=torch.uint8, device=cuda)
+        st = L.stream_handle()
+        L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+        L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dev_i32(dst_unique, cuda)), n_dst, None, L.ptr(uniq),
+                                         meta.data_ptr() + 4, st))
+        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(d_src), L.ptr(d_out), n_edges, None, n_dst, None,
+                                      meta.data_ptr(), L.ptr(uniq), capacity, flags, meta.data_ptr() + 4, L.ptr(ws), ws.numel(), st))
+        n_total, status = meta.tolist()
+        assert status == 0
+        probe = d_src.clone()
+        L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), n_edges, None, meta.data_ptr() + 4, st))
+        results.append((d_out.cpu().numpy(), uniq[:n_total].cpu().numpy(), probe.cpu().numpy()))
+    (out_a, uniq_a, look_a), (out_b, uniq_b, look_b) = results
+    ws_, _, wu = oracle.idmap(src, np.zeros(n_edges, np.int32) + dst_unique[0], dst_unique)
+    assert np.array_equal(out_a, ws_) and np.array_equal(uniq_a, wu)
+    assert np.array_equal(out_b, out_a) and np.array_equal(uniq_b, uniq_a)
+    assert np.array_equal(look_a, out_a)                      # written back: the table answers for every id
+    new = out_a >= n_dst
+    assert np.array_equal(look_b[~new], out_a[~new])          # ids numbered before the call: unchanged
+    assert (look_b[new] < 0).all()                            # new ids: still the transient value (top bit set)
