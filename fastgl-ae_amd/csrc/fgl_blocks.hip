@@ -176,7 +176,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
                                   d_counts + h + 1, d_uniq, grow_to,
                                   idmap_flags | (h == n_hops - 1 ? FGL_IDMAP_FINAL : 0), d_status, ws + ws_sample,
-                                  ws_bytes - ws_sample, s);
+                                  ws_bytes - ws_sample, s, /*counter_is_zeroed=*/true);
         if (rc != FGL_OK) return rc;
     }
     return FGL_OK;

@@ -335,57 +335,104 @@ __global__ __launch_bounds__(kBlock) void idmap_lookup_kernel(TableRef t, int32_
 // ---- arrival-order numbering (FGL_IDMAP_ARRIVAL) ---------------------------------------
 // The lane whose CAS installs a key numbers it at once from a global counter, as the
 // reference does (id_map.cu:314-321) -- but with one counter update per workgroup instead
-// of one per new id.  Fewer launches and about half the table traffic (though the two barriers
-// per round cost about what that saves); the numbering of new ids then depends on scheduling (any run is a valid map, and equal to
-// every other after sorting the new ids).
-__global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t, const int32_t* __restrict__ src,
+// of one per new id -- and relabels its edge on the spot; so does every lane that finds its id
+// already numbered (a destination, an id of an earlier hop, or a new id whose number has landed).
+// Only the lanes that meet a key between its install and its number (val still all ones) leave
+// their edge to the second, short pass.  Two passes over the edges, one table access per edge in
+// most cases; the numbering of new ids depends on scheduling (any run is a valid map, and equal
+// to every other after sorting the new ids).  `src` and `out` may be the same array.
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t, const int32_t* src,
                                                                       int64_t e_max, const int32_t* __restrict__ d_e,
                                                                       int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                       uint32_t* __restrict__ slot_of, int32_t* __restrict__ counter,
-                                                                      int32_t* __restrict__ uniq, int64_t capacity,
+                                                                      int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
                                                                       uint32_t* __restrict__ d_status)
 {
     __shared__ int smem[kBlock / kWave + 1];
     __shared__ int s_base;
+    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    const int64_t rounds = (n_e + stride - 1) / stride;  // same trip count for every lane: the loop holds barriers
-    for (int64_t r = 0; r < rounds; ++r) {
-        const int64_t e = r * stride + (int64_t)blockIdx.x * kBlock + threadIdx.x;
-        uint32_t p = kEmpty, id = 0;
-        int won = 0;
-        if (e < n_e) {
-            id = (uint32_t)src[e];
-            uint32_t q = (id * kHashMul) >> t.shift;
-            const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
-            for (uint32_t n = 0; n < limit; ++n) {
-                uint32_t k = t.words[2 * (size_t)q];
-                if (k == kEmpty) {
-                    const uint32_t seen = atomicCAS(&t.words[2 * (size_t)q], kEmpty, id);
-                    if (seen == kEmpty) { won = 1; k = id; } else k = seen;
+    constexpr int kEdges = kBlock * ITEMS;
+    const int64_t n_tiles = (n_e + kEdges - 1) / kEdges;
+    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
+    // A workgroup takes a tile of 256 * ITEMS edges at a time, ITEMS per lane (edge = tile start + j * 256 + lane).
+    // ITEMS = 8 for large inputs: one update of the global counter per 2048 edges -- updates of one address run one
+    // after the other, and one per 256 edges costs more than the probing (1.5 M edges: 100 -> 69 us) -- and eight
+    // independent probe sequences in flight per lane; ITEMS = 1 for small inputs, which need the workgroups.
+    // (The trip count is the same for every lane of the workgroup: the loop holds barriers.)
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t first = tile * kEdges + threadIdx.x;
+        // p: kDone = the edge is relabelled; a slot = its id is being numbered, see the second pass; kEmpty = table full
+        uint32_t p[ITEMS], id[ITEMS];
+        uint32_t won = 0;
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int64_t e = first + (int64_t)j * kBlock;
+            p[j] = kDone;
+            id[j] = 0;
+            if (e < n_e) {
+                id[j] = (uint32_t)src[e];
+                p[j] = kEmpty;
+                uint32_t q = (id[j] * kHashMul) >> t.shift;
+                for (uint32_t n = 0; n < limit; ++n) {
+                    unsigned long long slot = slots[q];
+                    if ((uint32_t)slot == kEmpty) {
+                        // the key goes in with val still all ones = "not numbered yet"
+                        const unsigned long long seen = atomicCAS(&slots[q], ~0ull, (unsigned long long)id[j] | 0xFFFFFFFF00000000ull);
+                        if (seen == ~0ull) {
+                            won |= 1u << j;
+                            p[j] = q;
+                            break;
+                        }
+                        slot = seen;
+                    }
+                    if ((uint32_t)slot == id[j]) {
+                        const uint32_t v = (uint32_t)(slot >> 32);
+                        if (v & 0x80000000u) {
+                            p[j] = q;
+                        } else {
+                            out[e] = (int32_t)v;
+                            p[j] = kDone;
+                        }
+                        break;
+                    }
+                    q = (q + 1) & t.mask;
                 }
-                if (k == id) { p = q; break; }
-                q = (q + 1) & t.mask;
+                if (p[j] == kEmpty) {
+                    out[e] = -1;
+                    if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+                }
             }
-            slot_of[e] = p;
-            if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
         }
         int total;
-        const int rank = block_exclusive_scan<kBlock>(won, smem, &total);
+        int rank = block_exclusive_scan<kBlock>(__popc(won), smem, &total);
         if (threadIdx.x == 0) s_base = total ? atomicAdd(counter, total) : 0;
         __syncthreads();
-        if (won) {
-            const int64_t local = n_base + s_base + rank;
-            if (local < capacity) {
-                t.words[2 * (size_t)p + 1] = (uint32_t)local;
-                uniq[local] = (int32_t)id;
+        const int64_t base = n_base + s_base;
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int64_t e = first + (int64_t)j * kBlock;
+            if ((won >> j) & 1u) {
+                const int64_t local = base + rank++;
+                if (local < capacity) {
+                    t.words[2 * (size_t)p[j] + 1] = (uint32_t)local;
+                    uniq[local] = (int32_t)id[j];
+                    out[e] = (int32_t)local;
+                } else {
+                    out[e] = -1;  // the unique list is full (reported by the second pass); val stays "not numbered"
+                }
+                p[j] = kDone;
             }
+            if (e < n_e) slot_of[e] = p[j];
         }
         __syncthreads();
     }
 }
 
+// Second pass of the arrival-order numbering: the edges whose id was between install and number when
+// their lane met it read the number now; also publishes the node total.
 __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
                                                                        const uint32_t* __restrict__ slot_of,
                                                                        int32_t* __restrict__ out, const int32_t* __restrict__ counter,
@@ -397,18 +444,18 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
-        out[e] = p == kEmpty ? -1 : (int32_t)t.words[2 * (size_t)p + 1];
+        if (p >= kDone) continue;  // relabelled by the first pass (kDone) or reported there (kEmpty)
+        const uint32_t v = t.words[2 * (size_t)p + 1];
+        out[e] = (v & 0x80000000u) ? -1 : (int32_t)v;  // (still unnumbered: the unique list was full)
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-        int64_t total = n_base + (int64_t)(*counter);
-        if (total > capacity) {
-            if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
-            total = capacity;
-        }
-        if (d_n_total_out) *d_n_total_out = (int32_t)total;
+        publish_node_total(n_base, *counter, capacity, d_n_total_out, d_status);
     }
 }
+
+// Inputs up to this many edges number their new ids one edge per lane (see idmap_insert_arrival_kernel).
+constexpr int64_t kArrivalSmallEdges = 1 << 18;
 
 // Workgroups for a grid-stride pass over n items: enough to fill every CU several times
 // over, never more than the work needs.
@@ -457,7 +504,7 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
 int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out, int64_t n_edges_max,
                          const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base, int32_t* d_n_total_out,
                          int32_t* d_uniq, int64_t uniq_capacity, int flags, uint32_t* d_status, void* d_ws,
-                         size_t ws_bytes, hipStream_t stream)
+                         size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
@@ -484,11 +531,22 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
 
     if (flags & FGL_IDMAP_ARRIVAL) {
-        int32_t* counter = sums;  // one int of the (otherwise unused) tile-sum array
-        int rc0 = launch_fill_u32(reinterpret_cast<uint32_t*>(counter), 1, 0u, stream);
-        if (rc0 != FGL_OK) return rc0;
-        hipLaunchKernelGGL(idmap_insert_arrival_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in, n_edges_max,
-                           d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_status);
+        // the counter of new ids: *d_n_total_out itself when the caller vouches that it holds zero (the all-hops
+        // entry point zeroes its counts when it resets the table), else one int of the (otherwise unused)
+        // tile-sum array, zeroed by a launch of its own
+        int32_t* counter = (counter_is_zeroed && d_n_total_out) ? d_n_total_out : sums;
+        if (counter == sums) {
+            int rc0 = launch_fill_u32(reinterpret_cast<uint32_t*>(counter), 1, 0u, stream);
+            if (rc0 != FGL_OK) return rc0;
+        }
+        if (n_edges_max > kArrivalSmallEdges)
+            hipLaunchKernelGGL(idmap_insert_arrival_kernel<kItems>, dim3(tile_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+                               n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
+                               d_status);
+        else
+            hipLaunchKernelGGL(idmap_insert_arrival_kernel<1>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+                               n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
+                               d_status);
         FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
         hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
                            slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
@@ -563,7 +621,7 @@ FGL_EXPORT int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_
                                  uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream)
 {
     return launch_idmap_map_src(d_table, slots, d_src_in, d_src_out, n_edges_max, d_n_edges, n_base, d_n_base,
-                                d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream));
+                                d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream), false);
 }
 
 FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,

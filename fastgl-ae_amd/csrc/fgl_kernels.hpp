@@ -32,7 +32,8 @@ int launch_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_i
 int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
                          int64_t n_edges_max, const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base,
                          int32_t* d_n_total_out, int32_t* d_uniq, int64_t uniq_capacity, int flags,
-                         uint32_t* d_status, void* d_ws, size_t ws_bytes, hipStream_t stream);
+                         uint32_t* d_status, void* d_ws, size_t ws_bytes, hipStream_t stream,
+                         bool counter_is_zeroed = false);  // arrival order: *d_n_total_out holds zero and may count the new ids
 
 // deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
 size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);

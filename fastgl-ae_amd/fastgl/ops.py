@@ -449,7 +449,8 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     ``table_slots`` (a power of two, default the plan's worst case) uses only that much of the
     hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL).
     ``id_order``: ``"first"`` numbers new ids by first occurrence (deterministic), ``"arrival"`` as
-    their inserts land (the reference's rule; any run is a valid map, equal to every other after sorting the new ids).
+    their inserts land (the reference's rule, and about a tenth faster; any run is a valid map, equal to every other after
+    sorting the new ids).
     ``stream_offset``: one-element int32 device tensor added to ``stream_base`` when the kernels run (for
     callers that capture this call in a graph and advance the random stream between replays)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)

@@ -67,7 +67,8 @@ enum fgl_zero_policy {
 
 #define FGL_IDMAP_ORDERED 0 /* new ids numbered by first occurrence (deterministic) */
 #define FGL_IDMAP_ARRIVAL 1 /* new ids numbered as their inserts land (the reference's rule,
-                               id_map.cu:314-321): fewer passes, order depends on scheduling */
+                               id_map.cu:314-321): two passes instead of three or four and about a
+                               tenth faster; the order of the new ids depends on scheduling */
 #define FGL_IDMAP_FINAL 2   /* (or'ed in) the table is not consulted after this call: the local ids of the
                                new ids go to the edges and the unique list, not back into the table */
 #define FGL_MAX_FANOUT 192

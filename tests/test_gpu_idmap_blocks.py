@@ -409,3 +409,49 @@ def test_final_call_leaves_the_table_alone_and_the_results_unchanged(cuda, oracl
     new = out_a >= n_dst
     assert np.array_equal(look_b[~new], out_a[~new])          # ids numbered before the call: unchanged
     assert (look_b[new] < 0).all()                            # new ids: still the transient value (top bit set)
+
+
+@pytest.mark.parametrize("n_edges", [5000, 262_144, 262_145, 900_000])
+def test_arrival_order_through_the_c_abi(cuda, oracle, n_edges):
+    """FGL_IDMAP_ARRIVAL (the reference's numbering rule) on both sides of the size where its insert pass changes
+    from one edge per lane to eight: the order-free characterisation of a correct map -- destinations keep their
+    positions, no id twice, the new ids are exactly the sources that are not destinations, every edge points at
+    its own id -- and equality with the oracle after sorting the new ids.  In place (src_out = src_in)."""
+    import fastgl
+    from fastgl import _lib as L
+    print("idmap arrival n_edges=%d" % n_edges, flush=True)
+    rng = np.random.default_rng(n_edges + 1)
+    n_dst = 500
+    dst_unique = rng.choice(10**6, size=n_dst, replace=False).astype(np.int32)
+    src = ((rng.pareto(1.1, size=n_edges) * 40).astype(np.int64) % (2 * 10**6)).astype(np.int32)   # hot ids repeat a lot
+    src[::6] = dst_unique[rng.integers(0, n_dst, size=src[::6].size)]
+    lib = fastgl.lib()
+    capacity = n_dst + n_edges
+    slots = lib.fgl_idmap_slots(capacity)
+    table = torch.empty(slots, dtype=torch.int64, device=cuda)
+    uniq = torch.empty(capacity, dtype=torch.int32, device=cuda)
+    meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+    d_src = dev_i32(src, cuda)
+    ws = torch.empty(lib.fgl_idmap_map_src_workspace_bytes(n_edges), dtype=torch.uint8, device=cuda)
+    st = L.stream_handle()
+    L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+    L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dev_i32(dst_unique, cuda)), n_dst, None, L.ptr(uniq),
+                                     meta.data_ptr() + 4, st))
+    L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(d_src), L.ptr(d_src), n_edges, None, n_dst, None,
+                                  meta.data_ptr(), L.ptr(uniq), capacity, L.IDMAP_ARRIVAL, meta.data_ptr() + 4, L.ptr(ws),
+                                  ws.numel(), st))
+    n_total, status = meta.tolist()
+    assert status == 0
+    out, u = d_src.cpu().numpy(), uniq[:n_total].cpu().numpy()
+    assert np.array_equal(u[:n_dst], dst_unique)
+    assert np.unique(u).size == u.size
+    assert set(u[n_dst:].tolist()) == set(src.tolist()) - set(dst_unique.tolist())
+    assert out.min() >= 0 and out.max() < n_total and np.array_equal(u[out], src)
+    ws_, _, wu = oracle.idmap(src, np.zeros(n_edges, np.int32) + dst_unique[0], dst_unique)
+    cs, cu = canonical(out, u, n_dst, None)
+    cws, cwu = canonical(ws_, wu, n_dst, None)
+    assert np.array_equal(cs, cws) and np.array_equal(cu, cwu)
+    # the table answers for every id afterwards (arrival order always writes the numbers back)
+    probe = dev_i32(src, cuda)
+    L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), n_edges, None, meta.data_ptr() + 4, st))
+    assert np.array_equal(probe.cpu().numpy(), out)
