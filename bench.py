@@ -315,7 +315,7 @@ def main():
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
 
-    def step(i, rec=None):
+    def step(i, rec=None, sampler=sampler):
         seeds = train[(i % n_batches) * B:(i % n_batches) * B + B]
         e0, e1, e2, e3, e4 = ev(), ev(), ev(), ev(), ev()
         e0.record()
@@ -364,6 +364,26 @@ def main():
         last_blocks = step(args.warmup + i, rec)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
+
+    # ---- the same steps with the other numbering rule of the id-map (context for `value`) ----------------
+    other_order = "arrival" if args.id_order == "first" else "first"
+    value_other = None
+    if sampler_mode == "eager":
+        keep_main = list(keep)
+        alt = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=other_order).set_graph(edge_ptr, edge_src)
+        for i in range(args.warmup):
+            step(i, None, alt)
+        torch.cuda.synchronize()
+        rec_alt = []
+        for i in range(args.steps):
+            step(args.warmup + i, rec_alt, alt)
+        torch.cuda.synchronize()
+        keep[:] = keep_main  # (the replay below uses the main run's blocks)
+        alt_edges = sum(r[0][0] for r in rec_alt)
+        alt_ms = sum(r[1][0].elapsed_time(r[1][1]) for r in rec_alt)
+        value_other = alt_edges / (alt_ms * 1e-3)
+        log("id order %s: %.3g sampled edges/s (sample+idmap %.3f ms)" % (other_order, value_other, alt_ms / args.steps))
+        del alt, rec_alt
 
     # ---- optional: the same steps with sampling of batch i+1 overlapped with aggregation of batch i ----
     ms_overlapped = None
@@ -555,6 +575,7 @@ def main():
                         "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
         "random_read_Gps": random_read_gps,
         "value_eager_launch": value_eager,
+        "value_other_id_order": {"id_order": other_order, "value": value_other},
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
