@@ -225,6 +225,8 @@ def main():
     ap.add_argument("--readback", choices=["hidden", "first"], default="hidden",
                     help="hidden: enqueue the outermost aggregation before waiting for the batch's sizes (default); "
                          "first: read the sizes back right after sampling, as sample_blocks() does")
+    ap.add_argument("--other-order", choices=["on", "off"], default="on",
+                    help="also time the steps with the other numbering rule of the id-map (value_other_id_order)")
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
@@ -368,7 +370,7 @@ def main():
     # ---- the same steps with the other numbering rule of the id-map (context for `value`) ----------------
     other_order = "arrival" if args.id_order == "first" else "first"
     value_other = None
-    if sampler_mode == "eager":
+    if sampler_mode == "eager" and args.other_order == "on":
         keep_main = list(keep)
         alt = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=other_order).set_graph(edge_ptr, edge_src)
         for i in range(args.warmup):
