@@ -358,9 +358,9 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
     const int64_t n_tiles = (n_e + kEdges - 1) / kEdges;
     const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
     // A workgroup takes a tile of 256 * ITEMS edges at a time, ITEMS per lane (edge = tile start + j * 256 + lane).
-    // ITEMS = 8 for large inputs: one update of the global counter per 2048 edges -- updates of one address run one
-    // after the other, and one per 256 edges costs more than the probing (1.5 M edges: 100 -> 69 us) -- and eight
-    // independent probe sequences in flight per lane; ITEMS = 1 for small inputs, which need the workgroups.
+    // Several edges per lane for large inputs: one update of the global counter per tile -- updates of one address
+    // run one after the other, and one per 256 edges costs more than the probing -- against the length of a
+    // lane's chain of probes; one edge per lane for small inputs, which need the workgroups.
     // (The trip count is the same for every lane of the workgroup: the loop holds barriers.)
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t first = tile * kEdges + threadIdx.x;
@@ -456,6 +456,7 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
 
 // Inputs up to this many edges number their new ids one edge per lane (see idmap_insert_arrival_kernel).
 constexpr int64_t kArrivalSmallEdges = 1 << 18;
+constexpr int kArrivalItems = 4;  // edges per lane for large inputs (measured on a 1.5 M-edge hop: 8 -> 69 us, 4 -> 62 us, 2 -> 66 us, 1 -> 100 us)
 
 // Workgroups for a grid-stride pass over n items: enough to fill every CU several times
 // over, never more than the work needs.
@@ -540,7 +541,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
             if (rc0 != FGL_OK) return rc0;
         }
         if (n_edges_max > kArrivalSmallEdges)
-            hipLaunchKernelGGL(idmap_insert_arrival_kernel<kItems>, dim3(tile_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+            hipLaunchKernelGGL(idmap_insert_arrival_kernel<kArrivalItems>, dim3(stride_grid(n_edges_max, kBlock * kArrivalItems)),
+                               dim3(kBlock), 0, stream, t, d_src_in,
                                n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
                                d_status);
         else
