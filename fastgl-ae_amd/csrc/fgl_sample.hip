@@ -15,10 +15,47 @@
 //                             `indices` contiguously.
 // Launches 1 and 3 are grid-stride loops over the tiles the actual seed count occupies, so
 // a host-side bound far above the actual count costs nothing.
+#include <mutex>
+
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
+// Scratch of fgl_sample_node_static: device memory that belongs to the library, one copy per GPU, held
+// until the process ends.  In host code this name is only a handle for hipGetSymbolAddress -- it is
+// not a device address and is never passed to a kernel or a memset; static_scratch() below resolves
+// it once per device and everything else uses the pointer it returns.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace fgl {
+
+constexpr int64_t kStaticMaxSeeds = (int64_t)1 << 20;  // 12.2 bytes of scratch per seed at most: fits 16 MiB
+constexpr int kStaticMaxDevices = 64;
+
+// The calling thread's current device's copy of `scratch` (each GPU holds its own at its own address).
+static int static_scratch(void** out)
+{
+    static std::mutex mu;
+    static void* ptr_of_device[kStaticMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) {
+        set_error("sample_node_static: cannot name the current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return FGL_ERR_HIP;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of_device[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            set_error("sample_node_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return FGL_ERR_HIP;
+        }
+        ptr_of_device[dev] = p;
+    }
+    *out = ptr_of_device[dev];
+    return FGL_OK;
+}
 
 template <int TS>
 __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restrict__ indptr, int is64, int64_t n_nodes,
@@ -378,5 +415,26 @@ FGL_EXPORT int fgl_sample_node(const void* d_indptr, int indptr_is64, const int3
 {
     return launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, rng_seed,
                          stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws, ws_bytes,
+                         as_stream(stream));
+}
+
+FGL_EXPORT int fgl_sample_node_static(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                                      const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                                      uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
+                                      int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* stream)
+{
+    FGL_REQUIRE(n_seeds_max >= 0 && n_seeds_max <= kStaticMaxSeeds,
+                "sample_node_static: %lld seeds outside [0, %lld] (the library's own scratch holds no more; "
+                "use fgl_sample_node with a caller workspace)", (long long)n_seeds_max, (long long)kStaticMaxSeeds);
+    FGL_REQUIRE(fanout >= 1 && fanout <= FGL_MAX_FANOUT, "sample_node_static: fanout %d outside [1, %d]", fanout, FGL_MAX_FANOUT);
+    const size_t need = sample_workspace_bytes(n_seeds_max, fanout);
+    FGL_REQUIRE(need <= kStaticScratchBytes, "sample_node_static: needs %zu bytes of scratch, the library holds %zu", need,
+                kStaticScratchBytes);
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != FGL_OK) return rc;
+    // (nothing in the scratch has to start at zero: the degree pass writes every entry the edges pass reads)
+    return launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, rng_seed,
+                         stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, ws, kStaticScratchBytes,
                          as_stream(stream));
 }

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 4
+#define FGL_ABI_VERSION 5
 
 enum fgl_error {
     FGL_OK = 0,
@@ -108,6 +108,22 @@ int fgl_sample_node(const void* d_indptr, int indptr_is64, const int32_t* d_indi
                     uint64_t rng_seed, uint32_t stream_id,
                     int32_t* d_src_out, int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out,
                     uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream);
+
+/* sample_node without a workspace argument.  Has no counterpart in the reference; it is for callers
+ * that cannot allocate device memory at the point of the call (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and therefore have no workspace to pass.  Same
+ * arguments, kernels and results as fgl_sample_node; the scratch is a 16 MiB device array that the
+ * library itself holds on every GPU it runs on until the process ends.  Limits: n_seeds_max <=
+ * 1 048 576 (FGL_ERR_ARG beyond).  The call allocates and frees nothing.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (different streams) race -- serialise them.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call
+ * outside stream capture. */
+#define FGL_STATIC_MAX_SEEDS 1048576
+int fgl_sample_node_static(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
+                           const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
+                           uint64_t rng_seed, uint32_t stream_id,
+                           int32_t* d_src_out, int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out,
+                           uint32_t* d_status, void* stream);
 
 /* TableSize -- the reference's sizing rule (cuda_hashtable.cuh:27-30), evaluated in 64 bits:
  * (largest power of two <= num) << scale.  Kept for callers that size by it. */

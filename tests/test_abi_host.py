@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_pure_host_entry_points():
     lib = fastgl.lib()
-    assert lib.fgl_abi_version() == 4
+    assert lib.fgl_abi_version() == 5
     assert fastgl.table_size(40960, 2) == 131072
     assert fastgl.table_size(8110080, 2) == 16777216
     assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25
@@ -68,6 +68,9 @@ def test_argument_errors_are_reported_not_launched():
     assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 1, None, -1, None, None, 8, None) == 1
     assert b"dtype" in lib.fgl_last_error()
     assert lib.fgl_rmat_keys(0, 10, 40, 100, 0, None, None) == 1
+    # the entry point with the library's own scratch states its limit before touching the GPU
+    assert lib.fgl_sample_node_static(None, 1, None, 10, None, (1 << 20) + 1, None, 5, 0, 0, None, None, None, None, None, None) == 1
+    assert b"1048576" in lib.fgl_last_error()
 
 
 def test_operator_input_checks_raise_runtime_error():
