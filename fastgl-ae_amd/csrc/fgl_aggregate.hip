@@ -62,13 +62,18 @@ struct RowIO<float, 4> {
 };
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+// Two floats to two bf16 in one 32-bit word (round to nearest even; low half = a): gfx950 has an instruction
+// for it, v_cvt_pk_bf16_f32, which the compiler emits for this vector conversion.  A wave64 ALU instruction
+// occupies its SIMD for four cycles, so the dozen integer operations of a hand-written rounding per element
+// were what bounded the bf16 kernels on short rows, not memory.
+typedef __bf16 Bf16x2 __attribute__((ext_vector_type(2)));
+typedef float Float2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float a, float b)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (u >> 16) | 0x40u;  // quiet NaN
-    u += 0x7FFFu + ((u >> 16) & 1u);                                                       // round to nearest even
-    return u >> 16;
+    const Float2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return f32x2_to_bf16x2_bits(f, 0.0f) & 0xFFFFu; }
 
 // bf16: eight elements per lane as four 32-bit words (rows must start on 4-byte boundaries)
 template <>
@@ -87,15 +92,15 @@ struct RowIO<uint16_t, 8> {
     {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            acc[2 * i] += w * bf16_bits_to_f32(r[i] & 0xFFFFu);
-            acc[2 * i + 1] += w * bf16_bits_to_f32(r[i] >> 16);
+            acc[2 * i] += w * __uint_as_float(r[i] << 16);
+            acc[2 * i + 1] += w * __uint_as_float(r[i] & 0xFFFF0000u);
         }
     }
     static __device__ __forceinline__ void store(uint16_t* p, const float (&acc)[8])
     {
         Raw r;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = f32_to_bf16_bits(acc[2 * i]) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) r[i] = f32x2_to_bf16x2_bits(acc[2 * i], acc[2 * i + 1]);
         *reinterpret_cast<Raw*>(p) = r;
     }
     static __device__ __forceinline__ void store_partial(uint16_t* p, const float (&acc)[8], int n)
@@ -345,7 +350,30 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
             float part[VEC];  // this chunk's sum (see the note on two-level summation in gather_row)
 #pragma unroll
             for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
-            for (int t = 0; t < cnt; ++t) {
+            int t = 0;
+            if (one_head) {
+                // as in gather_row: four row loads -- and the four weights that go with them -- are issued
+                // before the first FMA
+                for (; t + 4 <= cnt; t += 4) {
+                    const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
+                    const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
+                    const int64_t e0 = __shfl(my_eid, t, LPR), e1 = __shfl(my_eid, t + 1, LPR);
+                    const int64_t e2 = __shfl(my_eid, t + 2, LPR), e3 = __shfl(my_eid, t + 3, LPR);
+                    if (live) {
+                        const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                        const typename IO::Raw r1 = ls.load(X + (int64_t)c1 * ldx + col0);
+                        const typename IO::Raw r2 = ls.load(X + (int64_t)c2 * ldx + col0);
+                        const typename IO::Raw r3 = ls.load(X + (int64_t)c3 * ldx + col0);
+                        const float w0 = ew[e0 * H + head[0]], w1 = ew[e1 * H + head[0]];
+                        const float w2 = ew[e2 * H + head[0]], w3 = ew[e3 * H + head[0]];
+                        IO::fma(part, w0, r0);
+                        IO::fma(part, w1, r1);
+                        IO::fma(part, w2, r2);
+                        IO::fma(part, w3, r3);
+                    }
+                }
+            }
+            for (; t < cnt; ++t) {
                 const int c0 = __shfl(my_col, t, LPR);
                 const int64_t e0 = __shfl(my_eid, t, LPR);
                 if (live) {
@@ -371,6 +399,230 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
         else gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc);
     }
     if (live) ls.store(out + row * ldo + col0, acc);
+}
+
+// ---- few rows, long lists: several lane groups share a row -----------------------------------------
+// A block of a few thousand rows (8192 destination rows of 25 entries, say) gives aggregate_kernel one
+// lane group per row: 8192 rows of 64 bf16 columns are 1024 waves, four per CU, each lane with four
+// 16-byte loads in flight -- a few MB in flight on the whole chip, which at the latency of a memory
+// access is a fraction of what HBM delivers.  Here S lane groups of the same wave share a row: all S * LPR
+// lanes load the row's neighbour ids in one coalesced read, group p sums the entries p, p + S, p + 2S, ...
+// (four row loads in flight per lane, all groups at once), and the S partial sums are added with a
+// fixed-order __shfl_xor tree -- no LDS, no atomics, the same bits on every run.  S times the waves, S times
+// the bytes in flight.  Not for FGL_AGG_EDGE.
+template <typename T, int VEC, int LPR, int S, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_split_kernel(const AggArgs g)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int W = S * LPR;  // lanes per row: a divisor of the wave size
+    static_assert(W <= kWave && kWave % W == 0, "a row's lanes must lie within one wave");
+    constexpr int kRowsPerBlock = kBlock / W;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx;
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int q = (int)threadIdx.x % W;  // lane within the row's lanes
+    const int part = q / LPR, gl = q % LPR;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (int)threadIdx.x / W;
+    if (row >= n_rows) return;  // uniform over the row's lanes: the cross-lane reads below stay among live lanes
+    const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, g.D);
+    const int col0 = ls.col0;
+    const bool live = ls.live;
+    const bool all_full = all_lanes_full<T, VEC>(g.D);
+
+    const int a = indptr[row], b = indptr[row + 1];
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+    if (a == b) {
+        if (part == 0 && live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + col0));
+    } else {
+        float row_factor = 1.0f;
+        if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
+        if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
+        for (int base = a; base < b; base += W) {
+            const int cnt = (b - base) < W ? (b - base) : W;
+            int my_col = 0;
+            float my_w = 0.0f;
+            if (q < cnt) {
+                my_col = indices[base + q];
+                my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+            }
+            float sum[VEC];  // this chunk's share of the row (two-level summation, as in gather_row)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) sum[i] = 0.0f;
+            // every group runs the same number of rounds (the cross-lane reads need all of the row's lanes);
+            // entries past the end are read from lane 0 and neither loaded nor added
+            for (int t = part; t - part < cnt; t += 4 * S) {
+                int c[4];
+                float w[4];
+                typename IO::Raw x[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int src = t + j * S < cnt ? t + j * S : 0;
+                    c[j] = __shfl(my_col, src, W);
+                    w[j] = __shfl(my_w, src, W);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    x[j] = typename IO::Raw{};
+                    if (live && t + j * S < cnt)
+                        x[j] = all_full ? IO::load(X + (int64_t)c[j] * ldx + col0) : ls.load(X + (int64_t)c[j] * ldx + col0);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (t + j * S < cnt) IO::fma(sum, w[j], x[j]);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += sum[i];
+        }
+    }
+    // the groups' partial sums: pairwise, in an order that does not depend on scheduling
+#pragma unroll
+    for (int d = LPR; d < W; d <<= 1) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += __shfl_xor(acc[i], d, W);
+    }
+    if (part == 0 && live) ls.store(out + row * g.ldo + col0, acc);
+}
+
+// ---- many rows, short lists: a lane group takes several rows at once -------------------------------
+// The rows of a transposed block hold one entry on average (a third of them none): with one row per lane
+// group, a group's life is three dependent memory accesses -- its two offsets, its one neighbour id, one row
+// of data -- for 16 bytes per lane, and the chip spends its time waiting.  Here a group takes kBundleRows
+// consecutive rows: their offsets are one read, their entries are consecutive in `indices` and are read
+// (with their weights and the row each belongs to) in one coalesced chunk, and the data rows of all of
+// them are in flight together, four at a time; the running sum is stored and cleared whenever an entry is
+// the last of its row.  A bundle that holds a hub (more than 128 entries in all) falls back to one row
+// after the other.  Sums are in CSR order, as in aggregate_kernel.
+// Not for FGL_AGG_EDGE.
+#ifndef FGL_BUNDLE_ROWS
+#define FGL_BUNDLE_ROWS 4
+#endif
+constexpr int kBundleRows = FGL_BUNDLE_ROWS;
+
+template <typename T, int VEC, int LPR, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs g)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int R = kBundleRows;
+    static_assert(R + 1 <= LPR, "a group reads the offsets of its rows with one lane each");
+    constexpr int kGroups = kBlock / LPR;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx, ldo = g.ldo;
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int gl = (int)threadIdx.x % LPR;
+    const int64_t r0 = ((int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR) * R;
+    if (r0 >= n_rows) return;  // uniform per group
+    const int nr = n_rows - r0 < R ? (int)(n_rows - r0) : R;
+    const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, g.D);
+    const int col0 = ls.col0;
+    const bool live = ls.live;
+
+    const int my_off = indptr[r0 + (gl < nr ? gl : nr)];
+    int off[R + 1];  // off[j] = start of row j's entries; rows past the bundle's end are empty
+#pragma unroll
+    for (int j = 0; j <= R; ++j) off[j] = __shfl(my_off, j < nr ? j : nr, LPR);
+    int skip = g.skip_rows_longer_than;  // as in aggregate_kernel
+    if (g.longest_row != nullptr && *g.longest_row <= skip) skip = 0x7FFFFFFF;
+    const int total = off[R] - off[0];
+
+    if (total <= kLongRowEntries) {
+        // (no row of the bundle is long enough to be left to the long-row launch)
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+        // cnt entries from the bundle's entry number cb on: ids, weights and row ends in one coalesced read,
+        // then the data rows four at a time
+        auto chunk = [&](int cb, int cnt) {
+            int my_col = 0, my_tag = 0;  // tag: row within the bundle, + 256 if the entry is the last of its row
+            float my_w = 0.0f;
+            if (gl < cnt) {
+                const int e = off[0] + cb + gl;
+                my_col = indices[e];
+                int j = 0;  // the rows that start at or before e: the last of them, row j, holds e
+                int begin_j = off[0], end_j = off[1];
+#pragma unroll
+                for (int k = 1; k < R; ++k) {
+                    if (off[k] <= e) {
+                        j = k;
+                        begin_j = off[k];
+                        end_j = off[k + 1];
+                    }
+                }
+                float row_factor = 1.0f;
+                if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(end_j - begin_j);
+                if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[r0 + j]);
+                my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                my_tag = j | (e + 1 == end_j ? 256 : 0);
+            }
+            for (int t = 0; t < cnt; t += 4) {
+                int c[4], tag[4];
+                float w[4];
+                typename IO::Raw x[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int src = t + j < cnt ? t + j : t;
+                    c[j] = __shfl(my_col, src, LPR);
+                    w[j] = __shfl(my_w, src, LPR);
+                    tag[j] = __shfl(my_tag, src, LPR);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    x[j] = typename IO::Raw{};
+                    if (live && t + j < cnt) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (t + j < cnt) {
+                        IO::fma(acc, w[j], x[j]);
+                        if (tag[j] & 256) {
+                            if (live) ls.store(out + (r0 + (tag[j] & 255)) * ldo + col0, acc);
+#pragma unroll
+                            for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+                        }
+                    }
+                }
+            }
+        };
+        if (total <= LPR) {  // the usual case, without the loop around it
+            chunk(0, total);
+        } else {
+            for (int cb = 0; cb < total; cb += LPR) chunk(cb, total - cb < LPR ? total - cb : LPR);
+        }
+        // the rows without entries
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            if (j < nr && off[j + 1] == off[j] && live) {
+                float z[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) z[i] = 0.0f;
+                if (g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(z, 1.0f, ls.load(X + (r0 + j) * ldx + col0));
+                ls.store(out + (r0 + j) * ldo + col0, z);
+            }
+        }
+        return;
+    }
+    // a bundle with a longer list: one row after the other, as aggregate_kernel does
+    for (int j = 0; j < nr; ++j) {
+        const int a = off[j], b = off[j + 1];
+        if (b - a > skip) continue;  // left to aggregate_long_rows_kernel
+        const int64_t row = r0 + j;
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+        if (a == b) {
+            if (live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + col0));
+        } else {
+            gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc);
+        }
+        if (live) ls.store(out + row * ldo + col0, acc);
+    }
 }
 
 // Rows whose length fills a power-of-two lane group badly (602 floats = 151 vector lanes: 79 % of three
@@ -458,6 +710,130 @@ __global__ __launch_bounds__(kBlock) void aggregate_flat_kernel(const AggArgs g,
     }
     if (full) IO::store(out + row * g.ldo + col0, acc);
     else IO::store_partial(out + row * g.ldo + col0, acc, nvalid);
+}
+
+// The flat mapping for many rows of short lists (wide rows of a transposed block): lane t owns vector
+// t % lanes of the kBundleRows consecutive rows of bundle t / lanes.  As in aggregate_bundle_kernel the rows'
+// entries are walked as one list, four data rows in flight, the running sum stored at the end of each row;
+// as in aggregate_flat_kernel every lane reads offsets and neighbour ids itself (the same addresses in all
+// lanes of a bundle).
+template <typename T, int VEC, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_flat_bundle_kernel(const AggArgs g, int lanes)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int R = kBundleRows;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx, ldo = g.ldo;
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t r0 = (t / lanes) * R;
+    if (r0 >= n_rows) return;
+    const int nr = n_rows - r0 < R ? (int)(n_rows - r0) : R;
+    int col0 = (int)(t % lanes) * VEC;
+    if (col0 + VEC > g.D && tail_overlaps<T, VEC>(g.D)) col0 = g.D - VEC;
+    const int nvalid = g.D - col0;
+    const bool full = nvalid >= VEC;
+    auto load = [&](const T* p) -> typename IO::Raw { return full ? IO::load(p) : IO::load_partial(p, nvalid); };
+    auto store = [&](T* p, const float (&a)[VEC]) {
+        if (full) IO::store(p, a);
+        else IO::store_partial(p, a, nvalid);
+    };
+    int off[R + 1];
+#pragma unroll
+    for (int j = 0; j <= R; ++j) off[j] = indptr[r0 + (j < nr ? j : nr)];
+    int skip = g.skip_rows_longer_than;  // as in aggregate_kernel
+    if (g.longest_row != nullptr && *g.longest_row <= skip) skip = 0x7FFFFFFF;
+    const int total = off[R] - off[0];
+
+    if (total <= kLongRowEntries) {
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+        for (int cb = 0; cb < total; cb += 4) {
+            int c[4], tag[4];
+            float w[4];
+            typename IO::Raw x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c[j] = indices[off[0] + (cb + j < total ? cb + j : cb)];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                x[j] = typename IO::Raw{};
+                if (cb + j < total) x[j] = load(X + (int64_t)c[j] * ldx + col0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int e = off[0] + cb + j;
+                int row_j = 0, begin_j = off[0], end_j = off[1];  // the row that holds e
+#pragma unroll
+                for (int k = 1; k < R; ++k) {
+                    if (off[k] <= e) {
+                        row_j = k;
+                        begin_j = off[k];
+                        end_j = off[k + 1];
+                    }
+                }
+                float row_factor = 1.0f;
+                if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(end_j - begin_j);
+                if (MODE == FGL_AGG_GCN && cb + j < total) row_factor = 1.0f / sqrtf((float)g.row_norm[r0 + row_j]);
+                w[j] = cb + j < total ? edge_weight<MODE>(c[j], row_factor, g.col_norm) : 0.0f;
+                tag[j] = row_j | (e + 1 == end_j ? 256 : 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (cb + j < total) {
+                    IO::fma(acc, w[j], x[j]);
+                    if (tag[j] & 256) {
+                        store(out + (r0 + (tag[j] & 255)) * ldo + col0, acc);
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            if (j < nr && off[j + 1] == off[j]) {
+                float z[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) z[i] = 0.0f;
+                if (g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(z, 1.0f, load(X + (r0 + j) * ldx + col0));
+                store(out + (r0 + j) * ldo + col0, z);
+            }
+        }
+        return;
+    }
+    // a bundle that holds a hub: one row after the other, two-level sums as in aggregate_flat_kernel
+    for (int j = 0; j < nr; ++j) {
+        const int a = off[j], b = off[j + 1];
+        if (b - a > skip) continue;  // left to aggregate_long_rows_kernel
+        const int64_t row = r0 + j;
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+        if (a == b) {
+            if (g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, load(X + row * ldx + col0));
+        } else {
+            float row_factor = 1.0f;
+            if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
+            if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
+            for (int base = a; base < b; base += kFlatChunk) {
+                const int end = b - base < kFlatChunk ? b : base + kFlatChunk;
+                float part[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
+                for (int e = base; e < end; ++e) {
+                    const int c0 = indices[e];
+                    IO::fma(part, edge_weight<MODE>(c0, row_factor, g.col_norm), load(X + (int64_t)c0 * ldx + col0));
+                }
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += part[i];
+            }
+        }
+        store(out + row * ldo + col0, acc);
+    }
 }
 
 // The rows that aggregate_kernel skipped.  Every workgroup (512 lanes) looks through its share of the
@@ -729,18 +1105,22 @@ static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStre
 
 // Flat mapping (aggregate_flat_kernel) for the short rows, the usual second launch for the long ones.
 template <typename T, int VEC>
-static int launch_agg_flat(int mode, bool long_rows_possible, int lanes, hipStream_t stream, AggArgs g)
+static int launch_agg_flat(int mode, bool long_rows_possible, int lanes, bool bundle, hipStream_t stream, AggArgs g)
 {
     g.skip_rows_longer_than = long_rows_possible ? kLongRowEntries : 0x7FFFFFFF;
-    const int64_t blocks = ceil_div(g.n_rows_max * lanes, kBlock);
+    const int64_t blocks = ceil_div((bundle ? ceil_div(g.n_rows_max, kBundleRows) : g.n_rows_max) * lanes, kBlock);
     if (blocks > 0x7FFFFFFF) {
         set_error("aggregate: grid too large (%lld workgroups)", (long long)blocks);
         return FGL_ERR_UNSUPPORTED;
     }
 #define FGL_LAUNCH_FLAT(M)                                                                                          \
     do {                                                                                                            \
-        hipLaunchKernelGGL((aggregate_flat_kernel<T, VEC, M>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, g,    \
-                           lanes);                                                                                  \
+        if (bundle)                                                                                                 \
+            hipLaunchKernelGGL((aggregate_flat_bundle_kernel<T, VEC, M>), dim3((unsigned)blocks), dim3(kBlock), 0,   \
+                               stream, g, lanes);                                                                   \
+        else                                                                                                        \
+            hipLaunchKernelGGL((aggregate_flat_kernel<T, VEC, M>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,  \
+                               g, lanes);                                                                           \
         if (long_rows_possible) {                                                                                   \
             int64_t lb = ceil_div(g.n_rows_max, kLongBlock);                                                        \
             if (lb > kLongRowBlocks) lb = kLongRowBlocks;                                                           \
@@ -759,16 +1139,77 @@ static int launch_agg_flat(int mode, bool long_rows_possible, int lanes, hipStre
     return FGL_OK;
 }
 
+// Launches of the two special mappings.  (Only for rows that fit one lane group; never for FGL_AGG_EDGE.)
+#define FGL_FOR_PLAIN_MODE(mode, LAUNCH)                  \
+    switch (mode) {                                       \
+        case FGL_AGG_SUM: LAUNCH(FGL_AGG_SUM); break;     \
+        case FGL_AGG_MEAN: LAUNCH(FGL_AGG_MEAN); break;   \
+        case FGL_AGG_GCN: LAUNCH(FGL_AGG_GCN); break;     \
+        default: LAUNCH(FGL_AGG_COLMEAN); break;          \
+    }
+
+template <typename T, int VEC, int LPR, int S>
+static int launch_agg_split(int mode, unsigned gy, hipStream_t stream, AggArgs g)
+{
+    g.skip_rows_longer_than = 0x7FFFFFFF;
+    const int64_t gx = ceil_div(g.n_rows_max, kBlock / (S * LPR));
+#define FGL_LAUNCH_SPLIT(M) \
+    hipLaunchKernelGGL((aggregate_split_kernel<T, VEC, LPR, S, M>), dim3((unsigned)gx, gy), dim3(kBlock), 0, stream, g)
+    FGL_FOR_PLAIN_MODE(mode, FGL_LAUNCH_SPLIT)
+#undef FGL_LAUNCH_SPLIT
+    FGL_CHECK_LAUNCH("aggregate_split_kernel");
+    return FGL_OK;
+}
+
+template <typename T, int VEC, int LPR>
+static int launch_agg_bundle(int mode, bool long_rows_possible, unsigned gy, hipStream_t stream, AggArgs g)
+{
+    g.skip_rows_longer_than = long_rows_possible ? kLongRowEntries : 0x7FFFFFFF;
+    const int64_t gx = ceil_div(ceil_div(g.n_rows_max, kBundleRows), kBlock / LPR);
+#define FGL_LAUNCH_BUNDLE(M)                                                                                          \
+    do {                                                                                                              \
+        hipLaunchKernelGGL((aggregate_bundle_kernel<T, VEC, LPR, M>), dim3((unsigned)gx, gy), dim3(kBlock), 0, stream, g); \
+        if (long_rows_possible) {                                                                                     \
+            int64_t lb = ceil_div(g.n_rows_max, kLongBlock);                                                          \
+            if (lb > kLongRowBlocks) lb = kLongRowBlocks;                                                             \
+            hipLaunchKernelGGL((aggregate_long_rows_kernel<T, VEC, LPR, M>), dim3((unsigned)lb, gy), dim3(kLongBlock), \
+                               0, stream, g);                                                                         \
+        }                                                                                                             \
+    } while (0)
+    FGL_FOR_PLAIN_MODE(mode, FGL_LAUNCH_BUNDLE)
+#undef FGL_LAUNCH_BUNDLE
+    FGL_CHECK_LAUNCH("aggregate_bundle_kernel");
+    return FGL_OK;
+}
+
+// A launch of fewer waves than this leaves the chip waiting on memory latency (one lane group per row): rows
+// whose lists are known to be long enough are then shared by several groups (aggregate_split_kernel).
+#ifndef FGL_SPLIT_BELOW_WAVES
+#define FGL_SPLIT_BELOW_WAVES 2048
+#endif
+#ifndef FGL_SPLIT_TARGET_WAVES
+#define FGL_SPLIT_TARGET_WAVES 4096  // groups per row are doubled until the launch has this many waves
+#endif
+// Lists of at most this many entries on average (per row, from the caller's entry count) are taken several
+// rows at a time (aggregate_bundle_kernel).
+#ifndef FGL_BUNDLE_MAX_AVG_ENTRIES
+#define FGL_BUNDLE_MAX_AVG_ENTRIES 2
+#endif
+
 template <typename T, int VEC>
-static int launch_agg_vec(int mode, int64_t longest_row_max, hipStream_t stream, const AggArgs& g)
+static int launch_agg_vec(int mode, int64_t longest_row_max, int64_t n_entries_max, hipStream_t stream, const AggArgs& g)
 {
     const int lanes_needed = (g.D + VEC - 1) / VEC;
     int lpr = 8;
     while (lpr < 64 && lpr < lanes_needed) lpr <<= 1;
+    // many rows of short lists (a transposed block): several rows per lane group
+    const bool short_lists = mode != FGL_AGG_EDGE && n_entries_max >= 0 && g.n_rows_max >= 1024 &&
+                             n_entries_max <= (int64_t)FGL_BUNDLE_MAX_AVG_ENTRIES * g.n_rows_max;
     // rows wider than one 64-lane group that fill their groups to less than 90 %: flat mapping
     // (602 fp32 columns: 100 -> 80 us; 602 bf16: 59 -> 44 us forward, 135 -> 84 us on the transposed block)
     if (lanes_needed > 64 && mode != FGL_AGG_EDGE && lanes_needed * 10 < ceil_div(lanes_needed, 64) * 64 * 9)
-        return launch_agg_flat<T, VEC>(mode, longest_row_max < 0 || longest_row_max > kLongRowEntries, lanes_needed, stream, g);
+        return launch_agg_flat<T, VEC>(mode, longest_row_max < 0 || longest_row_max > kLongRowEntries, lanes_needed,
+                                       short_lists, stream, g);
     const int64_t groups = kBlock / lpr;
     const int64_t gx = ceil_div(g.n_rows_max, groups);
     const int64_t gy = ceil_div(lanes_needed, lpr);
@@ -779,6 +1220,31 @@ static int launch_agg_vec(int mode, int64_t longest_row_max, hipStream_t stream,
     const dim3 grid((unsigned)gx, (unsigned)gy);
     // a host-side bound that rules long rows out makes this exactly one launch of the plain kernel
     const bool long_rows_possible = longest_row_max < 0 || longest_row_max > kLongRowEntries;
+    if constexpr (VEC > 1) {
+        // few rows, lists known to be long: S lane groups per row, chosen so that each group still gets
+        // three entries or more and the launch reaches FGL_SPLIT_BELOW_WAVES waves
+        const int64_t waves = ceil_div(g.n_rows_max * lpr, kWave);
+        if (mode != FGL_AGG_EDGE && lpr < 64 && !long_rows_possible && waves < FGL_SPLIT_BELOW_WAVES) {
+            int s = 64 / lpr;
+            while (s > 1 && ((int64_t)s * 3 > longest_row_max || waves * (s / 2) >= FGL_SPLIT_TARGET_WAVES)) s >>= 1;
+#define FGL_SPLIT_CASE(L, S_) if (lpr == L && s == S_) return launch_agg_split<T, VEC, L, S_>(mode, grid.y, stream, g)
+            FGL_SPLIT_CASE(8, 8);
+            FGL_SPLIT_CASE(8, 4);
+            FGL_SPLIT_CASE(8, 2);
+            FGL_SPLIT_CASE(16, 4);
+            FGL_SPLIT_CASE(16, 2);
+            FGL_SPLIT_CASE(32, 2);
+#undef FGL_SPLIT_CASE
+        }
+        // (not for rows of eight lanes -- 128 bytes, one cache line: there the bundle's bookkeeping costs what it saves)
+        if (short_lists && lpr >= 16) {
+            switch (lpr) {
+                case 16: return launch_agg_bundle<T, VEC, 16>(mode, long_rows_possible, grid.y, stream, g);
+                case 32: return launch_agg_bundle<T, VEC, 32>(mode, long_rows_possible, grid.y, stream, g);
+                default: return launch_agg_bundle<T, VEC, 64>(mode, long_rows_possible, grid.y, stream, g);
+            }
+        }
+    }
     switch (lpr) {
         case 8: return launch_agg_mode<T, VEC, 8>(mode, long_rows_possible, grid, stream, g);
         case 16: return launch_agg_mode<T, VEC, 16>(mode, long_rows_possible, grid, stream, g);
@@ -801,8 +1267,8 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
                              const int32_t* d_n_rows, const void* d_x, int64_t ldx, int D, int dtype, int mode,
                              int zero_policy, const int32_t* d_row_norm, const int32_t* d_col_norm,
                              const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
-                             int64_t longest_row_max, const int32_t* d_longest_row, void* d_out, int64_t ldo,
-                             void* stream)
+                             int64_t longest_row_max, const int32_t* d_longest_row, int64_t n_entries_max,
+                             void* d_out, int64_t ldo, void* stream)
 {
     FGL_REQUIRE(n_rows_max >= 0, "aggregate: negative row count");
     FGL_REQUIRE(D >= 1, "aggregate: feature length %d < 1", D);
@@ -823,9 +1289,9 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     g.out = d_out; g.ldo = ldo; g.edge_w = d_edge_w; g.edge_index = d_edge_index; g.longest_row = d_longest_row;
     g.n_heads = n_heads > 0 ? n_heads : 1; g.unit_dim = D / g.n_heads;
     hipStream_t s = as_stream(stream);
-    if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, longest_row_max, s, g);
-    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, longest_row_max, s, g);
-    return launch_agg_vec<uint16_t, 1>(mode, longest_row_max, s, g);
+    if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, longest_row_max, n_entries_max, s, g);
+    if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, longest_row_max, n_entries_max, s, g);
+    return launch_agg_vec<uint16_t, 1>(mode, longest_row_max, n_entries_max, s, g);
 }
 
 FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)

@@ -354,8 +354,8 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
             L.check(L.lib().fgl_aggregate(L.ptr(indptr), idx_ptr, n, L.ptr(n_rows_dev), L.ptr(feat), int(feat.stride(0)), D,
                                           L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
                                           L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index),
-                                          longest_host, L.ptr(longest_dev), L.ptr(out), int(out.stride(0)),
-                                          L.stream_handle()))
+                                          longest_host, L.ptr(longest_dev), int(indices.numel()), L.ptr(out),
+                                          int(out.stride(0)), L.stream_handle()))
     return out
 
 

@@ -57,7 +57,12 @@ class Block:
         return self
 
     def to(self, device):
-        if torch.device(device) != self.edge_ptr.device:
+        # a device without an index ("cuda") means the current device of that type
+        want, have = torch.device(device), self.edge_ptr.device
+        same = want.type == have.type
+        if same and have.type == "cuda":
+            same = (torch.cuda.current_device() if want.index is None else want.index) == have.index
+        if not same:
             raise RuntimeError("Block.to: blocks live on the device they were sampled on")
         return self
 

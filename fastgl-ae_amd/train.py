@@ -59,7 +59,8 @@ def run(args):
     print("config:dataset=rmat_%d nodes=%d edges=%d train=%d" % (args.nodes, args.nodes, edge_src.numel(), train_nids.numel()))
     for k, v in sorted(vars(args).items()):
         print("config:{:}={:}".format(k, v))
-    sampler = fastgl.FusedMapSampler(args.fanout, rng_seed=args.seed, id_order=args.id_order).set_graph(edge_ptr, edge_src)
+    sampler = fastgl.FusedMapSampler(args.fanout, rng_seed=args.seed, id_order=args.id_order,
+                                     deterministic=bool(args.deterministic)).set_graph(edge_ptr, edge_src)
     model = build_model(args.model, args.feat_dim, args.num_hidden, args.classes, len(args.fanout), args.dropout).to(device)
     loss_fcn = torch.nn.CrossEntropyLoss()
     optimizer = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
@@ -162,6 +163,9 @@ def parse_args(argv=None):
     ap.add_argument("--weight_decay", type=float, default=0.0005)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--id_order", default="first", choices=["first", "arrival"])
+    ap.add_argument("--deterministic", type=int, default=0,
+                    help="1: order the transposed blocks' lists too, so that the fp32 sums of the backward pass -- and with them "
+                         "the whole run -- are reproducible bit for bit (one radix sort per block; needs --id_order first)")
     ap.add_argument("--prefetch", type=int, default=1, help="1: sample the next mini-batch on a second stream (default)")
     ap.add_argument("--log_every", type=int, default=10)
     ap.add_argument("--log_path", default="")

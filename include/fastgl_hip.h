@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 5
+#define FGL_ABI_VERSION 6
 
 enum fgl_error {
     FGL_OK = 0,
@@ -254,13 +254,18 @@ int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
  * more (hubs of a transposed block) are summed by a second launch in which a whole
  * workgroup shares each such row; a host bound that rules them out saves that launch, a
  * device value that does lets it end at once.  Speed only: wrong values still give correct sums.
+ * n_entries_max: what the caller knows about the number of entries (indptr[n_rows]): an upper bound, or
+ * < 0 for "unknown".  Together with n_rows_max and longest_row_max it picks the lane mapping -- several
+ * lane groups per row for a few thousand rows of long lists (a small sampled block), several rows per lane
+ * group for many rows of one entry on average (a transposed block), one group per row otherwise.  Speed
+ * only as well; the order of the fp32 additions within a row depends on the mapping, not on the run.
  * ------------------------------------------------------------------------------- */
 int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
                   int64_t n_rows_max, const int32_t* d_n_rows,
                   const void* d_x, int64_t ldx, int D, int dtype, int mode, int zero_policy,
                   const int32_t* d_row_norm, const int32_t* d_col_norm,
                   const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
-                  int64_t longest_row_max, const int32_t* d_longest_row,
+                  int64_t longest_row_max, const int32_t* d_longest_row, int64_t n_entries_max,
                   void* d_out, int64_t ldo, void* stream);
 
 /* ---------------------------------------------------------------------------------

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_pure_host_entry_points():
     lib = fastgl.lib()
-    assert lib.fgl_abi_version() == 5
+    assert lib.fgl_abi_version() == 6
     assert fastgl.table_size(40960, 2) == 131072
     assert fastgl.table_size(8110080, 2) == 16777216
     assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25
@@ -65,7 +65,7 @@ def test_argument_errors_are_reported_not_launched():
     assert b"fanout" in lib.fgl_last_error()
     assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
     assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table
-    assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 1, None, -1, None, None, 8, None) == 1
+    assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 1, None, -1, None, -1, None, 8, None) == 1
     assert b"dtype" in lib.fgl_last_error()
     assert lib.fgl_rmat_keys(0, 10, 40, 100, 0, None, None) == 1
     # the entry point with the library's own scratch states its limit before touching the GPU
@@ -97,6 +97,9 @@ def test_sampler_front_end_without_gpu():
     src, dst = b.edges()
     assert dst.tolist() == [0, 0, 2, 2, 2] and b.num_src_nodes() == 5 and b.num_dst_nodes() == 3 and b.num_edges() == 5
     assert b.in_degrees().tolist() == [2, 0, 3]
+    assert b.int().to("cpu") is b and b.to(torch.device("cpu")) is b
+    with pytest.raises(RuntimeError, match="live on the device"):
+        b.to("cuda")
     b.edge_ptr.fgl_longest_row = 3
     c = b.clone()
     assert c.edge_ptr.data_ptr() != b.edge_ptr.data_ptr() and c.edge_ptr.fgl_longest_row == 3

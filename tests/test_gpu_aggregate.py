@@ -386,3 +386,59 @@ def test_edge_softmax_vs_oracle_and_torch(cuda, oracle, H):
     # an empty block
     empty = fastgl.edge_softmax(dev_i32(np.zeros(4, np.int32), cuda), dev_i32(np.zeros(0, np.int32), cuda), d_el, d_er[:3], 0.2)
     assert tuple(empty.shape) == (0, H)
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 24), (torch.float32, 64), (torch.float32, 100), (torch.bfloat16, 64),
+                                     (torch.bfloat16, 50), (torch.bfloat16, 128), (torch.bfloat16, 256)])
+@pytest.mark.parametrize("bound", [6, 12, 25, 64, 100])
+def test_few_rows_of_long_lists(cuda, oracle, dtype, D, bound):
+    """A block of a few rows whose lists are known to be long (the caller names a bound, as the sampler names its
+    fanout): several lane groups share a row and their partial sums are added across lanes.  Rows of every
+    length from none to the bound, row counts that do not fill a workgroup, all modes and both policies."""
+    import fastgl
+    print("few long rows D=%d %s bound=%d" % (D, dtype, bound), flush=True)
+    rng = np.random.default_rng(D * 1000 + bound)
+    for n_dst in (1, 7, 333, 4000):
+        n_src = 5000
+        deg = rng.integers(0, bound + 1, size=n_dst)
+        deg[rng.integers(0, n_dst)] = bound
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+        idx = rng.integers(0, n_src, size=ptr[-1]).astype(np.int32)
+        X = torch.from_numpy(rng.standard_normal((n_src, D)).astype(np.float32)).to(cuda).to(dtype)
+        X_ref = X.float().cpu().numpy()
+        rn = np.maximum(deg, 1).astype(np.int32)
+        cn = np.maximum(np.bincount(idx, minlength=n_src), 1).astype(np.int32)
+        d_ptr, d_idx, d_rn, d_cn = dev_i32(ptr, cuda), dev_i32(idx, cuda), dev_i32(rn, cuda), dev_i32(cn, cuda)
+        for mode in ("sum", "mean", "gcn", "colmean"):
+            for pol_name, pol in (("self", 0), ("zeros", 1)):
+                want = oracle.aggregate(ptr, idx, X_ref, mode, pol, rn, cn)
+                got = fastgl.aggregate(d_ptr, d_idx, X, mode=mode, zero_policy=pol_name, row_norm=d_rn, col_norm=d_cn,
+                                       longest_row=bound)
+                err = rel_err(got.float().cpu().numpy(), want)
+                assert err < TOL[dtype], (n_dst, mode, pol_name, err)
+                # the same sums bit for bit on a second run (the cross-lane additions have a fixed order)
+                again = fastgl.aggregate(d_ptr, d_idx, X, mode=mode, zero_policy=pol_name, row_norm=d_rn, col_norm=d_cn,
+                                         longest_row=bound)
+                assert torch.equal(got, again)
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.float32, 128), (torch.float32, 256), (torch.float32, 602),
+                                     (torch.bfloat16, 64), (torch.bfloat16, 128), (torch.bfloat16, 602), (torch.bfloat16, 31)])
+def test_many_rows_of_short_lists(cuda, oracle, dtype, D):
+    """What a transposed block looks like: thousands of rows with one entry on average (many with none), which a lane
+    group takes several at a time; with a few lists long enough to span the group's chunks, hubs that go to the
+    long-row launch, and row counts that leave the last bundle incomplete."""
+    import fastgl
+    print("many short rows D=%d %s" % (D, dtype), flush=True)
+    rng = np.random.default_rng(D)
+    for n_dst, hubs in ((1024, []), (4099, [(5, 70), (6, 9), (7, 140), (2000, 33), (4098, 600)]), (6001, [(6000, 17), (0, 129)])):
+        n_src = 3000
+        deg = rng.poisson(1.0, size=n_dst)
+        for r, d in hubs:
+            deg[r] = d
+        deg[0] = 0 if not hubs else deg[0]
+        assert deg.sum() <= 2 * n_dst
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+        idx = rng.integers(0, n_src, size=ptr[-1]).astype(np.int32)
+        X = torch.from_numpy(rng.standard_normal((max(n_src, n_dst), D)).astype(np.float32)).to(cuda).to(dtype)
+        run_modes(cuda, oracle, ptr, idx, deg, X, max(n_src, n_dst), TOL[dtype])

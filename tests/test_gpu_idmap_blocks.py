@@ -159,7 +159,9 @@ def test_begin_sample_then_finish(cuda, oracle, small_graph):
         check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], got, 4, 64 * batch)
         b0 = got[2][0]
         late = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
-        assert torch.equal(early[:b0.num_dst_nodes()], late)
+        # (the two launches may map lanes to rows differently -- the bound-sized one has many more rows -- and the
+        # order of the fp32 additions within a row follows the mapping: equal up to rounding, not bit for bit)
+        assert torch.allclose(early[:b0.num_dst_nodes()], late, rtol=1e-5, atol=1e-6)
     sampler._nodes_seen = [700, 800, 900, 1000]                             # (pretend the batches stayed tiny)
     hubs = np.argsort(-np.diff(indptr))[:700].astype(np.int32)
     pend = sampler.begin_sample(dev_i32(hubs, cuda))
