@@ -8,18 +8,65 @@
 // Also: the seeded R-MAT key generator used to build the synthetic benchmark graphs.
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
+#include "fgl_table.hpp"
 
 namespace fgl {
 
-// Start of a mini-batch in one launch: every table slot back to empty (all ones), node count of
-// hop 0 = the seed count, the other counts and the status word zero.
-__global__ __launch_bounds__(kBlock) void blocks_reset_kernel(uint32_t* __restrict__ table_words, int64_t n_words,
-                                                              int32_t* __restrict__ counts, int n_entries, int32_t n_seeds)
+// Start of a mini-batch in one launch (the table is empty -- left so by the call before, or by a fill launch):
+//   - counts: node count of hop 0 = the seed count, the other counts and the status word zero;
+//   - the per-tile edge counts of the later hops zero (they are accumulated with atomics as hops run);
+//   - every seed: its id into the unique list and the table (local id = position), the start and length of
+//     its row in the graph for the first hop's sampling kernel, and the first hop's per-tile edge counts.
+// The status word is being initialised by this launch, so nothing here reports through it: a seed outside the
+// graph or one that found the table full gets a negative row start, which the first hop's sampling kernel
+// (the next launch) reports.
+template <int TS>
+__global__ __launch_bounds__(TS) void blocks_prepare_kernel(TableRef t, const void* __restrict__ indptr, int is64,
+                                                            int64_t n_nodes, const int32_t* __restrict__ seeds,
+                                                            int64_t n_seeds, int fanout, int32_t* __restrict__ uniq,
+                                                            int64_t* __restrict__ row_start, int32_t* __restrict__ deg_out,
+                                                            int32_t* __restrict__ tile_sums, int32_t* __restrict__ later_sums,
+                                                            int64_t n_later_sums, int32_t* __restrict__ counts, int n_counts)
 {
-    const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (first < n_entries) counts[first] = (first == 0) ? n_seeds : 0;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = first; i < n_words; i += stride) table_words[i] = 0xFFFFFFFFu;
+    __shared__ int smem[TS / kWave + 1];
+    const int64_t first = (int64_t)blockIdx.x * TS + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * TS;
+    if (first < n_counts) counts[first] = (first == 0) ? (int32_t)n_seeds : 0;
+    for (int64_t i = first; i < n_later_sums; i += stride) later_sums[i] = 0;
+    const int64_t n_tiles = (n_seeds + TS - 1) / TS;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t i = tile * TS + threadIdx.x;
+        int k = 0;
+        if (i < n_seeds) {
+            const int32_t s = seeds[i];
+            if (uniq != seeds) uniq[i] = s;
+            int64_t a = kRowBadId, deg = 0;
+            if (s >= 0 && (int64_t)s < n_nodes) {
+                if (is64) {
+                    const int64_t* p = static_cast<const int64_t*>(indptr);
+                    a = p[s];
+                    deg = p[s + 1] - a;
+                } else {
+                    const int32_t* p = static_cast<const int32_t*>(indptr);
+                    a = p[s];
+                    deg = (int64_t)p[s + 1] - a;
+                }
+                if (deg < 0) deg = 0;
+                if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
+                uint32_t seen;
+                if (find_or_insert(t, (uint32_t)s, (uint32_t)i, &seen) == kEmpty) {  // a repeated seed keeps its first position
+                    a = kRowTableFull;
+                    deg = 0;
+                }
+            }
+            row_start[i] = a;
+            deg_out[i] = (int32_t)deg;
+            k = deg < fanout ? (int)deg : fanout;
+        }
+        int total;
+        (void)block_exclusive_scan<TS>(k, smem, &total);
+        if (threadIdx.x == 0) tile_sums[tile] = total;
+    }
 }
 
 struct BlocksPlan {
@@ -28,7 +75,35 @@ struct BlocksPlan {
     int64_t cap_uniq;
     int64_t table_slots;
     size_t ws_bytes;
+    // layout of the workspace: what persists over the hops of a mini-batch, then the id-map's per-hop scratch
+    int64_t n_positions;       // row start / degree entries: one per node that is a seed of some hop
+    int64_t tile_first[33];    // per-tile edge counts of hop h start at entry tile_first[h]; [n_hops] = their total
+    int64_t max_tiles;
+    int64_t max_edges;
+    size_t idmap_bytes;
 };
+
+struct BlocksScratch {
+    int64_t* row_start;
+    int32_t* deg;
+    int32_t* tile_sums;
+    int32_t* tile_prefix;
+    uint8_t* lowered;  // one byte per edge of a hop: cleared by the hop's sampling kernel, used by its id-map passes
+    char* idmap_ws;
+};
+
+static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
+{
+    Carver c(ws);
+    int64_t* row_start = c.take<int64_t>((size_t)p.n_positions);
+    int32_t* deg = c.take<int32_t>((size_t)p.n_positions);
+    int32_t* tile_sums = c.take<int32_t>((size_t)p.tile_first[32]);
+    int32_t* tile_prefix = c.take<int32_t>((size_t)p.max_tiles);
+    uint8_t* lowered = c.take<uint8_t>((size_t)p.max_edges);
+    char* idmap_ws = c.take<char>(p.idmap_bytes);
+    if (out) *out = BlocksScratch{row_start, deg, tile_sums, tile_prefix, lowered, idmap_ws};
+    return c.used();
+}
 
 // node_capacity (optional, n_hops+1 entries): the caller's own limit on the number of nodes before
 // hop h (entry n_hops: after the last hop).  The plan is the worst case clipped to it.
@@ -38,7 +113,8 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
     FGL_REQUIRE(n_hops >= 1 && n_hops <= 32, "sample_blocks: %d hops outside [1, 32]", n_hops);
     FGL_REQUIRE(n_nodes >= 0 && n_seeds >= 0 && fanouts != nullptr, "sample_blocks: bad sizes");
     int64_t cur = n_seeds;
-    size_t ws = 0;
+    size_t idmap_ws = 0;
+    int64_t tiles_total = 0, max_tiles = 1, max_edges = 1;
     for (int h = 0; h < n_hops; ++h) {
         FGL_REQUIRE(fanouts[h] >= 1 && fanouts[h] <= FGL_MAX_FANOUT, "sample_blocks: fanout %d outside [1, %d]", fanouts[h], FGL_MAX_FANOUT);
         if (node_capacity) {
@@ -48,13 +124,19 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
         p->cap_dst[h] = cur;
         p->cap_edges[h] = cur * fanouts[h];
         FGL_REQUIRE(p->cap_edges[h] <= 0x7FFFFFFF, "sample_blocks: hop %d may produce %lld edges, beyond int32 offsets", h, (long long)p->cap_edges[h]);
-        size_t w = sample_workspace_bytes(p->cap_dst[h], fanouts[h]) + idmap_map_src_workspace_bytes(p->cap_edges[h]);
-        if (w > ws) ws = w;
+        if (p->cap_edges[h] > max_edges) max_edges = p->cap_edges[h];
+        const size_t w = idmap_map_src_workspace_bytes(p->cap_edges[h]);
+        if (w > idmap_ws) idmap_ws = w;
+        const int64_t tiles = sample_tile_count(p->cap_dst[h], fanouts[h]);
+        p->tile_first[h] = tiles_total;
+        tiles_total += tiles;
+        if (tiles > max_tiles) max_tiles = tiles;
         // every node is numbered once; repeated seeds are the only way past n_nodes
         int64_t next = cur + p->cap_edges[h];
         if (next > n_nodes + n_seeds) next = n_nodes + n_seeds;
         cur = next;
     }
+    for (int h = n_hops; h <= 32; ++h) p->tile_first[h] = tiles_total;
     if (node_capacity) {
         FGL_REQUIRE(node_capacity[n_hops] >= p->cap_dst[n_hops - 1], "sample_blocks: node_capacity[%d] is below an earlier entry", n_hops);
         if (cur > node_capacity[n_hops]) cur = node_capacity[n_hops];
@@ -62,7 +144,11 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
     p->cap_uniq = cur;
     p->table_slots = fgl_idmap_slots(cur);
     FGL_REQUIRE(p->table_slots <= ((int64_t)1 << 31), "sample_blocks: table too large");
-    p->ws_bytes = ws;
+    p->n_positions = p->cap_dst[n_hops - 1] > 0 ? p->cap_dst[n_hops - 1] : 1;
+    p->max_tiles = max_tiles;
+    p->max_edges = max_edges;
+    p->idmap_bytes = idmap_ws;
+    p->ws_bytes = carve_scratch(*p, nullptr, nullptr);
     return FGL_OK;
 }
 
@@ -129,7 +215,11 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     BlocksPlan p;
     int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
     if (rc != FGL_OK) return rc;
-    FGL_REQUIRE(idmap_flags == FGL_IDMAP_ORDERED || idmap_flags == FGL_IDMAP_ARRIVAL, "sample_blocks: unknown id-map flags %d", idmap_flags);
+    const int order = idmap_flags & FGL_IDMAP_ARRIVAL;
+    const bool table_is_empty = (idmap_flags & FGL_BLOCKS_TABLE_EMPTY) != 0;
+    const bool leave_empty = (idmap_flags & FGL_BLOCKS_LEAVE_TABLE_EMPTY) != 0;
+    FGL_REQUIRE((idmap_flags & ~(FGL_IDMAP_ARRIVAL | FGL_BLOCKS_TABLE_EMPTY | FGL_BLOCKS_LEAVE_TABLE_EMPTY)) == 0,
+                "sample_blocks: unknown flags %d", idmap_flags);
     FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
     FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
     // A table smaller than the plan's worst case is accepted (batches are usually far below the
@@ -146,37 +236,68 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     hipStream_t s = as_stream(stream);
     const int n_counts = 2 * n_hops + 2;
     uint32_t* d_status = reinterpret_cast<uint32_t*>(d_counts + 2 * n_hops + 1);
-    FGL_REQUIRE(table_slots >= 64 && table_slots <= ((int64_t)1 << 31) && (table_slots & (table_slots - 1)) == 0,
-                "sample_blocks: slot count %lld is not a power of two in [64, 2^31]", (long long)table_slots);
-    {
-        const int64_t n_words = table_slots * 2;
-        int64_t blocks = ceil_div(n_words, (int64_t)kBlock * 4);
-        if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL(blocks_reset_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, static_cast<uint32_t*>(d_table),
-                           n_words, d_counts, n_counts, (int32_t)n_seeds);
-        FGL_CHECK_LAUNCH("blocks_reset_kernel");
+    FGL_REQUIRE(valid_slots(table_slots), "sample_blocks: slot count %lld is not a power of two in [64, 2^31]", (long long)table_slots);
+    BlocksScratch ws;
+    carve_scratch(p, d_ws, &ws);
+    const TableRef t = make_ref(d_table, table_slots);
+
+    // launch 1 (only if the caller does not vouch for an empty table): every slot to empty
+    if (!table_is_empty) {
+        rc = launch_fill_u32(t.words, table_slots * 2, kEmpty, s);
+        if (rc != FGL_OK) return rc;
     }
-    rc = launch_idmap_insert_dst(d_table, table_slots, d_seeds, n_seeds, nullptr, d_uniq, d_status, s);
-    if (rc != FGL_OK) return rc;
+    // launch 2: counts, the later hops' tile sums, the seeds into the table, the first hop's rows and tile sums
+    {
+        const int ts0 = sample_tile_seeds(fanouts[0], n_seeds);
+        const int64_t tiles0 = sample_tile_count(n_seeds, fanouts[0]);
+        const int64_t n_later = p.tile_first[n_hops] - p.tile_first[1];
+        int64_t blocks = tiles0;
+        if (blocks < ceil_div(n_later, ts0)) blocks = ceil_div(n_later, ts0);
+        if (blocks > 8192) blocks = 8192;
+        if (blocks < 1) blocks = 1;
+        if (ts0 == 256)
+            hipLaunchKernelGGL(blocks_prepare_kernel<256>, dim3((unsigned)blocks), dim3(256), 0, s, t, d_indptr, indptr_is64, n_nodes,
+                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+        else
+            hipLaunchKernelGGL(blocks_prepare_kernel<64>, dim3((unsigned)blocks), dim3(64), 0, s, t, d_indptr, indptr_is64, n_nodes,
+                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+        FGL_CHECK_LAUNCH("blocks_prepare_kernel");
+    }
 
     for (int h = 0; h < n_hops; ++h) {
+        const bool last = h == n_hops - 1;
         const int32_t* hop_seeds = (h == 0) ? d_seeds : d_uniq;
         int32_t* d_n_dst = d_counts + h;
         int32_t* d_n_edges = d_counts + n_hops + 1 + h;
         int32_t* sampled = (src_global && src_global[h]) ? src_global[h] : src_local[h];
-        char* ws = static_cast<char*>(d_ws);
-        const size_t ws_sample = sample_workspace_bytes(p.cap_dst[h], fanouts[h]);
-        rc = launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], rng_seed,
-                           stream_base + (uint32_t)h, sampled, nullptr, block_ptr[h], d_n_edges, d_status, ws, ws_sample, s,
-                           d_stream_offset);
+        // what this hop's passes prepare for the next hop's sampling: the hop's seeds are the next hop's first
+        // seeds (their row starts and degrees are in place already; the sampling kernel adds their share of the
+        // next tile sums), the nodes it numbers are the rest (the id-map's numbering pass fills in theirs)
+        NextHop next{};
+        if (!last) {
+            next.indptr = d_indptr;
+            next.is64 = indptr_is64;
+            next.n_nodes = n_nodes;
+            next.row_start = ws.row_start;
+            next.deg = ws.deg;
+            next.tile_sums = ws.tile_sums + p.tile_first[h + 1];
+            next.fanout = fanouts[h + 1];
+            next.tile_seeds = sample_tile_seeds(fanouts[h + 1], p.cap_dst[h + 1]);
+        }
+        rc = launch_sample_edges(d_indices, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], ws.row_start, ws.deg,
+                                 ws.tile_sums + p.tile_first[h], ws.tile_prefix, rng_seed, stream_base + (uint32_t)h, sampled,
+                                 nullptr, block_ptr[h], d_n_edges, d_status, s, d_stream_offset, last ? nullptr : &next,
+                                 ws.lowered);
         if (rc != FGL_OK) return rc;
         // the node count this hop may grow to: what the next hop's buffers (or the unique list) hold;
         // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped
-        const int64_t grow_to = (h + 1 < n_hops && p.cap_dst[h + 1] < p.cap_uniq) ? p.cap_dst[h + 1] : p.cap_uniq;
+        const int64_t grow_to = (!last && p.cap_dst[h + 1] < p.cap_uniq) ? p.cap_dst[h + 1] : p.cap_uniq;
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
-                                  d_counts + h + 1, d_uniq, grow_to,
-                                  idmap_flags | (h == n_hops - 1 ? FGL_IDMAP_FINAL : 0), d_status, ws + ws_sample,
-                                  ws_bytes - ws_sample, s, /*counter_is_zeroed=*/true);
+                                  d_counts + h + 1, d_uniq, grow_to, order | (last ? FGL_IDMAP_FINAL : 0), d_status,
+                                  ws.idmap_ws, p.idmap_bytes, s, /*counter_is_zeroed=*/true, last ? nullptr : &next,
+                                  /*leave_table_empty=*/last && leave_empty, ws.lowered);
         if (rc != FGL_OK) return rc;
     }
     return FGL_OK;

@@ -20,7 +20,7 @@
 //   3. prefix     single workgroup over the tile counts; publishes the new node total
 //                 (the edge-parallel launches are grid-stride loops over the actual count,
 //                 so a bound much larger than the batch costs nothing).  Skipped while the bound
-//                 is at most 1024 tiles (2 M edges): the number pass then scans the tile counts
+//                 is at most 2048 tiles (4 M edges): the number pass then scans the tile counts
 //                 itself in every workgroup, and its first workgroup publishes the total
 //   4. number     per edge, coalesced: the local id follows from the first-edge index that the mark
 //                 pass left for the edge and the three counts (cache-resident arrays): no table read.
@@ -29,92 +29,12 @@
 //                 will not consult the table again (the last hop of a mini-batch: most of its edges).
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
+#include "fgl_table.hpp"
 
 namespace fgl {
 
-constexpr uint32_t kEmpty = 0xFFFFFFFFu;
-constexpr uint32_t kDone = 0xFFFFFFFEu;  // slot_of[] marker: the edge already has its local id
-constexpr uint32_t kPending = 0x80000000u;  // val = kPending | first edge index until the id is numbered
-constexpr uint32_t kHashMul = 0x9E3779B1u;
 constexpr int kItems = 8;
 constexpr int kTile = kBlock * kItems;
-
-struct TableRef {
-    uint32_t* words;  // 2 per slot: key, val
-    uint32_t mask;
-    int shift;
-};
-
-static inline int log2_slots(int64_t slots)
-{
-    int lg = 0;
-    while (((int64_t)1 << lg) < slots) ++lg;
-    return lg;
-}
-
-static inline bool valid_slots(int64_t slots) { return slots >= 64 && slots <= ((int64_t)1 << 31) && (slots & (slots - 1)) == 0; }
-
-static inline TableRef make_ref(void* d_table, int64_t slots)
-{
-    TableRef t;
-    t.words = static_cast<uint32_t*>(d_table);
-    t.mask = (uint32_t)(slots - 1);
-    t.shift = 32 - log2_slots(slots);
-    return t;
-}
-
-// A probe sequence longer than this is reported as "table full" (at load <= 1/2 with this
-// hash, sequences stay far below it), which also bounds the time a mis-sized table can cost.
-constexpr uint32_t kMaxProbes = 4096;
-
-// Finds the slot of `id`, inserting {id, val_if_new} if absent; if the key is already there,
-// lowers its val to `val_if_new` when that is smaller (val_if_new = 0xFFFFFFFF: leave it).
-// Returns kEmpty if the table is full.
-//
-// One 8-byte load per probe reads key and val together.  Keys only ever change from empty to a
-// key and vals only ever decrease while inserts run, so an ordinary (cacheable, possibly stale)
-// load is enough for the first look: a stale "empty" is settled by the 64-bit CAS, which
-// installs key and val in one atomic, and a stale val can only cause a redundant atomicMin.
-// *seen_val receives the val found with the key (val_if_new if this call installed the key).
-__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new, uint32_t* seen_val)
-{
-    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
-    const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)val_if_new << 32);
-    uint32_t p = (id * kHashMul) >> t.shift;
-    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
-    for (uint32_t n = 0; n < limit; ++n) {
-        unsigned long long s = slots[p];
-        if ((uint32_t)s == kEmpty) {
-            const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
-            if (seen == ~0ull) {
-                *seen_val = val_if_new;
-                return p;
-            }
-            s = seen;
-        }
-        if ((uint32_t)s == id) {
-            *seen_val = (uint32_t)(s >> 32);
-            if (*seen_val > val_if_new) atomicMin(&t.words[2 * (size_t)p + 1], val_if_new);
-            return p;
-        }
-        p = (p + 1) & t.mask;
-    }
-    return kEmpty;
-}
-
-// Finds the slot of `id` without inserting.  kEmpty if absent.
-__device__ __forceinline__ uint32_t find_only(const uint32_t* __restrict__ words, uint32_t mask, int shift, uint32_t id)
-{
-    uint32_t p = (id * kHashMul) >> shift;
-    const uint32_t limit = mask < kMaxProbes ? mask + 1 : kMaxProbes;
-    for (uint32_t n = 0; n < limit; ++n) {
-        const uint32_t k = words[2 * (size_t)p];
-        if (k == id) return p;
-        if (k == kEmpty) return kEmpty;
-        p = (p + 1) & mask;
-    }
-    return kEmpty;
-}
 
 __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, const int32_t* __restrict__ ids,
                                                                   int64_t n_max, const int32_t* __restrict__ d_n,
@@ -125,15 +45,66 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, co
     if (i >= n) return;
     const int32_t id = ids[i];
     if (uniq != nullptr && uniq != ids) uniq[i] = id;
+    if (id < 0) {  // not a node id (and -1 would read as the empty marker): reported, never inserted
+        if (d_status) atomicOr(d_status, FGL_STATUS_BAD_ID);
+        return;
+    }
     uint32_t seen;
     const uint32_t p = find_or_insert(t, (uint32_t)id, (uint32_t)i, &seen);  // a repeated id keeps its first position
     if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
 }
 
+constexpr uint32_t kHolderBit = 0x80000000u;  // slot_of[]: the edge was the first known mention of its id when its insert ran
+
+// find_or_insert for an edge's source id, which also says what the mark pass would otherwise have to read back
+// from the table: *holder = this edge became the first known mention of the id (it installed the key, or lowered
+// the key's first-edge index to its own); *displaced = the pending value it took that place from (kEmpty: none).
+// An edge that became holder and is never displaced is the id's first mention.
+__device__ __forceinline__ uint32_t insert_mention(const TableRef t, uint32_t id, uint32_t mine, uint32_t* seen_val,
+                                                   bool* holder, uint32_t* displaced)
+{
+    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
+    const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)mine << 32);
+    uint32_t p = (id * kHashMul) >> t.shift;
+    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
+    *holder = false;
+    *displaced = kEmpty;
+    for (uint32_t n = 0; n < limit; ++n) {
+        unsigned long long s = slots[p];
+        if ((uint32_t)s == kEmpty) {
+            const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
+            if (seen == ~0ull) {
+                *seen_val = mine;
+                *holder = true;
+                return p;
+            }
+            s = seen;
+        }
+        if ((uint32_t)s == id) {
+            const uint32_t v = (uint32_t)(s >> 32);
+            *seen_val = v;
+            if ((v & kPending) && v > mine) {
+                const uint32_t old = atomicMin(&t.words[2 * (size_t)p + 1], mine);
+                if (old > mine) {  // (else an even earlier mention got there between the load and the atomic)
+                    *holder = true;
+                    *displaced = old;
+                }
+            }
+            return p;
+        }
+        p = (p + 1) & t.mask;
+    }
+    return kEmpty;
+}
+
 // `src` and `out` may be the same array (relabelling in place): neither is __restrict__.
+// lowered (may be null; one byte per edge, zero on entry): lowered[e] is set when a later-running insert takes the
+// place of edge e as its id's first known mention.  Together with the holder bit in slot_of[] it tells the mark pass
+// which edges are first mentions without a look at the table.
 __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* src,
                                                                   int64_t e_max, const int32_t* __restrict__ d_e,
                                                                   uint32_t* __restrict__ slot_of, int32_t* out,
+                                                                  uint8_t* __restrict__ lowered,
                                                                   uint32_t* __restrict__ d_status)
 {
     const int64_t n_e = actual_count(e_max, d_e);
@@ -141,15 +112,22 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         // ids numbered earlier hold a local id (no pending bit) and stay as they are; a new id keeps
         // the smallest pending edge index among the edges that mention it
-        uint32_t seen;
-        uint32_t p = find_or_insert(t, (uint32_t)src[e], kPending | (uint32_t)e, &seen);
+        uint32_t seen = 0, displaced = kEmpty;
+        bool holder = false;
+        const int32_t id = src[e];
+        uint32_t p = id >= 0 ? insert_mention(t, (uint32_t)id, kPending | (uint32_t)e, &seen, &holder, &displaced) : kEmpty;
         if (p == kEmpty) {
-            if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+            // table full, or not a node id: reported; the edge's local id becomes -1 (written by the number pass)
+            if (d_status) atomicOr(d_status, id >= 0 ? FGL_STATUS_TABLE_FULL : FGL_STATUS_BAD_ID);
         } else if (!(seen & kPending)) {
             // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
             // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
             out[e] = (int32_t)seen;
             p = kDone;
+        } else if (lowered != nullptr) {
+            if (holder) p |= kHolderBit;
+            // (a pending value left over from an earlier call's overflow may name an edge beyond this call's)
+            if ((displaced & kPending) && displaced != kEmpty && (int64_t)(displaced & ~kPending) < n_e) lowered[displaced & ~kPending] = 1;
         }
         slot_of[e] = p;
     }
@@ -162,6 +140,7 @@ __device__ __forceinline__ int64_t tiles_of(int64_t n) { return (n + kTile - 1) 
 // first_of[e] = pending | index of the first edge that mentions e's id (edges that take part only)
 __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t e_max, const int32_t* __restrict__ d_e,
                                                             const uint32_t* __restrict__ slot_of,
+                                                            const uint8_t* __restrict__ lowered,
                                                             uint32_t* __restrict__ first_of,
                                                             uint8_t* __restrict__ flags8, uint16_t* __restrict__ before8,
                                                             int32_t* __restrict__ tile_sums)
@@ -182,9 +161,31 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
 #pragma unroll
             for (int j = 0; j < kItems; ++j) p[j] = (first + j < n_e) ? slot_of[first + j] : kEmpty;
         }
+        // An edge that became its id's first known mention when it was inserted and was not displaced afterwards
+        // is the first mention: nothing to read.  The others (an eighth of the edges of a large hop, where the
+        // inserts run nearly in edge order) read what the slot holds now.
+        uint32_t low[kItems];
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) low[j] = 1u;  // without the bookkeeping: every edge reads its slot
+        if (lowered != nullptr) {
+            if (whole) {
+                const uint2 b = *reinterpret_cast<const uint2*>(lowered + first);
+#pragma unroll
+                for (int j = 0; j < kItems; ++j) low[j] = ((j < 4 ? b.x : b.y) >> (8 * (j & 3))) & 0xFFu;
+            } else {
+#pragma unroll
+                for (int j = 0; j < kItems; ++j) low[j] = (first + j < n_e) ? lowered[first + j] : 1u;
+            }
+        }
         uint32_t v[kItems];
 #pragma unroll
-        for (int j = 0; j < kItems; ++j) v[j] = (p[j] < kDone) ? t.words[2 * (size_t)p[j] + 1] : 0u;
+        for (int j = 0; j < kItems; ++j) {
+            v[j] = 0u;
+            if (p[j] < kDone) {
+                if ((p[j] & kHolderBit) && low[j] == 0u) v[j] = kPending | (uint32_t)(first + j);
+                else v[j] = t.words[2 * (size_t)(p[j] & ~kHolderBit) + 1];
+            }
+        }
         uint32_t bits = 0;
 #pragma unroll
         for (int j = 0; j < kItems; ++j)
@@ -246,8 +247,63 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
 // Up to this many tiles the number pass scans the tile counts itself (every workgroup, into LDS) and
 // its first workgroup publishes the node total: one launch less per call where launches, not
 // edges, set the time.  Above it the single-workgroup prefix launch prepares the array once.
-constexpr int kSelfTilesPerLane = 4;
+constexpr int kSelfTilesPerLane = 8;
+#ifndef FGL_NUMBER_SELF_MAX_BLOCKS
+#define FGL_NUMBER_SELF_MAX_BLOCKS 1024
+#endif
 constexpr int kIdmapSelfPrefixTiles = kBlock * kSelfTilesPerLane;
+
+// A node that has just been given position `local` in the unique list is a seed of the next hop: its row start
+// and degree go to that position.  Returns its min(fanout, degree), which the caller adds to the next hop's
+// per-tile edge counts (entry local / tile_seeds).  An id outside the graph is marked for the next hop's
+// sampling kernel to report.
+__device__ __forceinline__ int prepare_next_hop(const NextHop& next, int32_t id, int64_t local)
+{
+    int64_t a = kRowBadId, deg = 0;
+    if (id >= 0 && (int64_t)id < next.n_nodes) {
+        if (next.is64) {
+            const int64_t* p = static_cast<const int64_t*>(next.indptr);
+            a = p[id];
+            deg = p[id + 1] - a;
+        } else {
+            const int32_t* p = static_cast<const int32_t*>(next.indptr);
+            a = p[id];
+            deg = (int64_t)p[id + 1] - a;
+        }
+        if (deg < 0) deg = 0;
+        if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
+    }
+    next.row_start[local] = a;
+    next.deg[local] = (int32_t)deg;
+    return deg < next.fanout ? (int)deg : next.fanout;
+}
+
+// The new nodes that the lanes of a wave number in one step have consecutive positions (a position is a count of
+// earlier new nodes, and the lanes hold consecutive edges), so their tiles of the next hop are at most two:
+// one atomic per tile and wave instead of one per node -- updates of one address run one after the other, and a
+// tile's 256 nodes would otherwise queue up on it.  k = 0 for lanes without a new node.  Every lane of the wave
+// must call this.
+__device__ __forceinline__ void add_next_tile_sums(const NextHop& next, int k, int tile)
+{
+    if (__ballot(k != 0) == 0) return;  // uniform
+    int tmin = k != 0 ? tile : 0x7FFFFFFF;
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) {
+        const int o = __shfl_xor(tmin, d, kWave);
+        tmin = o < tmin ? o : tmin;
+    }
+    int s0 = (k != 0 && tile == tmin) ? k : 0;
+    int s1 = (k != 0 && tile != tmin) ? k : 0;
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) {
+        s0 += __shfl_xor(s0, d, kWave);
+        s1 += __shfl_xor(s1, d, kWave);
+    }
+    if (lane_id() == 0) {
+        atomicAdd(&next.tile_sums[tmin], s0);
+        if (s1 != 0) atomicAdd(&next.tile_sums[tmin + 1], s1);
+    }
+}
 
 // Lane per edge, coalesced.  `src` and `out` may be the same array: an entry is read and written by one lane only.
 // (Edges whose id was numbered before this call were relabelled by the insert pass.)  The local id of an
@@ -268,7 +324,8 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                                                               const int32_t* __restrict__ tile_prefix,
                                                               int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
                                                               int32_t* __restrict__ d_n_total_out,
-                                                              uint32_t* __restrict__ d_status)
+                                                              uint32_t* __restrict__ d_status, const NextHop next,
+                                                              uint32_t* __restrict__ clear_words, int64_t n_clear_words)
 {
     __shared__ int s_prefix[SELF ? kIdmapSelfPrefixTiles : 1];
     __shared__ int smem[kBlock / kWave + 1];
@@ -295,24 +352,41 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
         if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status);
     }
     const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
-        const uint32_t p = slot_of[e];
-        if (p == kDone) continue;
-        int64_t local = -1;
-        if (p != kEmpty) {
-            const int64_t ef = (int64_t)(first_of[e] & ~kPending);  // first edge of this edge's id (ef <= e)
-            if (ef < n_e) {
-                const int64_t tile = ef / kTile;
-                const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
-                local = n_base + before_tile + before8[ef >> 3] + __popc((uint32_t)flags8[ef >> 3] & ((1u << (ef & 7)) - 1u));
+    // the last pass of a mini-batch, which no longer reads the table, can leave it empty for the next one
+    // (first, so that the stores drain while the edges are being numbered)
+    if (!WRITE_BACK && clear_words != nullptr) {
+        uint4* v = reinterpret_cast<uint4*>(clear_words);  // (a table is 8-byte slots, a power of two of them, 16-byte aligned)
+        const uint4 empty = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
+        for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_clear_words / 4; i += stride) v[i] = empty;
+    }
+    // (the trip count is the same for all lanes of a wave: they add up their next-hop tile sums together)
+    for (int64_t base = (int64_t)blockIdx.x * kBlock; base < n_e; base += stride) {
+        const int64_t e = base + threadIdx.x;
+        int next_k = 0, next_tile = 0;
+        const uint32_t p = e < n_e ? slot_of[e] : kDone;
+        if (p != kDone) {
+            int64_t local = -1;
+            if (p != kEmpty) {
+                const int64_t ef = (int64_t)(first_of[e] & ~kPending);  // first edge of this edge's id (ef <= e)
+                if (ef < n_e) {
+                    const int64_t tile = ef / kTile;
+                    const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
+                    local = n_base + before_tile + before8[ef >> 3] + __popc((uint32_t)flags8[ef >> 3] & ((1u << (ef & 7)) - 1u));
+                }
+                if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
+                if (ef == e && local >= 0) {
+                    const int32_t id = src[e];
+                    uniq[local] = id;
+                    if (WRITE_BACK) t.words[2 * (size_t)(p & ~kHolderBit) + 1] = (uint32_t)local;
+                    if (next.row_start != nullptr) {
+                        next_k = prepare_next_hop(next, id, local);
+                        next_tile = (int)(local / next.tile_seeds);
+                    }
+                }
             }
-            if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
-            if (ef == e && local >= 0) {
-                uniq[local] = src[e];
-                if (WRITE_BACK) t.words[2 * (size_t)p + 1] = (uint32_t)local;
-            }
+            out[e] = (int32_t)local;
         }
-        out[e] = (int32_t)local;
+        if (next.row_start != nullptr) add_next_tile_sums(next, next_k, next_tile);
     }
 }
 
@@ -347,10 +421,12 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                                                                       int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                       uint32_t* __restrict__ slot_of, int32_t* __restrict__ counter,
                                                                       int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
-                                                                      uint32_t* __restrict__ d_status)
+                                                                      uint32_t* __restrict__ d_status, const NextHop next)
 {
     __shared__ int smem[kBlock / kWave + 1];
     __shared__ int s_base;
+    constexpr int kNextTiles = kBlock * ITEMS / kWave + 2;  // next-hop tiles (64 seeds or more each) that a tile's new nodes can touch
+    __shared__ int s_next[kNextTiles];
     unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
@@ -376,7 +452,8 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                 id[j] = (uint32_t)src[e];
                 p[j] = kEmpty;
                 uint32_t q = (id[j] * kHashMul) >> t.shift;
-                for (uint32_t n = 0; n < limit; ++n) {
+                // (a negative id is not a node id -- and -1 would read as the empty marker: no probe, reported below)
+                for (uint32_t n = 0; n < ((int32_t)id[j] >= 0 ? limit : 0u); ++n) {
                     unsigned long long slot = slots[q];
                     if ((uint32_t)slot == kEmpty) {
                         // the key goes in with val still all ones = "not numbered yet"
@@ -402,13 +479,15 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                 }
                 if (p[j] == kEmpty) {
                     out[e] = -1;
-                    if (d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
+                    if (d_status) atomicOr(d_status, (int32_t)id[j] >= 0 ? FGL_STATUS_TABLE_FULL : FGL_STATUS_BAD_ID);
                 }
             }
         }
         int total;
         int rank = block_exclusive_scan<kBlock>(__popc(won), smem, &total);
         if (threadIdx.x == 0) s_base = total ? atomicAdd(counter, total) : 0;
+        if (next.row_start != nullptr)
+            for (int i = threadIdx.x; i < kNextTiles; i += kBlock) s_next[i] = 0;
         __syncthreads();
         const int64_t base = n_base + s_base;
 #pragma unroll
@@ -420,6 +499,11 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                     t.words[2 * (size_t)p[j] + 1] = (uint32_t)local;
                     uniq[local] = (int32_t)id[j];
                     out[e] = (int32_t)local;
+                    if (next.row_start != nullptr) {
+                        // (the tile's new nodes have consecutive positions: few next-hop tiles, summed in LDS first)
+                        const int k = prepare_next_hop(next, (int32_t)id[j], local);
+                        if (k != 0) atomicAdd(&s_next[(int)(local / next.tile_seeds - base / next.tile_seeds)], k);
+                    }
                 } else {
                     out[e] = -1;  // the unique list is full (reported by the second pass); val stays "not numbered"
                 }
@@ -428,6 +512,11 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
             if (e < n_e) slot_of[e] = p[j];
         }
         __syncthreads();
+        if (next.row_start != nullptr) {
+            for (int i = threadIdx.x; i < kNextTiles; i += kBlock)
+                if (s_next[i] != 0) atomicAdd(&next.tile_sums[base / next.tile_seeds + i], s_next[i]);
+            __syncthreads();  // s_next is cleared again at the top of the next tile
+        }
     }
 }
 
@@ -505,7 +594,8 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
 int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out, int64_t n_edges_max,
                          const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base, int32_t* d_n_total_out,
                          int32_t* d_uniq, int64_t uniq_capacity, int flags, uint32_t* d_status, void* d_ws,
-                         size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed)
+                         size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed, const NextHop* next_hop,
+                         bool leave_table_empty, uint8_t* d_lowered)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
@@ -528,8 +618,11 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     int32_t* sums = c.take<int32_t>((size_t)tiles);
     int32_t* prefix = c.take<int32_t>((size_t)tiles);
     const TableRef t = make_ref(d_table, slots);
-    const unsigned edge_blocks = stride_grid(n_edges_max, kBlock);
+    unsigned edge_blocks = stride_grid(n_edges_max, kBlock);
     const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
+    NextHop next{};  // all null: nothing to prepare
+    if (next_hop != nullptr) next = *next_hop;
+    FGL_REQUIRE(!leave_table_empty || final_call, "idmap_map_src: only a final call can leave the table empty");
 
     if (flags & FGL_IDMAP_ARRIVAL) {
         // the counter of new ids: *d_n_total_out itself when the caller vouches that it holds zero (the all-hops
@@ -544,28 +637,42 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
             hipLaunchKernelGGL(idmap_insert_arrival_kernel<kArrivalItems>, dim3(stride_grid(n_edges_max, kBlock * kArrivalItems)),
                                dim3(kBlock), 0, stream, t, d_src_in,
                                n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
-                               d_status);
+                               d_status, next);
         else
             hipLaunchKernelGGL(idmap_insert_arrival_kernel<1>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
                                n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
-                               d_status);
+                               d_status, next);
         FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
         hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
                            slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
         FGL_CHECK_LAUNCH("idmap_relabel_publish_kernel");
+        // (the second pass reads the table, so emptying it takes a launch of its own here)
+        if (leave_table_empty) return launch_fill_u32(t.words, slots * 2, kEmpty, stream);
         return FGL_OK;
     }
 
+    // (the holder bit shares a word with the slot index: tables of 2^31 slots go without the bookkeeping)
+    uint8_t* lowered = slots <= ((int64_t)1 << 30) ? d_lowered : nullptr;
     hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
-                       n_edges_max, d_n_edges, slot_of, d_src_out, d_status);
+                       n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                       slot_of, first_of, flags8, before8, sums);
+                       slot_of, lowered, first_of, flags8, before8, sums);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
 #define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS)                                                              \
     hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
-                       uniq_capacity, d_src_out, TOTAL, STATUS)
+                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words)
+    // emptying the table rides on the last pass: enough workgroups for a fill of that size
+    uint32_t* clear_words = leave_table_empty ? t.words : nullptr;
+    const int64_t n_clear_words = leave_table_empty ? slots * 2 : 0;
+    if (leave_table_empty) {
+        const unsigned fill_blocks = stride_grid(n_clear_words, kBlock * 8);
+        if (fill_blocks > edge_blocks) edge_blocks = fill_blocks;
+    }
+    // every workgroup of a pass that scans the tile counts itself pays for that scan once: a few workgroups per
+    // compute unit, each looping over several tiles of edges, instead of one per 256 edges
+    if (tiles <= kIdmapSelfPrefixTiles && edge_blocks > FGL_NUMBER_SELF_MAX_BLOCKS) edge_blocks = FGL_NUMBER_SELF_MAX_BLOCKS;
     if (tiles <= kIdmapSelfPrefixTiles) {
         if (final_call) FGL_LAUNCH_NUMBER(true, false, nullptr, d_n_total_out, d_status);
         else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status);
@@ -623,7 +730,8 @@ FGL_EXPORT int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_
                                  uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream)
 {
     return launch_idmap_map_src(d_table, slots, d_src_in, d_src_out, n_edges_max, d_n_edges, n_base, d_n_base,
-                                d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream), false);
+                                d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream), false,
+                                nullptr, false, nullptr);
 }
 
 FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,

@@ -16,8 +16,35 @@ int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_pref
                        hipStream_t stream);
 int launch_fill_u32(uint32_t* p, int64_t n, uint32_t value, hipStream_t stream);
 
+// Row start of a node whose id lies outside the graph / whose insert found the table full: how a launch that
+// must not touch the status word hands the error to the next one that reads the entry.
+constexpr int64_t kRowBadId = -1;
+constexpr int64_t kRowTableFull = -2;
+
+// What a pass over a hop's nodes prepares for the sampling of the next hop: row start and degree of every node
+// at its position in the unique list, and the per-tile sums of min(fanout, degree) that place the tiles' output.
+struct NextHop {
+    const void* indptr;
+    int is64;
+    int64_t n_nodes;
+    int64_t* row_start;
+    int32_t* deg;
+    int32_t* tile_sums;  // zeroed by the caller; [position / tile_seeds] += min(fanout, degree)
+    int fanout;
+    int tile_seeds;
+};
+
 // neighbour sampling (fgl_sample.hip)
+int sample_tile_seeds(int fanout, int64_t n_seeds_max);
+int64_t sample_tile_count(int64_t n_seeds_max, int fanout);
 size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout);
+// the second half of launch_sample, for callers that hold row starts, degrees and tile sums already
+int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds,
+                        int fanout, const int64_t* row_start, const int32_t* deg, const int32_t* tile_sums,
+                        int32_t* tile_prefix, uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out,
+                        int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
+                        hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next,
+                        uint8_t* d_zero_per_edge = nullptr);  // (optional) one byte per output edge, cleared along with the writes
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
@@ -33,7 +60,10 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          int64_t n_edges_max, const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base,
                          int32_t* d_n_total_out, int32_t* d_uniq, int64_t uniq_capacity, int flags,
                          uint32_t* d_status, void* d_ws, size_t ws_bytes, hipStream_t stream,
-                         bool counter_is_zeroed = false);  // arrival order: *d_n_total_out holds zero and may count the new ids
+                         bool counter_is_zeroed,          // arrival order: *d_n_total_out holds zero and may count the new ids
+                         const NextHop* next_hop,         // (may be null) the new nodes are seeds of a next hop: prepare its sampling
+                         bool leave_table_empty,          // final calls only: every slot of the table is empty when the call's work is done
+                         uint8_t* d_lowered);             // (may be null) n_edges_max bytes, zero on entry: lets the mark pass skip most table reads
 
 // deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
 size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);

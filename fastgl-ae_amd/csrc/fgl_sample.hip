@@ -126,6 +126,34 @@ __device__ __forceinline__ void publish_empty(const int32_t* __restrict__ tile_p
     }
 }
 
+// Two things the edges kernels do for every seed besides sampling it.
+// (1) A negative row start is how the launch that prepared the seed's row start and degree (the first launch
+// of a mini-batch, or the id-map pass that numbered the node) says that something was wrong with it; it
+// is reported here, where the status word is no longer being initialised, and the seed gets no edges.
+// (2) The seeds of this hop are also the first seeds of the next one (a hop's nodes are a prefix of the next
+// hop's): their share of the next hop's per-tile edge counts, sum of min(next fanout, degree), is added
+// here -- one integer atomic per wave, order-independent -- so that the next hop needs no pass of its own
+// over degrees.  Call from uniform control flow (all lanes of the workgroup).
+template <int TS>
+__device__ __forceinline__ void seed_checks_and_next_hop(bool valid, int64_t tile, int64_t& row, int& deg,
+                                                         uint32_t* __restrict__ d_status, int next_fanout,
+                                                         int next_tile_seeds, int32_t* __restrict__ next_tile_sums)
+{
+    if (valid && row < 0) {
+        if (d_status) atomicOr(d_status, row == kRowBadId ? FGL_STATUS_BAD_SEED : FGL_STATUS_TABLE_FULL);
+        row = 0;
+        deg = 0;
+    }
+    if (next_tile_sums != nullptr) {
+        int kn = valid ? (deg < next_fanout ? deg : next_fanout) : 0;
+#pragma unroll
+        for (int d = kWave / 2; d >= 1; d >>= 1) kn += __shfl_xor(kn, d, kWave);
+        // (tiles are multiples of the wave size: a wave's seeds lie in one tile of the next hop)
+        if (lane_id() == 0 && kn != 0)
+            atomicAdd(&next_tile_sums[(tile * TS + (int64_t)(threadIdx.x / kWave) * kWave) / next_tile_seeds], kn);
+    }
+}
+
 template <int TS, int U>
 __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restrict__ indices,
                                                           const int32_t* __restrict__ seeds, int64_t n_max,
@@ -137,7 +165,9 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                                                           uint32_t seed_hi, uint32_t stream_id,
                                                           const uint32_t* __restrict__ d_stream_add,
                                                           int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
-                                                          int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+                                                          int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
+                                                          uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
+                                                          int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge)
 {
     extern __shared__ uint32_t s_sel[];  // [fanout][TS] picked positions
     __shared__ int s_scan[TS / kWave + 1];
@@ -160,6 +190,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
             row = row_start[i];
             seed = seeds[i];
         }
+        seed_checks_and_next_hop<TS>(i < n, tile, row, deg, d_status, next_fanout, next_tile_seeds, next_tile_sums);
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
@@ -214,6 +245,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                 if (x < total) {
                     src_out[(int64_t)base + x] = got[u];
                     if (dst_out) dst_out[(int64_t)base + x] = seed_of[u];
+                    if (zero_per_edge) zero_per_edge[(int64_t)base + x] = 0;
                 }
             }
         }
@@ -236,7 +268,9 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
                                                               uint32_t seed_hi, uint32_t stream_id,
                                                               const uint32_t* __restrict__ d_stream_add,
                                                               int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
-                                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+                                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
+                                                              uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
+                                                              int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge)
 {
     extern __shared__ int32_t s_stage[];  // [TS*fanout] sampled ids (+ [TS*fanout] seed ids when dst_out is wanted)
     __shared__ int s_scan[TS / kWave + 1];
@@ -257,6 +291,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
             row = row_start[i];
             seed = seeds[i];
         }
+        seed_checks_and_next_hop<TS>(i < n, tile, row, deg, d_status, next_fanout, next_tile_seeds, next_tile_sums);
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
@@ -296,12 +331,23 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
         for (int x = tid; x < total; x += TS) {
             src_out[(int64_t)base + x] = s_val[x];
             if (dst_out) dst_out[(int64_t)base + x] = s_dst[x];
+            if (zero_per_edge) zero_per_edge[(int64_t)base + x] = 0;
         }
         __syncthreads();  // the staging area is reused by the next tile
     }
 }
 
-static inline int tile_seeds_for(int fanout) { return fanout <= 48 ? 256 : 64; }
+// Seeds per workgroup of the sampling kernels.  Small hops take one wave per tile: a hop of a few ten thousand
+// seeds is a chain of latencies, and 64-seed tiles spread it over four times the compute units.
+#ifndef FGL_SMALL_HOP_SEEDS
+#define FGL_SMALL_HOP_SEEDS 65536
+#endif
+int sample_tile_seeds(int fanout, int64_t n_seeds_max) { return (fanout <= 48 && n_seeds_max > FGL_SMALL_HOP_SEEDS) ? 256 : 64; }
+
+int64_t sample_tile_count(int64_t n_seeds_max, int fanout)
+{
+    return ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, sample_tile_seeds(fanout, n_seeds_max));
+}
 
 // Up to this many tiles of seeds the edges kernel derives its tile offsets itself (at most 16 KiB of
 // tile sums per workgroup, read from L2); above it a scan launch prepares them.
@@ -309,8 +355,7 @@ constexpr int64_t kSampleSelfPrefixTiles = 4096;
 
 size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
 {
-    const int ts = tile_seeds_for(fanout);
-    const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, ts);
+    const int64_t tiles = sample_tile_count(n_seeds_max, fanout);
     Carver c(nullptr);
     c.take<int64_t>((size_t)n_seeds_max);
     c.take<int32_t>((size_t)n_seeds_max);
@@ -320,23 +365,14 @@ size_t sample_workspace_bytes(int64_t n_seeds_max, int fanout)
 }
 
 template <int TS>
-static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
-                            const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
-                            uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
-                            int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws,
-                            hipStream_t stream, const uint32_t* d_stream_add)
+static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds,
+                           int fanout, const int64_t* row_start, const int32_t* deg, const int32_t* sums, int32_t* prefix,
+                           uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
+                           int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, hipStream_t stream,
+                           const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge)
 {
     const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, TS);
-    Carver c(d_ws);
-    int64_t* row_start = c.take<int64_t>((size_t)n_seeds_max);
-    int32_t* deg = c.take<int32_t>((size_t)n_seeds_max);
-    int32_t* sums = c.take<int32_t>((size_t)tiles);
-    int32_t* prefix = c.take<int32_t>((size_t)tiles);
-
     const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
-    hipLaunchKernelGGL(sample_degree_kernel<TS>, dim3(grid), dim3(TS), 0, stream, d_indptr, indptr_is64,
-                       n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
-    FGL_CHECK_LAUNCH("sample_degree_kernel");
     // few tiles: each workgroup of the edges kernel sums the earlier tile sums itself (the last one
     // publishes the totals), which saves the scan launch in between
     if (tiles > kSampleSelfPrefixTiles) {
@@ -346,14 +382,18 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
     } else {
         prefix = nullptr;
     }
+    const int next_fanout = next ? next->fanout : 0;
+    const int next_ts = next ? next->tile_seeds : TS;
+    int32_t* next_sums = next ? next->tile_sums : nullptr;
     // the register variant stages the tile's output (and, if wanted, the seed ids) in LDS: it is used
     // while that fits comfortably in the 64 KiB a workgroup may take
     const size_t lds_reg = (size_t)fanout * TS * sizeof(int32_t) * (d_dst_out ? 2 : 1);
-    if constexpr (TS == 256) if (fanout <= 32 && lds_reg <= 60 * 1024) {
+    if (fanout <= 32 && lds_reg <= 60 * 1024) {
 #define FGL_LAUNCH_REG(F)                                                                                           \
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out)
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, \
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge)
         if (fanout <= 8) FGL_LAUNCH_REG(8);
         else if (fanout <= 16) FGL_LAUNCH_REG(16);
         else FGL_LAUNCH_REG(32);
@@ -362,14 +402,27 @@ static int launch_sample_ts(const void* d_indptr, int indptr_is64, const int32_t
         return FGL_OK;
     }
     const size_t lds = (size_t)fanout * TS * sizeof(uint32_t);
-#define FGL_LAUNCH_EDGES(U)                                                                                        \
-    hipLaunchKernelGGL((sample_edges_kernel<TS, U>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,          \
-                       n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
-                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out)
-    FGL_LAUNCH_EDGES(16);
-#undef FGL_LAUNCH_EDGES
+    hipLaunchKernelGGL((sample_edges_kernel<TS, 16>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,
+                       n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,
+                       (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out,
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge);
     FGL_CHECK_LAUNCH("sample_edges_kernel");
     return FGL_OK;
+}
+
+int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds,
+                        int fanout, const int64_t* row_start, const int32_t* deg, const int32_t* tile_sums,
+                        int32_t* tile_prefix, uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out,
+                        int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
+                        hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge)
+{
+    if (sample_tile_seeds(fanout, n_seeds_max) == 256)
+        return launch_edges_ts<256>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
+                                    rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
+                                    d_stream_add, next, d_zero_per_edge);
+    return launch_edges_ts<64>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
+                               rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
+                               d_stream_add, next, d_zero_per_edge);
 }
 
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
@@ -388,13 +441,24 @@ int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indice
         set_error("sample_node: workspace too small (%zu < %zu)", ws_bytes, sample_workspace_bytes(n_seeds_max, fanout));
         return FGL_ERR_WORKSPACE;
     }
-    if (tile_seeds_for(fanout) == 256)
-        return launch_sample_ts<256>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
-                                     rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status,
-                                     d_ws, stream, d_stream_add);
-    return launch_sample_ts<64>(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout,
-                                rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws,
-                                stream, d_stream_add);
+    const int ts = sample_tile_seeds(fanout, n_seeds_max);
+    const int64_t tiles = sample_tile_count(n_seeds_max, fanout);
+    Carver c(d_ws);
+    int64_t* row_start = c.take<int64_t>((size_t)n_seeds_max);
+    int32_t* deg = c.take<int32_t>((size_t)n_seeds_max);
+    int32_t* sums = c.take<int32_t>((size_t)tiles);
+    int32_t* prefix = c.take<int32_t>((size_t)tiles);
+    const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    if (ts == 256)
+        hipLaunchKernelGGL(sample_degree_kernel<256>, dim3(grid), dim3(256), 0, stream, d_indptr, indptr_is64, n_nodes, d_seeds,
+                           n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
+    else
+        hipLaunchKernelGGL(sample_degree_kernel<64>, dim3(grid), dim3(64), 0, stream, d_indptr, indptr_is64, n_nodes, d_seeds,
+                           n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, d_status);
+    FGL_CHECK_LAUNCH("sample_degree_kernel");
+    return launch_sample_edges(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, rng_seed,
+                               stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream, d_stream_add,
+                               nullptr, nullptr);
 }
 
 }  // namespace fgl

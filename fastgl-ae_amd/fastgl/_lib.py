@@ -19,9 +19,10 @@ CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
 F32, BF16 = 0, 1
 AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE = 0, 1, 2, 3, 4
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
-ABI_VERSION = 6  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
-STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED = 1, 2, 4, 8
+ABI_VERSION = 7  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
+STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL = 0, 1, 2
+BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
 MAX_FANOUT = 192
 
 _i64, _i32, _u64, _u32, _vp, _sz = C.c_int64, C.c_int, C.c_uint64, C.c_uint32, C.c_void_p, C.c_size_t
@@ -124,4 +125,6 @@ def status_message(bits: int) -> str:
         names.append("an id to relabel is not in the map")
     if bits & STATUS_BAD_SEED:
         names.append("a seed id lies outside the graph")
+    if bits & STATUS_BAD_ID:
+        names.append("a negative id was handed to the id-map")
     return ", ".join(names) or "ok"

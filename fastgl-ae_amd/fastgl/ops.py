@@ -435,6 +435,8 @@ class BlocksPlan:
         self.cap_uniq, self.slots, self.ws_bytes = cap_uniq.value, slots.value, ws_bytes.value
         self.table = torch.empty(self.slots, dtype=torch.int64, device=self.device)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=self.device)
+        # the slot count that the last call on this plan's table left empty (None: unknown contents)
+        self.empty_slots = None
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
@@ -473,12 +475,19 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
                       for h in range(H)]
         counts = torch.empty(2 * H + 2, dtype=torch.int32, device=dev)
         arr = lambda ts: (C.c_void_p * H)(*[L.ptr(t) for t in ts])
+        # every call leaves the table empty for the next one (its last pass no longer reads it), so only a
+        # plan's first call -- or the first after a failed one, or with another slot count -- pays for a fill
+        flags = {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order] | L.BLOCKS_LEAVE_TABLE_EMPTY
+        if plan.empty_slots == slots:
+            flags |= L.BLOCKS_TABLE_EMPTY
+        plan.empty_slots = None
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF, L.ptr(stream_offset),
-                                      {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order], L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
+                                      flags, L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
                                       L.stream_handle()))
+        plan.empty_slots = slots
     return uniq, block_ptr, src_local, src_global, counts
 
 

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 6
+#define FGL_ABI_VERSION 7
 
 enum fgl_error {
     FGL_OK = 0,
@@ -64,6 +64,7 @@ enum fgl_zero_policy {
 #define FGL_STATUS_UNIQ_OVERFLOW 2u /* more unique ids than uniq_capacity   */
 #define FGL_STATUS_MISSING_KEY 4u  /* a looked-up id is not in the table    */
 #define FGL_STATUS_BAD_SEED 8u     /* a seed id outside [0, n_nodes)        */
+#define FGL_STATUS_BAD_ID 16u      /* a negative id handed to the id-map    */
 
 #define FGL_IDMAP_ORDERED 0 /* new ids numbered by first occurrence (deterministic) */
 #define FGL_IDMAP_ARRIVAL 1 /* new ids numbered as their inserts land (the reference's rule,
@@ -71,6 +72,12 @@ enum fgl_zero_policy {
                                tenth faster; the order of the new ids depends on scheduling */
 #define FGL_IDMAP_FINAL 2   /* (or'ed in) the table is not consulted after this call: the local ids of the
                                new ids go to the edges and the unique list, not back into the table */
+/* fgl_sample_blocks only, or'ed into idmap_flags: */
+#define FGL_BLOCKS_TABLE_EMPTY 4       /* the caller vouches that every slot of the table is empty (as fgl_idmap_reset
+                                          leaves it, or an earlier fgl_sample_blocks call with FGL_BLOCKS_LEAVE_TABLE_EMPTY
+                                          on the same slots): the call's fill launch is skipped */
+#define FGL_BLOCKS_LEAVE_TABLE_EMPTY 8 /* the last pass of the call also empties the table again (it no longer reads
+                                          it), so that the next call may say FGL_BLOCKS_TABLE_EMPTY */
 #define FGL_MAX_FANOUT 192
 
 int fgl_abi_version(void);
@@ -171,7 +178,13 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * in one call with no host synchronisation: per hop sample_node -> id-map, the table and
  * the numbering persisting across hops (hop h's unique list is hop h+1's seed list).
  * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0];
- * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL (the last hop adds FGL_IDMAP_FINAL by itself).
+ * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL (the last hop adds FGL_IDMAP_FINAL by itself), optionally
+ * or'ed with FGL_BLOCKS_TABLE_EMPTY and / or FGL_BLOCKS_LEAVE_TABLE_EMPTY.
+ * Launches for H hops, first-occurrence numbering: one that starts the batch (counts, seeds into the table, the
+ * first hop's row offsets) and four per hop (sample, insert, mark, number) = 4H + 1, plus a table fill unless the
+ * caller vouches for an empty table, plus one scan per hop beyond a million seeds or four million edges.  Each
+ * hop's passes also prepare the next hop's sampling (row starts, degrees and per-tile edge counts of the nodes
+ * they touch), so no hop after the first reads the graph's offsets in a pass of its own.
  * (The reference lists fanouts the other way round and iterates reversed(); the caller
  * passes them already reversed.)
  *
@@ -200,7 +213,8 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * d_counts int32[2*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
  * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word.
  * The table is scratch: after the call it holds the local ids of the nodes of every hop but the
- * last (whose new nodes keep a transient value there); d_uniq is the complete map local -> global.
+ * last (whose new nodes keep a transient value there) -- or nothing, with FGL_BLOCKS_LEAVE_TABLE_EMPTY;
+ * d_uniq is the complete map local -> global.
  * ------------------------------------------------------------------------------- */
 int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
                            const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,

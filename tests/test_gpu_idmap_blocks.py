@@ -457,3 +457,53 @@ def test_arrival_order_through_the_c_abi(cuda, oracle, n_edges):
     probe = dev_i32(src, cuda)
     L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), n_edges, None, meta.data_ptr() + 4, st))
     assert np.array_equal(probe.cpu().numpy(), out)
+
+
+def test_negative_ids_are_reported_not_inserted(cuda):
+    """An id of -1 has the bit pattern of the table's empty marker, any negative id is no node id: the id-map
+    reports them (status bit, RuntimeError from the operator), gives their edges the local id -1 and leaves the
+    table intact -- lookups of the good ids still work."""
+    import fastgl
+    from fastgl import _lib as L
+    print("id-map: negative ids", flush=True)
+    lib = L.lib()
+    for flags in (L.IDMAP_ORDERED, L.IDMAP_ARRIVAL):
+        slots = lib.fgl_idmap_slots(64)
+        table = torch.empty(slots, dtype=torch.int64, device=cuda)
+        dst = torch.tensor([7, 3, 9], dtype=torch.int32, device=cuda)
+        src = torch.tensor([3, -1, 11, 7, -5, 11, 12], dtype=torch.int32, device=cuda)
+        uniq = torch.full((16,), -9, dtype=torch.int32, device=cuda)
+        meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+        ws = torch.empty(lib.fgl_idmap_map_src_workspace_bytes(src.numel()), dtype=torch.uint8, device=cuda)
+        st = L.stream_handle()
+        L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+        L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dst), 3, None, L.ptr(uniq), meta.data_ptr() + 4, st))
+        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(src), L.ptr(src), src.numel(), None, 3, None, meta.data_ptr(),
+                                      L.ptr(uniq), 16, flags, meta.data_ptr() + 4, L.ptr(ws), ws.numel(), st))
+        n_total, status = meta.tolist()
+        assert status == L.STATUS_BAD_ID and n_total == 5
+        got = src.tolist()
+        assert got[0] == 1 and got[3] == 0 and got[1] == -1 and got[4] == -1
+        assert got[2] == got[5] and sorted({got[2], got[6]}) == [3, 4]
+        assert sorted(uniq[3:5].tolist()) == [11, 12] and uniq[:3].tolist() == [7, 3, 9]
+        probe = torch.tensor([12, 9, 11, 3], dtype=torch.int32, device=cuda)
+        meta.zero_()
+        L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), 4, None, meta.data_ptr() + 4, st))
+        assert meta.tolist()[1] == 0 and probe.tolist() == [got[6], 2, got[2], 1]
+    # through the drop-in operator: a RuntimeError that names the cause
+    src = torch.tensor([3, -1, 11], dtype=torch.int32, device=cuda)
+    d = torch.tensor([7, 7, 3], dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError, match="negative id"):
+        fastgl.transfer_edge_id(src, d, torch.tensor([7, 3], dtype=torch.int32, device=cuda), 2, 5, 3, 3)
+    # a negative destination id
+    meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+    slots = lib.fgl_idmap_slots(8)
+    table = torch.empty(slots, dtype=torch.int64, device=cuda)
+    L.check(lib.fgl_idmap_reset(L.ptr(table), slots, L.stream_handle()))
+    bad = torch.tensor([4, -1, 6], dtype=torch.int32, device=cuda)
+    L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(bad), 3, None, None, meta.data_ptr() + 4, L.stream_handle()))
+    assert meta.tolist()[1] == L.STATUS_BAD_ID
+    probe = torch.tensor([6, 4], dtype=torch.int32, device=cuda)
+    meta.zero_()
+    L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), 2, None, meta.data_ptr() + 4, L.stream_handle()))
+    assert probe.tolist() == [2, 0] and meta.tolist()[1] == 0
