@@ -25,10 +25,49 @@ for _p in (ROOT, os.path.join(ROOT, "fastgl-ae_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM traffic per launch of the dominant kernel on workload c3, from two `rocprofv3 --pmc` runs
-# (FETCH_SIZE 370030 KiB x 1.898 + WRITE_SIZE 55671 KiB x 1.000, the factors being what the same
-# counters read for this kernel run as a plain copy of known size: 1064960 KiB read -> 561177)
-TRAFFIC_BYTES_C3 = 370030 * 1024 * 1.898 + 55671 * 1024 * 1.0
+# HBM traffic per launch of the dominant kernel comes from the tracked summary of two `rocprofv3 --pmc` runs
+# (FETCH_SIZE, WRITE_SIZE, each scaled by what the same counter reads for this kernel run as a plain copy of
+# known size).  The summary carries a record line with the kernel source's hash and the algorithmic bytes
+# per launch that it was taken at; `traffic` is reported only while both still match this run.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "aggregate_kernel_c3_pmc.md")
+AGGREGATE_SOURCE = os.path.join(ROOT, "fastgl-ae_amd", "csrc", "fgl_aggregate.hip")
+
+
+def source_hash(path=AGGREGATE_SOURCE):
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic_from_profile(workload, bytes_per_launch):
+    """HBM bytes per launch of the dominant kernel from the tracked counter summary, or None (with a note on
+    stderr) when the summary is missing, covers another workload, or was taken with another kernel source or
+    at another problem size."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        log("roofline.traffic: %s is missing -> null" % TRAFFIC_PROFILE)
+        return None
+    rec = None
+    for line in text.splitlines():
+        if line.startswith("traffic_record:"):
+            rec = json.loads(line[len("traffic_record:"):])
+    if rec is None:
+        log("roofline.traffic: no traffic_record line in %s -> null" % TRAFFIC_PROFILE)
+        return None
+    if rec.get("workload") != workload:
+        log("roofline.traffic: the counter summary covers workload %s, not %s -> null" % (rec.get("workload"), workload))
+        return None
+    if rec.get("source_sha16") != source_hash():
+        log("roofline.traffic: fgl_aggregate.hip has changed since the counter runs (%s -> %s): profile again -> null"
+            % (rec.get("source_sha16"), source_hash()))
+        return None
+    if abs(rec["algorithmic_bytes_per_launch"] - bytes_per_launch) > 0.03 * bytes_per_launch:
+        log("roofline.traffic: the counter runs moved %.1f MB per launch, this run %.1f MB -> null"
+            % (rec["algorithmic_bytes_per_launch"] / 1e6, bytes_per_launch / 1e6))
+        return None
+    return rec["traffic_bytes_per_launch"]
+
 
 WORKLOADS = {
     # name: nodes, R-MAT draws, feature dim, feature dtype, hidden, batch, training seeds, fanouts (reference order)
@@ -230,6 +269,20 @@ def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
 
+def load_compiled_module():
+    """The compiled torch extension module `fastgl` (fastgl-ae_amd/csrc/fastgl_module.cpp), loaded from its file
+    under a private name: in this process the name `fastgl` belongs to the Python package."""
+    import glob
+    import importlib.util
+    paths = glob.glob(os.path.join(ROOT, "fastgl-ae_amd", "fastgl_ext", "fastgl*.so"))
+    if not paths:
+        raise RuntimeError("not built: make -C fastgl-ae_amd/csrc module")
+    spec = importlib.util.spec_from_file_location("fastgl", paths[0])
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -247,6 +300,9 @@ def main():
                          "first: read the sizes back right after sampling, as sample_blocks() does")
     ap.add_argument("--other-order", choices=["on", "off"], default="on",
                     help="also time the steps with the other numbering rule of the id-map (value_other_id_order)")
+    ap.add_argument("--other-forms", choices=["on", "off"], default="on",
+                    help="also time sample_blocks() with its read-back (value_sample_blocks) and the reference's per-hop call "
+                         "pattern through the compiled extension module (value_drop_in_api)")
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
     ap.add_argument("--c4-eager", action="store_true",
@@ -410,6 +466,58 @@ def main():
         log("id order %s: %.3g sampled edges/s (sample+idmap %.3f ms)" % (other_order, value_other, alt_ms / args.steps))
         del alt, rec_alt
 
+    # ---- the same mini-batches through the two other forms of the sampler (context for `value`) -------------
+    # value_sample_blocks: FusedMapSampler.sample_blocks(), i.e. the fused call followed at once by the one
+    # read-back of the batch's sizes (the host's wait is inside the interval).
+    # value_drop_in_api: the reference's own call pattern -- sample_node + transfer_edge_id per hop, each returning
+    # exact-size tensors (FusedMapSampler.py:72-107) -- through the compiled extension module.
+    def time_sampler(fn):
+        for i in range(args.warmup):
+            fn(train[(i % n_batches) * B:(i % n_batches) * B + B])
+        torch.cuda.synchronize()
+        edges, ms = 0, 0.0
+        for i in range(args.steps):
+            seeds = train[((args.warmup + i) % n_batches) * B:((args.warmup + i) % n_batches) * B + B]
+            a, b = ev(), ev()
+            a.record()
+            n_e = fn(seeds)
+            b.record()
+            torch.cuda.synchronize()
+            edges += n_e
+            ms += a.elapsed_time(b)
+        return edges / (ms * 1e-3), ms / args.steps
+
+    value_sample_blocks = value_drop_in = None
+    if args.other_forms == "on":
+        plain = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
+        value_sample_blocks, ms_sb = time_sampler(lambda seeds: sum(b.num_edges() for b in plain.sample_blocks(None, seeds)[2]))
+        log("sample_blocks() with its read-back: %.3g sampled edges/s (%.3f ms per mini-batch)" % (value_sample_blocks, ms_sb))
+        del plain
+        try:
+            ext = load_compiled_module()
+        except Exception as exc:  # noqa: BLE001 -- reported, not fatal: the figure is context
+            log("compiled module unavailable (%s): value_drop_in_api -> null" % exc)
+            ext = None
+        if ext is not None:
+            nodes_num = int(edge_ptr.numel()) - 1
+
+            def reference_loop(seeds):  # FusedMapSampler.py:63-109 without the DGL block objects
+                seed_nodes_acc, dst_nodes, total = seeds, int(seeds.size(0)), 0
+                for block_index, fanout in enumerate(reversed(w["fanouts"])):
+                    src_out, dst_out, _ = ext.sample_node(edge_src, edge_src, edge_ptr, seed_nodes_acc.int(), dst_nodes, fanout)
+                    edge_nums = src_out.size(0)
+                    dst_unique = seeds if block_index == 0 else seed_nodes_acc
+                    max_src = nodes_num if fanout * dst_unique.size(0) > nodes_num else fanout * dst_unique.size(0)
+                    _, _, seed_nodes_acc = ext.transfer_edge_id(src_out, dst_out, dst_unique, dst_nodes, dst_nodes + edge_nums,
+                                                                max_src, edge_nums)
+                    dst_nodes = int(seed_nodes_acc.size(0))
+                    total += edge_nums
+                return total
+
+            value_drop_in, ms_di = time_sampler(reference_loop)
+            log("reference call pattern through the compiled module: %.3g sampled edges/s (%.3f ms per mini-batch)"
+                % (value_drop_in, ms_di))
+
     # ---- optional: the same steps with sampling of batch i+1 overlapped with aggregation of batch i ----
     ms_overlapped = None
     if args.overlap:
@@ -517,7 +625,7 @@ def main():
         x = a.view(torch.float32)[:rows * 128].view(rows, 128)
         ident_ptr = torch.arange(rows + 1, dtype=torch.int32, device=dev)
         ident_idx = torch.arange(rows, dtype=torch.int32, device=dev)
-        y = fastgl.aggregate(ident_ptr, ident_idx, x, mode="sum", zero_policy="zeros", longest_row=1)
+        y = fastgl.aggregate(ident_ptr, ident_idx, x, mode="sum", zero_policy="zeros", mapping="row")
         torch.cuda.synchronize()
         del a, b, c, x, y
 
@@ -600,11 +708,15 @@ def main():
                         "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
         "random_read_Gps": random_read_gps,
         "value_eager_launch": value_eager,
+        "value_sample_blocks": value_sample_blocks,
+        "value_drop_in_api": value_drop_in,
         "value_other_id_order": {"id_order": other_order, "value": value_other},
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
-                     "traffic": TRAFFIC_BYTES_C3 if args.workload == "c3" and args.id_order == "first" else None,
+                     "traffic": traffic_from_profile(args.workload, bytes_agg0 / K),
+                     "achieved_is": "algorithmic bytes (every sampled edge counted as one row fetch) / kernel time; "
+                                    "traffic = HBM bytes per launch from rocprofv3 counters (repeated rows that hit in cache are not in it)",
                      "kernel": "aggregate_kernel<float,4,32,MEAN> (outermost block, forward)",
                      "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_kernel0 / K * 1e3},
         "cpu_baseline": cpu,

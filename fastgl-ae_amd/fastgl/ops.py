@@ -286,7 +286,7 @@ _ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
 
 
 def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
-              out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None, n_rows_dev=None):
+              out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None, n_rows_dev=None, mapping="auto"):
     """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
     accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge;
     ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``.
@@ -297,7 +297,10 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     ``mode="edge"``: ``edge_weight`` float32 [n_entries, n_heads], weight of entry e for column f is
     ``edge_weight[edge_index[e] if edge_index is not None else e, f // (D // n_heads)]``.
     ``n_rows_dev``: one-element int32 device tensor with the actual row count when the host only knows the
-    bound ``n_rows`` (a block whose sizes have not been read back yet): rows past it are left unwritten."""
+    bound ``n_rows`` (a block whose sizes have not been read back yet): rows past it are left unwritten.
+    ``mapping``: ``"auto"`` lets the library pick how lanes are dealt to rows from the row count, the entry count
+    and ``longest_row`` (several lane groups per row for few long rows, several rows per group for many short
+    ones); ``"row"`` asks for one lane group per row whatever the shape (what measurements of that kernel use)."""
     _check_input(indptr, "indptr", _I32)
     _check_input(indices, "indices", _I32)
     if not isinstance(feat, torch.Tensor) or not feat.is_cuda:
@@ -338,6 +341,8 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     n = int(indptr.numel()) - 1 if n_rows is None else int(n_rows)
     if n < 0 or n > indptr.numel() - 1:
         raise RuntimeError("n_rows (%d) does not match indptr (%d entries)" % (n, indptr.numel()))
+    if mapping not in ("auto", "row"):
+        raise RuntimeError("mapping must be 'auto' or 'row'")
     m = _MODES[mode]
     z = _ZERO[zero_policy]
     if z == L.ZERO_COPY_SELF and n > feat.size(0):
@@ -354,7 +359,8 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
             L.check(L.lib().fgl_aggregate(L.ptr(indptr), idx_ptr, n, L.ptr(n_rows_dev), L.ptr(feat), int(feat.stride(0)), D,
                                           L.F32 if feat.dtype == torch.float32 else L.BF16, m, z, L.ptr(row_norm),
                                           L.ptr(col_norm), L.ptr(edge_weight), int(n_heads), L.ptr(edge_index),
-                                          longest_host, L.ptr(longest_dev), int(indices.numel()), L.ptr(out),
+                                          longest_host if mapping == "auto" else -1, L.ptr(longest_dev),
+                                          int(indices.numel()) if mapping == "auto" else -1, L.ptr(out),
                                           int(out.stride(0)), L.stream_handle()))
     return out
 

@@ -130,3 +130,48 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "--gpus 1" in (r.stdout + r.stderr)
+
+
+def test_compiled_module_loads_and_exports_the_reference_names():
+    """The torch extension module `fastgl` built from csrc/fastgl_module.cpp: loadable without a GPU, exports the ten
+    operator names the reference's Python code calls (aggregate_acc.cpp:601-621), raises RuntimeError on host tensors."""
+    import glob
+    import importlib.util
+    paths = glob.glob(os.path.join(ROOT, "fastgl-ae_amd", "fastgl_ext", "fastgl*.so"))
+    assert paths, "make -C fastgl-ae_amd/csrc module"
+    spec = importlib.util.spec_from_file_location("fastgl", paths[0])
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for name in ("sample_node", "transfer_edge_id", "cal_deg", "exclusive_sum", "forward_gcn", "backward_gcn", "forwaed_gin",
+                 "backward_gin", "forward_gat", "backward_gat"):
+        assert callable(getattr(mod, name)), name
+    assert mod.abi_version() == fastgl.lib().fgl_abi_version()
+    cpu = torch.zeros(4, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        mod.sample_node(cpu, cpu, cpu, cpu, 4, 2)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        mod.transfer_edge_id(cpu, cpu, cpu, 4, 8, 4, 4)
+    with pytest.raises(TypeError):
+        mod.cal_deg(cpu)  # positional signature as the reference's: (edges, nodes_num)
+
+
+def test_traffic_record_is_only_used_while_it_matches(tmp_path, monkeypatch, capsys):
+    """bench.py reports roofline.traffic from the tracked counter summary only while the kernel source's hash and the
+    bytes per launch match the run."""
+    import importlib.util
+    import json
+    spec = importlib.util.spec_from_file_location("bench_mod", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    rec = {"workload": "c3", "source_sha16": bench.source_hash(), "algorithmic_bytes_per_launch": 800e6, "traffic_bytes_per_launch": 700e6}
+    f = tmp_path / "p.md"
+    f.write_text("# x\n\ntraffic_record: " + json.dumps(rec) + "\n")
+    monkeypatch.setattr(bench, "TRAFFIC_PROFILE", str(f))
+    assert bench.traffic_from_profile("c3", 810e6) == 700e6
+    assert bench.traffic_from_profile("c3", 900e6) is None       # another problem size
+    assert bench.traffic_from_profile("c2", 800e6) is None       # another workload
+    rec["source_sha16"] = "0" * 16
+    f.write_text("traffic_record: " + json.dumps(rec) + "\n")
+    assert bench.traffic_from_profile("c3", 800e6) is None       # the kernel has changed since
+    monkeypatch.setattr(bench, "TRAFFIC_PROFILE", str(tmp_path / "missing.md"))
+    assert bench.traffic_from_profile("c3", 800e6) is None
