@@ -79,6 +79,8 @@ WORKLOADS = {
                    fanouts=[10, 10, 10, 10, 10]),
     "c4": None,  # aggregation-only microbench, see run_c4
     "ceiling": None,  # random row gathers from a 48 GB table, see run_ceiling
+    "reuse_ab": None,  # outermost block in one launch vs two passes by source id, see run_reuse_ab
+    "idmap_stats": None,  # intra-tile repeats and probes per lookup on real mini-batches, see run_idmap_stats
 }
 DESCRIPTIONS = {
     "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
@@ -91,6 +93,9 @@ DESCRIPTIONS = {
               "batch 8192, fanout [10,10,10,10,10]",
     "ceiling": "random row gathers from a 48 GB table: 2^20 output rows x 1 or 13 uniformly random source rows of 256 B - 2 KB, "
                "fp32 and bf16, through the aggregation kernel and through torch.index_select; streaming copy and add",
+    "reuse_ab": "outermost block of c3 mini-batches (1.5 M gathered rows of 512 B, 1.0 M distinct, 57 GB table): one launch vs "
+                "two launches cut by a source-id threshold",
+    "idmap_stats": "c3 mini-batches: ids repeated within a 2048-edge tile per hop; slots probed per lookup in the id-map's table",
     "c4": "aggregation microbench: 8192 dst x exactly 25 src out of 200K rows (int32 CSR), D in {64,128,256,602}, fp32 and bf16, "
           "sum and mean, forward and backward",
 }
@@ -179,6 +184,31 @@ def run_c4(args):
                     % (name, D, mode, uf, bf / uf / 1e3, bf / uf / 1e3 / HBM_PEAK_GBPS * 100, uc, bf / uc / 1e3,
                        bf / uc / 1e3 / HBM_PEAK_GBPS * 100, ub, bb / ub / 1e3, bb / ub / 1e3 / HBM_PEAK_GBPS * 100))
             del Xs
+    # attention-weighted aggregation (GAT): one float per (entry, head) on top of the row gather
+    gat_rows = []
+    n_heads = 4
+    alpha = torch.rand((E, n_heads), generator=g).to(dev)
+    t_ptr3, t_idx3, t_edge3 = fastgl.block_transpose(ptr, idx, n_dst, n_src, edge_ids=True)
+    for dt, name, esz in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
+        for D in (128, 256):
+            X = torch.randn(n_src, D, generator=g).to(dt).to(dev)
+            dO = torch.randn(n_dst, D, generator=g).to(dt).to(dev)
+            of = torch.empty((n_dst, D), dtype=dt, device=dev)
+            ob = torch.empty((n_src, D), dtype=dt, device=dev)
+            bf = E * D * esz + n_dst * D * esz + 4 * E + 4 * (n_dst + 1) + 4 * n_heads * E
+            bb = E * D * esz + n_src * D * esz + 4 * E + 4 * (n_src + 1) + 4 * n_heads * E + 4 * E  # + edge ids of the transposed entries
+            us = timed(lambda: fastgl.aggregate(ptr, idx, X, mode="sum", zero_policy="zeros", out=of, longest_row=k))
+            uf = timed(lambda: fastgl.aggregate(ptr, idx, X, mode="edge", zero_policy="zeros", out=of, longest_row=k,
+                                                edge_weight=alpha, n_heads=n_heads))
+            ub = timed(lambda: fastgl.aggregate(t_ptr3, t_idx3, dO, mode="edge", zero_policy="zeros", out=ob, edge_weight=alpha,
+                                                n_heads=n_heads, edge_index=t_edge3))
+            bs = bf - 4 * n_heads * E
+            gat_rows.append({"dtype": name, "D": D, "heads": n_heads, "fwd_us": uf, "fwd_GBps": bf / uf / 1e3,
+                             "fwd_frac_peak": bf / uf / 1e3 / HBM_PEAK_GBPS, "sum_fwd_us": us, "sum_fwd_GBps": bs / us / 1e3,
+                             "bwd_us": ub, "bwd_GBps": bb / ub / 1e3, "bwd_frac_peak": bb / ub / 1e3 / HBM_PEAK_GBPS})
+            log("%-4s D=%-3d edge weights x%d: fwd %6.1f us %5.0f GB/s (%4.1f%%; plain sum %6.1f us %5.0f GB/s) | bwd %6.1f us %5.0f GB/s (%4.1f%%)"
+                % (name, D, n_heads, uf, bf / uf / 1e3, bf / uf / 1e3 / HBM_PEAK_GBPS * 100, us, bs / us / 1e3, ub, bb / ub / 1e3,
+                   bb / ub / 1e3 / HBM_PEAK_GBPS * 100))
     head = [r for r in rows if r["dtype"] == "f32" and r["D"] == 128 and r["mode"] == "mean"][0]
     print(json.dumps({
         "metric": "aggregation HBM GB/s (% peak), 1 MI355X", "value": head["fwd_GBps"], "unit": "GB/s", "n_gpus": 1,
@@ -186,7 +216,7 @@ def run_c4(args):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": DESCRIPTIONS["c4"]},
         "roofline": {"bound": "hbm", "achieved": head["fwd_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": head["fwd_frac_peak"], "traffic": None, "kernel": "aggregate_kernel (D=128 fp32 mean forward)"},
-        "cpu_baseline": None, "cases": rows}), flush=True)
+        "cpu_baseline": None, "cases": rows, "edge_weighted_cases": gat_rows}), flush=True)
 
 
 
@@ -265,6 +295,150 @@ def run_ceiling(args):
         "cpu_baseline": None, "stream_copy_GBps": copy_gbps, "stream_add_GBps": add_gbps, "cases": rows_out}), flush=True)
 
 
+def _c3_inputs(torch, fastgl, dev, need_features=True):
+    w = WORKLOADS["c3"]
+    edge_ptr, edge_src = fastgl.graph.rmat_csr(w["nodes"], w["draws"], seed=0, device=dev)
+    torch.cuda.empty_cache()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    feat = None
+    if need_features:
+        feat = torch.empty((w["nodes"], w["dim"]), dtype=torch.float32, device=dev)
+        for lo in range(0, w["nodes"], 1 << 22):
+            hi = min(w["nodes"], lo + (1 << 22))
+            feat[lo:hi] = torch.randn((hi - lo, w["dim"]), generator=gen, device=dev, dtype=torch.float32)
+    train = torch.randperm(w["nodes"], generator=gen, device=dev)[:w["train"]].to(torch.int32)
+    return w, edge_ptr, edge_src, feat, train
+
+
+def run_reuse_ab(args):
+    """Does it pay to gather the outermost block in two passes by source id, so that each pass's distinct rows fit the
+    256 MB Infinity Cache?  (A mini-batch's outermost block gathers 1.5 M rows of which 1.0 M are distinct.)  Times
+    the whole block in one launch against the same block cut in two by a source-id threshold -- the launches of the
+    two halves only; the pass that would add the two partial outputs is not even counted -- for the threshold that
+    halves the ids and the one that halves the gathered rows."""
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    w, edge_ptr, edge_src, feat, train = _c3_inputs(torch, fastgl, dev)
+    B, D = w["batch"], w["dim"]
+    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0).set_graph(edge_ptr, edge_src)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def timed(fn, reps=10):
+        for _ in range(3):
+            fn()
+        a, b = ev(), ev()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3
+
+    cases = []
+    for batch in range(3):
+        _, _, blocks = sampler.sample_blocks(None, train[batch * B:(batch + 1) * B])
+        b0 = blocks[0]
+        n_dst, E = b0.num_dst_nodes(), b0.num_edges()
+        src = b0.src_global.long()
+        rows = torch.repeat_interleave(torch.arange(n_dst, device=dev), b0.in_degrees().long())
+        distinct = int(torch.unique(src).numel())
+        out = torch.empty((n_dst, D), device=dev)
+        t_full = timed(lambda: fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="sum", zero_policy="zeros", out=out,
+                                                longest_row=w["fanouts"][0]))
+        case = {"edges": E, "distinct_rows": distinct, "rows": n_dst, "one_launch_us": t_full,
+                "one_launch_GBps": (E * D * 4 + n_dst * D * 4 + 4 * E + 4 * n_dst) / t_full / 1e3}
+        for name, thr in (("half_of_the_ids", w["nodes"] // 2), ("half_of_the_gathered_rows", int(torch.median(src)))):
+            halves = []
+            for keep in (src < thr, src >= thr):
+                sub_src = b0.src_global[keep].contiguous()
+                counts = torch.bincount(rows[keep], minlength=n_dst)
+                sub_ptr = torch.zeros(n_dst + 1, dtype=torch.int32, device=dev)
+                sub_ptr[1:] = torch.cumsum(counts, 0).int()
+                halves.append((sub_ptr, sub_src, int(torch.unique(sub_src).numel())))
+            outs = [torch.empty((n_dst, D), device=dev) for _ in halves]
+
+            def two():
+                for (p_, s_, _), o_ in zip(halves, outs):
+                    fastgl.aggregate(p_, s_, feat, mode="sum", zero_policy="zeros", out=o_, longest_row=w["fanouts"][0])
+
+            t_two = timed(two)
+            case[name] = {"threshold": thr, "edges": [int(h[1].numel()) for h in halves], "distinct_rows": [h[2] for h in halves],
+                          "two_launches_us": t_two}
+            log("batch %d: %d edges, %d distinct rows: one launch %.1f us | cut at %s (%d): halves of %s edges / %s distinct rows, "
+                "two launches %.1f us" % (batch, E, distinct, t_full, name, thr, case[name]["edges"], case[name]["distinct_rows"], t_two))
+        cases.append(case)
+    print(json.dumps({"metric": "outermost-block gather in one launch vs two passes by source id (us), 1 MI355X",
+                      "value": cases[-1]["one_launch_us"], "unit": "us", "n_gpus": 1, "steps": 10, "warmup": 3, "ms_per_step": None,
+                      "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": DESCRIPTIONS["reuse_ab"]}, "roofline": None, "cpu_baseline": None, "cases": cases}), flush=True)
+
+
+def run_idmap_stats(args):
+    """The numbers behind two design decisions of the id-map, on real mini-batches of workload c3: how many edges of a
+    2048-edge tile repeat an id already seen in the same tile (what a per-tile LDS dedup before the global table could
+    save), and how many slots a lookup probes in the table at the load factor the sampler runs it at (what probing with
+    several lanes per key could save)."""
+    import numpy as np
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    w, edge_ptr, edge_src, _, train = _c3_inputs(torch, fastgl, dev, need_features=False)
+    B = w["batch"]
+    sampler = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0).set_graph(edge_ptr, edge_src)
+    hops = []
+    for batch in range(3):
+        input_nodes, _, blocks = sampler.sample_blocks(None, train[batch * B:(batch + 1) * B])
+        uniq = input_nodes.long()
+        for h, block in enumerate(reversed(blocks)):
+            src_l = block.src_local.long()
+            src_g = uniq[src_l]
+            E = int(src_g.numel())
+            tile = torch.arange(E, device=dev) // 2048
+            pair = tile * (1 << 32) + src_g
+            repeats_in_tile = E - int(torch.unique(pair).numel())
+            new_edges = int((src_l >= block.num_dst_nodes()).sum())
+            new_ids = block.num_src_nodes() - block.num_dst_nodes()
+            hops.append({"batch": batch, "hop": h, "edges": E, "repeat_an_id_of_the_same_tile": repeats_in_tile,
+                         "frac": repeats_in_tile / max(E, 1), "edges_of_new_ids": new_edges, "new_ids": new_ids})
+            log("batch %d hop %d: %d edges, %d (%.2f %%) repeat an id of their own 2048-edge tile; %d edges mention %d new ids"
+                % (batch, h, E, repeats_in_tile, 100 * repeats_in_tile / max(E, 1), new_edges, new_ids))
+    # probes per lookup: the table as the sampler sizes it (a power of two of at least 4 x the ids), filled with the
+    # last batch's ids by the library's hash and linear probing, replayed on the host
+    ids = input_nodes.cpu().numpy().astype(np.uint64)
+    slots = 64
+    while slots < 4 * ids.size:
+        slots *= 2
+    shift = 32 - int(np.log2(slots))
+    home = ((ids * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)) >> np.uint64(shift)
+    occupied = bytearray(slots)
+    lookups = np.empty(ids.size, dtype=np.int64)  # slots a lookup of the id reads = 1 + its distance from its home slot
+    mask = slots - 1
+    for i, h in enumerate(home.tolist()):
+        p, c = h, 1
+        while occupied[p]:
+            p = (p + 1) & mask
+            c += 1
+        occupied[p] = 1
+        lookups[i] = c
+    stats = {"ids": int(ids.size), "slots": int(slots), "load": ids.size / slots, "mean_probes": float(lookups.mean()),
+             "p99_probes": int(np.percentile(lookups, 99)), "max_probes": int(lookups.max()),
+             "within_first_64B_line": float(np.mean((home.astype(np.int64) % 8) + lookups <= 8))}
+    log("table of %d slots for %d ids (load %.2f): %.2f slots probed per lookup on average, 99 %% within %d, max %d; %.1f %% of the "
+        "lookups end in the 64-byte line of their first slot" % (slots, ids.size, stats["load"], stats["mean_probes"], stats["p99_probes"],
+                                                               stats["max_probes"], 100 * stats["within_first_64B_line"]))
+    print(json.dumps({"metric": "id-map design statistics (intra-tile repeats, probes per lookup), workload c3", "value": stats["mean_probes"],
+                      "unit": "slots probed per lookup", "n_gpus": 1, "steps": 3, "warmup": 0, "ms_per_step": None, "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+                      "config": {"workload": DESCRIPTIONS["idmap_stats"]}, "roofline": None, "cpu_baseline": None,
+                      "hops": hops, "probing": stats}), flush=True)
+
+
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
@@ -332,6 +506,10 @@ def main():
         return run_c4(args)
     if args.workload == "ceiling":
         return run_ceiling(args)
+    if args.workload == "reuse_ab":
+        return run_reuse_ab(args)
+    if args.workload == "idmap_stats":
+        return run_idmap_stats(args)
     w = WORKLOADS[args.workload]
     N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
     fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16

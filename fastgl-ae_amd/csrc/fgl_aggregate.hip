@@ -286,6 +286,84 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
     }
 }
 
+// acc += sum over the entries [a, b) of one row (a < b) with per-entry, per-head weights (FGL_AGG_EDGE).
+template <typename T, int VEC, int LPR>
+__device__ __forceinline__ void gather_row_edge(const AggArgs& g, const LaneSlice<T, VEC>& ls, int gl, int a, int b,
+                                                float (&acc)[VEC])
+{
+    using IO = RowIO<T, VEC>;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    const int64_t ldx = g.ldx;
+    const int D = g.D;
+    const int col0 = ls.col0;
+    const bool live = ls.live;
+    // attention-style weights: one float per (entry, head); a lane's VEC columns lie in one
+    // head when unit_dim is a multiple of VEC, else each column looks its head up
+    const float* __restrict__ ew = g.edge_w;
+    const int H = g.n_heads, unit = g.unit_dim;
+    const bool one_head = (unit % VEC) == 0;
+    int head[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        const int c = col0 + i < D ? col0 + i : D - 1;
+        head[i] = c / unit;
+    }
+    for (int base = a; base < b; base += LPR) {
+        const int cnt = (b - base) < LPR ? (b - base) : LPR;
+        int my_col = 0, my_eid = 0;
+        if (gl < cnt) {
+            my_col = indices[base + gl];
+            my_eid = g.edge_index ? g.edge_index[base + gl] : base + gl;
+        }
+        float part[VEC];  // this chunk's sum (see the note on two-level summation in gather_row)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
+        int t = 0;
+        if (one_head) {
+            // as in gather_row: four row loads -- and the four weights that go with them -- are issued
+            // before the first FMA
+            for (; t + 4 <= cnt; t += 4) {
+                const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
+                const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
+                const int64_t e0 = __shfl(my_eid, t, LPR), e1 = __shfl(my_eid, t + 1, LPR);
+                const int64_t e2 = __shfl(my_eid, t + 2, LPR), e3 = __shfl(my_eid, t + 3, LPR);
+                if (live) {
+                    const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                    const typename IO::Raw r1 = ls.load(X + (int64_t)c1 * ldx + col0);
+                    const typename IO::Raw r2 = ls.load(X + (int64_t)c2 * ldx + col0);
+                    const typename IO::Raw r3 = ls.load(X + (int64_t)c3 * ldx + col0);
+                    const float w0 = ew[e0 * H + head[0]], w1 = ew[e1 * H + head[0]];
+                    const float w2 = ew[e2 * H + head[0]], w3 = ew[e3 * H + head[0]];
+                    IO::fma(part, w0, r0);
+                    IO::fma(part, w1, r1);
+                    IO::fma(part, w2, r2);
+                    IO::fma(part, w3, r3);
+                }
+            }
+        }
+        for (; t < cnt; ++t) {
+            const int c0 = __shfl(my_col, t, LPR);
+            const int64_t e0 = __shfl(my_eid, t, LPR);
+            if (live) {
+                const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
+                if (one_head) {
+                    IO::fma(part, ew[e0 * H + head[0]], r0);
+                } else {
+                    float x[VEC];
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) x[i] = 0.0f;
+                    IO::fma(x, 1.0f, r0);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) part[i] += ew[e0 * H + head[i]] * x[i];
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += part[i];
+    }
+}
+
 // A list with more entries than this is left to aggregate_long_rows_kernel when the caller cannot rule
 // such lists out: a hub of a transposed block can hold thousands of entries, the one lane group that
 // walks a list here would outlast the rest of the launch, and hubs sit next to each other.  (Measured on
@@ -329,70 +407,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
     if (a == b) {
         if (live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + col0));
     } else if constexpr (MODE == FGL_AGG_EDGE) {
-        // attention-style weights: one float per (entry, head); a lane's VEC columns lie in one
-        // head when unit_dim is a multiple of VEC, else each column looks its head up
-        const float* __restrict__ ew = g.edge_w;
-        const int H = g.n_heads, unit = g.unit_dim;
-        const bool one_head = (unit % VEC) == 0;
-        int head[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const int c = col0 + i < D ? col0 + i : D - 1;
-            head[i] = c / unit;
-        }
-        for (int base = a; base < b; base += LPR) {
-            const int cnt = (b - base) < LPR ? (b - base) : LPR;
-            int my_col = 0, my_eid = 0;
-            if (gl < cnt) {
-                my_col = indices[base + gl];
-                my_eid = g.edge_index ? g.edge_index[base + gl] : base + gl;
-            }
-            float part[VEC];  // this chunk's sum (see the note on two-level summation in gather_row)
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
-            int t = 0;
-            if (one_head) {
-                // as in gather_row: four row loads -- and the four weights that go with them -- are issued
-                // before the first FMA
-                for (; t + 4 <= cnt; t += 4) {
-                    const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
-                    const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
-                    const int64_t e0 = __shfl(my_eid, t, LPR), e1 = __shfl(my_eid, t + 1, LPR);
-                    const int64_t e2 = __shfl(my_eid, t + 2, LPR), e3 = __shfl(my_eid, t + 3, LPR);
-                    if (live) {
-                        const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
-                        const typename IO::Raw r1 = ls.load(X + (int64_t)c1 * ldx + col0);
-                        const typename IO::Raw r2 = ls.load(X + (int64_t)c2 * ldx + col0);
-                        const typename IO::Raw r3 = ls.load(X + (int64_t)c3 * ldx + col0);
-                        const float w0 = ew[e0 * H + head[0]], w1 = ew[e1 * H + head[0]];
-                        const float w2 = ew[e2 * H + head[0]], w3 = ew[e3 * H + head[0]];
-                        IO::fma(part, w0, r0);
-                        IO::fma(part, w1, r1);
-                        IO::fma(part, w2, r2);
-                        IO::fma(part, w3, r3);
-                    }
-                }
-            }
-            for (; t < cnt; ++t) {
-                const int c0 = __shfl(my_col, t, LPR);
-                const int64_t e0 = __shfl(my_eid, t, LPR);
-                if (live) {
-                    const typename IO::Raw r0 = ls.load(X + (int64_t)c0 * ldx + col0);
-                    if (one_head) {
-                        IO::fma(part, ew[e0 * H + head[0]], r0);
-                    } else {
-                        float x[VEC];
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i) x[i] = 0.0f;
-                        IO::fma(x, 1.0f, r0);
-#pragma unroll
-                        for (int i = 0; i < VEC; ++i) part[i] += ew[e0 * H + head[i]] * x[i];
-                    }
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] += part[i];
-        }
+        gather_row_edge<T, VEC, LPR>(g, ls, gl, a, b, acc);
     } else {
         // one test per launch instead of one per load: is every live lane's vector whole?
         if (all_lanes_full<T, VEC>(D)) gather_row<T, VEC, LPR, MODE, true>(g, ls, gl, row, a, b, acc);
@@ -497,7 +512,6 @@ __global__ __launch_bounds__(kBlock) void aggregate_split_kernel(const AggArgs g
 // them are in flight together, four at a time; the running sum is stored and cleared whenever an entry is
 // the last of its row.  A bundle that holds a hub (more than 128 entries in all) falls back to one row
 // after the other.  Sums are in CSR order, as in aggregate_kernel.
-// Not for FGL_AGG_EDGE.
 #ifndef FGL_BUNDLE_ROWS
 #define FGL_BUNDLE_ROWS 4
 #endif
@@ -539,12 +553,17 @@ __global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs 
         for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
         // cnt entries from the bundle's entry number cb on: ids, weights and row ends in one coalesced read,
         // then the data rows four at a time
+        // FGL_AGG_EDGE (only where a lane's columns lie in one head, which the launcher checks): a lane looks up the
+        // weight of (entry, its head) itself, next to the row load
+        const int head = MODE == FGL_AGG_EDGE ? col0 / g.unit_dim : 0;
         auto chunk = [&](int cb, int cnt) {
             int my_col = 0, my_tag = 0;  // tag: row within the bundle, + 256 if the entry is the last of its row
+            int my_eid = 0;
             float my_w = 0.0f;
             if (gl < cnt) {
                 const int e = off[0] + cb + gl;
                 my_col = indices[e];
+                if (MODE == FGL_AGG_EDGE) my_eid = g.edge_index ? g.edge_index[e] : e;
                 int j = 0;  // the rows that start at or before e: the last of them, row j, holds e
                 int begin_j = off[0], end_j = off[1];
 #pragma unroll
@@ -558,7 +577,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs 
                 float row_factor = 1.0f;
                 if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(end_j - begin_j);
                 if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[r0 + j]);
-                my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                if (MODE != FGL_AGG_EDGE) my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
                 my_tag = j | (e + 1 == end_j ? 256 : 0);
             }
             for (int t = 0; t < cnt; t += 4) {
@@ -569,13 +588,17 @@ __global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs 
                 for (int j = 0; j < 4; ++j) {
                     const int src = t + j < cnt ? t + j : t;
                     c[j] = __shfl(my_col, src, LPR);
-                    w[j] = __shfl(my_w, src, LPR);
+                    if (MODE == FGL_AGG_EDGE) w[j] = __int_as_float(__shfl(my_eid, src, LPR));  // (the entry's id, for now)
+                    else w[j] = __shfl(my_w, src, LPR);
                     tag[j] = __shfl(my_tag, src, LPR);
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     x[j] = typename IO::Raw{};
-                    if (live && t + j < cnt) x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                    if (live && t + j < cnt) {
+                        x[j] = ls.load(X + (int64_t)c[j] * ldx + col0);
+                        if (MODE == FGL_AGG_EDGE) w[j] = g.edge_w[(int64_t)__float_as_int(w[j]) * g.n_heads + head];
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -618,6 +641,8 @@ __global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs 
         for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
         if (a == b) {
             if (live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + col0));
+        } else if constexpr (MODE == FGL_AGG_EDGE) {
+            gather_row_edge<T, VEC, LPR>(g, ls, gl, a, b, acc);
         } else {
             gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc);
         }
@@ -1140,6 +1165,14 @@ static int launch_agg_flat(int mode, bool long_rows_possible, int lanes, bool bu
 }
 
 // Launches of the two special mappings.  (Only for rows that fit one lane group; never for FGL_AGG_EDGE.)
+#define FGL_FOR_ANY_MODE(mode, LAUNCH)                    \
+    switch (mode) {                                       \
+        case FGL_AGG_SUM: LAUNCH(FGL_AGG_SUM); break;     \
+        case FGL_AGG_MEAN: LAUNCH(FGL_AGG_MEAN); break;   \
+        case FGL_AGG_GCN: LAUNCH(FGL_AGG_GCN); break;     \
+        case FGL_AGG_COLMEAN: LAUNCH(FGL_AGG_COLMEAN); break; \
+        default: LAUNCH(FGL_AGG_EDGE); break;             \
+    }
 #define FGL_FOR_PLAIN_MODE(mode, LAUNCH)                  \
     switch (mode) {                                       \
         case FGL_AGG_SUM: LAUNCH(FGL_AGG_SUM); break;     \
@@ -1176,7 +1209,7 @@ static int launch_agg_bundle(int mode, bool long_rows_possible, unsigned gy, hip
                                0, stream, g);                                                                         \
         }                                                                                                             \
     } while (0)
-    FGL_FOR_PLAIN_MODE(mode, FGL_LAUNCH_BUNDLE)
+    FGL_FOR_ANY_MODE(mode, FGL_LAUNCH_BUNDLE)
 #undef FGL_LAUNCH_BUNDLE
     FGL_CHECK_LAUNCH("aggregate_bundle_kernel");
     return FGL_OK;
@@ -1203,8 +1236,9 @@ static int launch_agg_vec(int mode, int64_t longest_row_max, int64_t n_entries_m
     int lpr = 8;
     while (lpr < 64 && lpr < lanes_needed) lpr <<= 1;
     // many rows of short lists (a transposed block): several rows per lane group
-    const bool short_lists = mode != FGL_AGG_EDGE && n_entries_max >= 0 && g.n_rows_max >= 1024 &&
-                             n_entries_max <= (int64_t)FGL_BUNDLE_MAX_AVG_ENTRIES * g.n_rows_max;
+    const bool short_lists = n_entries_max >= 0 && g.n_rows_max >= 1024 &&
+                             n_entries_max <= (int64_t)FGL_BUNDLE_MAX_AVG_ENTRIES * g.n_rows_max &&
+                             (mode != FGL_AGG_EDGE || (g.unit_dim % VEC == 0 && lanes_needed <= 64));
     // rows wider than one 64-lane group that fill their groups to less than 90 %: flat mapping
     // (602 fp32 columns: 100 -> 80 us; 602 bf16: 59 -> 44 us forward, 135 -> 84 us on the transposed block)
     if (lanes_needed > 64 && mode != FGL_AGG_EDGE && lanes_needed * 10 < ceil_div(lanes_needed, 64) * 64 * 9)
