@@ -99,6 +99,15 @@ class Block:
         return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())
 
 
+class _ShapeState:
+    """What the sampler has learned about mini-batches of one shape (seed count, fanouts, graph size, device)."""
+
+    def __init__(self):
+        self.plans = {}         # node-capacity tuple (None = worst case) -> BlocksPlan
+        self.nodes_seen = None  # per hop: the node counts that the buffer sizes are derived from
+        self.graphs = None      # (plan, table slots) -> captured launch sequences, see FusedMapSampler._replay
+
+
 class PendingBatch:
     """A mini-batch whose kernels are enqueued and whose sizes are still on the device
     (``FusedMapSampler.begin_sample``).  The sizes travel to a pinned host buffer on a second stream as soon as
@@ -174,7 +183,6 @@ class FusedMapSampler:
         self.graph_slots = int(graph_slots)
         if self.graph_slots < 0 or self.graph_slots == 1:
             raise ValueError("graph_slots must be 0 (off) or at least 2")
-        self._graphs = None      # (plan, table slots) -> list of captured slots
         self._graph_turn = 0
         self.rng_seed = int(rng_seed)
         self.batches = 0
@@ -183,9 +191,7 @@ class FusedMapSampler:
         self.edge_dst = None  # unused by the kernels; kept because the reference's trainer sets it
         self.edge_ptr = None  # CSR indptr (int32 or int64)
         self.output_nodes = None
-        self._shape = None
-        self._plans = {}        # node-capacity tuple (None = worst case) -> BlocksPlan
-        self._nodes_seen = None  # per hop: the node counts that the buffer sizes are derived from
+        self._states = {}       # shape of a mini-batch -> _ShapeState
         self._side = None        # second stream of iter_batches
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
@@ -209,45 +215,57 @@ class FusedMapSampler:
         return self._sample_layerwise(seeds, stream_base)
 
     # -- fused path: enqueue (no host synchronisation) / finish (one read-back) -----------------
-    def _caps(self, n_seeds):
+    @staticmethod
+    def _caps(state, n_seeds):
         # Worst-case bounds assume that no neighbour ever repeats: 8.6 M nodes for 8192 seeds and
         # fanouts 5/10/15 where real batches hold ~1 M, and the whole graph for deep fanouts.  A hash
         # table that fits the caches is much faster and output buffers sized by the bound cost GBs,
         # so after the first batch both are sized from the largest batch seen (x1.5, table load <=
         # 1/4).  A batch that outgrows them is detected by the kernels (status word) and simply
         # redone with the worst-case plan; results do not depend on the sizes.
-        if self._nodes_seen is None:
+        if state.nodes_seen is None:
             return None
-        return tuple(max(n_seeds, -(-int(1.5 * n) // 4096) * 4096) for n in self._nodes_seen)
+        return tuple(max(n_seeds, -(-int(1.5 * n) // 4096) * 4096) for n in state.nodes_seen)
 
-    def _launch_fused(self, seeds, stream_base, caps):
+    def _state_for(self, seeds):
+        # Plans, learned buffer sizes and captured graphs are kept per shape: the short last batch of an epoch gets
+        # an entry of its own and does not throw away what the full-size batches have learned.
+        shape = (int(seeds.numel()), tuple(reversed(self.fanouts)), self.nodes_num, seeds.device)
+        state = self._states.get(shape)
+        if state is None:
+            if len(self._states) >= 4:  # (a sampler fed ever-changing batch sizes: forget the oldest shape)
+                self._states.pop(next(iter(self._states)))
+            state = self._states[shape] = _ShapeState()
+        return state
+
+    def _launch_fused(self, seeds, stream_base, worst_case=False, state=None):
         hop_fanouts = list(reversed(self.fanouts))
         lib = ops.L.lib()
         n_seeds = int(seeds.numel())
-        shape = (n_seeds, tuple(hop_fanouts), self.nodes_num, seeds.device)
-        if self._shape != shape:
-            self._shape, self._plans, self._nodes_seen, caps, self._graphs = shape, {}, None, None, None
-        plan = self._plans.get(caps)
+        if state is None:
+            state = self._state_for(seeds)
+        caps = None if worst_case else self._caps(state, n_seeds)
+        plan = state.plans.get(caps)
         if plan is None:
             plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
-            self._plans = {k: v for k, v in self._plans.items() if k is None}  # keep the worst-case plan only
-            self._plans[caps] = plan
+            state.plans = {k: v for k, v in state.plans.items() if k is None}  # keep the worst-case plan only
+            state.plans[caps] = plan
         slots = plan.slots
         if caps is not None:
-            slots = min(slots, max(lib.fgl_idmap_slots(2 * self._nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
+            slots = min(slots, max(lib.fgl_idmap_slots(2 * state.nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
         if self.graph_slots and caps is not None:  # steady state only: the worst-case plan (first batch, redo) runs eagerly
-            out = self._replay(plan, slots, seeds, stream_base)
+            out = self._replay(state, plan, slots, seeds, stream_base)
         else:
             out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
                                           keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order)
-        return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out)
+        return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state)
 
-    def _replay(self, plan, slots, seeds, stream_base):
+    def _replay(self, state, plan, slots, seeds, stream_base):
         """Graph mode: copy the seeds and the random-stream offset into the turn's slot, replay its graph."""
         key = (id(plan), slots)
-        if self._graphs is None or self._graphs[0] != key:
-            self._graphs = (key, plan, [None] * self.graph_slots)  # graphs of an outgrown plan are dropped
-        ring = self._graphs[2]
+        if state.graphs is None or state.graphs[0] != key:
+            state.graphs = (key, plan, [None] * self.graph_slots)  # graphs of an outgrown plan are dropped
+        ring = state.graphs[2]
         turn = self._graph_turn % self.graph_slots
         self._graph_turn += 1
         if ring[turn] is None:
@@ -286,9 +304,10 @@ class FusedMapSampler:
         H = len(self.fanouts)
         c = counts_host
         status = c[2 * H + 1]
+        state = pending["state"]
         if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and pending["caps"] is not None:
-            self._nodes_seen = None
-            pending = self._launch_fused(pending["seeds"], pending["stream_base"], None)
+            state.nodes_seen = None
+            pending = self._launch_fused(pending["seeds"], pending["stream_base"], worst_case=True, state=state)
             c = pending["out"][4].tolist()
             status = c[2 * H + 1]
         if status:
@@ -296,10 +315,10 @@ class FusedMapSampler:
         seen = c[:H + 1]
         # the sizes are kept while batches stay within 1.25 x what they were derived from (the buffers hold 1.5 x):
         # every change means a new plan, new buffers and, in graph mode, new captures
-        if self._nodes_seen is None:
-            self._nodes_seen = seen
-        elif any(a > 1.25 * b for a, b in zip(seen, self._nodes_seen)):
-            self._nodes_seen = [max(a, b) for a, b in zip(seen, self._nodes_seen)]
+        if state.nodes_seen is None:
+            state.nodes_seen = seen
+        elif any(a > 1.25 * b for a, b in zip(seen, state.nodes_seen)):
+            state.nodes_seen = [max(a, b) for a, b in zip(seen, state.nodes_seen)]
         uniq, bptr, src_l, src_g, _ = pending["out"]
         blocks = []
         for h in range(H):
@@ -323,10 +342,10 @@ class FusedMapSampler:
         seeds = seed_nodes.to(device=self.edge_src.device, dtype=torch.int32).contiguous()
         stream_base = (self.batches * 64) & 0xFFFFFFFF
         self.batches += 1
-        return PendingBatch(self, self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel()))))
+        return PendingBatch(self, self._launch_fused(seeds, stream_base))
 
     def _sample_fused(self, seeds, stream_base):
-        pending = self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel())))
+        pending = self._launch_fused(seeds, stream_base)
         return self._finish_fused(pending, pending["out"][4].tolist())  # the one host synchronisation of the mini-batch
 
     def _side_stream(self, dev):
@@ -354,7 +373,7 @@ class FusedMapSampler:
             self.batches += 1
             side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
             with torch.cuda.stream(side):
-                pending = self._launch_fused(seeds, stream_base, self._caps(int(seeds.numel())))
+                pending = self._launch_fused(seeds, stream_base)
                 host = torch.empty(2 * H + 2, dtype=torch.int32, pin_memory=True)
                 host.copy_(pending["out"][4], non_blocking=True)
                 done = torch.cuda.Event()

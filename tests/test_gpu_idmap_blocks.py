@@ -162,8 +162,8 @@ def test_begin_sample_then_finish(cuda, oracle, small_graph):
         # (the two launches may map lanes to rows differently -- the bound-sized one has many more rows -- and the
         # order of the fp32 additions within a row follows the mapping: equal up to rounding, not bit for bit)
         assert torch.allclose(early[:b0.num_dst_nodes()], late, rtol=1e-5, atol=1e-6)
-    sampler._nodes_seen = [700, 800, 900, 1000]                             # (pretend the batches stayed tiny)
     hubs = np.argsort(-np.diff(indptr))[:700].astype(np.int32)
+    sampler._state_for(dev_i32(hubs, cuda)).nodes_seen = [700, 800, 900, 1000]  # (pretend the batches stayed tiny)
     pend = sampler.begin_sample(dev_i32(hubs, cuda))
     fastgl.aggregate(pend.outer_edge_ptr, pend.outer_src_global, feat, mode="mean", zero_policy="zeros",
                      n_rows=pend.outer_n_dst_bound, n_rows_dev=pend.outer_n_dst)  # on an overflowed batch: stays in bounds
@@ -183,11 +183,12 @@ def test_undersized_buffers_are_detected_and_redone(cuda, oracle, small_graph):
     low = np.flatnonzero(np.diff(indptr) <= 1)[:512].astype(np.int32)       # a batch that hardly grows ...
     got = sampler.sample_blocks(None, dev_i32(low, cuda))
     check_blocks(oracle, indptr, indices, low, [15, 10, 5], got, 9, 0)
-    sampler._nodes_seen = [512, 600, 700, 800]                              # (pretend it stayed tiny)
+    state = sampler._state_for(dev_i32(low, cuda))
+    state.nodes_seen = [512, 600, 700, 800]                                 # (pretend it stayed tiny)
     hubs = np.argsort(-np.diff(indptr))[:512].astype(np.int32)              # ... followed by one that explodes
     got = sampler.sample_blocks(None, dev_i32(hubs, cuda))
     check_blocks(oracle, indptr, indices, hubs, [15, 10, 5], got, 9, 64)
-    assert sampler._nodes_seen[-1] == got[0].numel() > 4096                 # outgrew the 4096-node buffers, was redone
+    assert state.nodes_seen[-1] == got[0].numel() > 4096                    # outgrew the 4096-node buffers, was redone
     got = sampler.sample_blocks(None, dev_i32(low, cuda))                   # and sized-by-experience again
     check_blocks(oracle, indptr, indices, low, [15, 10, 5], got, 9, 128)
     # the raw entry point reports both kinds of overflow instead of faulting or spinning
@@ -282,9 +283,10 @@ def test_graph_replay_equals_the_oracle_batch_after_batch(cuda, oracle, small_gr
         out = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")  # eager work between replays
         want = oracle.aggregate(b0.edge_ptr.cpu().numpy(), b0.src_global.cpu().numpy(), feat.cpu().numpy(), "mean", 1)
         assert np.abs(out.cpu().numpy() - want).max() < 1e-5
-        if sampler._graphs is not None:
-            captures.add(sampler._graphs[0])
-    assert sampler._graphs is not None and all(slot is not None for slot in sampler._graphs[2])  # graphs were used
+        state = sampler._state_for(seeds_dev[i])
+        if state.graphs is not None:
+            captures.add(state.graphs[0])
+    assert state.graphs is not None and all(slot is not None for slot in state.graphs[2])  # graphs were used
     assert len(captures) >= 2  # ... and captured anew after the plan changed
 
 
@@ -507,3 +509,31 @@ def test_negative_ids_are_reported_not_inserted(cuda):
     meta.zero_()
     L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(probe), 2, None, meta.data_ptr() + 4, L.stream_handle()))
     assert probe.tolist() == [2, 0] and meta.tolist()[1] == 0
+
+
+def test_a_short_last_batch_keeps_what_the_full_batches_learned(cuda, oracle, small_graph):
+    """An epoch ends with a batch of fewer seeds; the next epoch starts with full batches again.  Plans, learned
+    buffer sizes and captured graphs are kept per batch shape, so neither change of shape starts from the
+    worst-case plan again -- also with the next batch launched before the current one is finished."""
+    import fastgl
+    print("sample_blocks: short last batch", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    rng = np.random.default_rng(17)
+    sizes = [600, 600, 600, 150, 600, 600, 150, 600]
+    batches = [rng.permutation(indptr.size - 1)[:n].astype(np.int32) for n in sizes]
+    for pipelined in (False, True):
+        sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=2).set_graph(ptr, idx)
+        seeds_dev = [dev_i32(b, cuda) for b in batches]
+        results = sampler.iter_batches(iter(seeds_dev)) if pipelined else (sampler.sample_blocks(None, s) for s in seeds_dev)
+        plans_full = []
+        for i, got in enumerate(results):
+            check_blocks(oracle, indptr, indices, batches[i], [15, 10, 5], got, 2, i * 64)
+            full = sampler._state_for(seeds_dev[0])
+            plans_full.append({k: id(v) for k, v in full.plans.items()})
+        assert len(sampler._states) == 2
+        full, short = sampler._state_for(seeds_dev[0]), sampler._state_for(seeds_dev[3])
+        assert full.nodes_seen is not None and short.nodes_seen is not None and full.nodes_seen[0] == 600 and short.nodes_seen[0] == 150
+        # the full-size shape's sized-by-experience plan of batch 2 is still the one in use at the end
+        sized = [k for k in plans_full[2] if k is not None]
+        assert sized and all(plans_full[j].get(sized[0]) == plans_full[2][sized[0]] for j in range(3, len(sizes)))
