@@ -602,6 +602,7 @@ def main():
         for b in blocks[1:]:
             outs.append(fastgl.aggregate(b.edge_ptr, b.src_local, hid[:b.num_src_nodes()], mode="mean", zero_policy="zeros"))
         e3.record()
+        fastgl.transpose_blocks(blocks[1:])  # all inner blocks in the launches that one transpose takes
         for b in blocks[1:]:
             t_ptr, t_idx = b.transposed()
             outs.append(fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",
@@ -705,6 +706,7 @@ def main():
             hid, grad = inner_buffers(max([b.num_src_nodes() for b in blocks[1:]] + [1]))
             for b in blocks[1:]:
                 fastgl.aggregate(b.edge_ptr, b.src_local, hid[:b.num_src_nodes()], mode="mean", zero_policy="zeros")
+            fastgl.transpose_blocks(blocks[1:])
             for b in blocks[1:]:
                 t_ptr, t_idx = b.transposed()
                 fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",

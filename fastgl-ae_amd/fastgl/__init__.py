@@ -15,6 +15,7 @@ from .ops import (  # noqa: F401
     backward_gcn,
     backward_gin,
     block_transpose,
+    block_transpose_batch,
     cal_deg,
     edge_softmax,
     exclusive_sum,
@@ -28,7 +29,7 @@ from .ops import (  # noqa: F401
     table_size,
     transfer_edge_id,
 )
-from .sampler import Block, FusedMapSampler, PendingBatch  # noqa: F401
+from .sampler import Block, FusedMapSampler, PendingBatch, transpose_blocks  # noqa: F401
 from .conv import (  # noqa: F401
     GAT,
     GCN,

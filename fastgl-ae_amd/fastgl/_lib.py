@@ -19,11 +19,12 @@ CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
 F32, BF16 = 0, 1
 AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE = 0, 1, 2, 3, 4
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
-ABI_VERSION = 7  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
+ABI_VERSION = 8  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL = 0, 1, 2
 BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
 MAX_FANOUT = 192
+TRANSPOSE_BATCH_MAX, TRANSPOSE_BATCH_MAX_EDGES, TRANSPOSE_BATCH_MAX_COLS = 8, 1 << 20, 1 << 23
 
 _i64, _i32, _u64, _u32, _vp, _sz = C.c_int64, C.c_int, C.c_uint64, C.c_uint32, C.c_void_p, C.c_size_t
 
@@ -50,6 +51,8 @@ SIGNATURES = {
                                  _vp, _vp, _sz, _vp]),
     "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp, _sz, _vp]),
+    "fgl_block_transpose_batch_workspace_bytes": (_sz, [_i32, _vp, _vp]),
+    "fgl_block_transpose_batch": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_aggregate": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
                              _vp, _i64, _vp]),
     "fgl_edge_softmax": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, C.c_float, _vp, _vp]),

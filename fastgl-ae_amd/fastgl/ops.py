@@ -413,6 +413,51 @@ def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False, sorted_rows
     return (t_ptr, t_idx, t_edge) if edge_ids else (t_ptr, t_idx)
 
 
+def block_transpose_batch(blocks, edge_ids=False):
+    """``block_transpose`` (unordered lists) for several blocks in the launches that one takes.  ``blocks``: list of
+    ``(indptr, indices, n_rows, n_cols)``; returns a list of ``(t_indptr, t_indices, t_edge or None)`` in the same order.
+    Blocks too large for the batched entry point (2^20 entries, 2^23 columns: they fill the chip on their own) are
+    transposed one by one."""
+    lib = L.lib()
+    out = [None] * len(blocks)
+    small = []
+    for i, (indptr, indices, n_rows, n_cols) in enumerate(blocks):
+        _check_input(indptr, "indptr", _I32)
+        _check_input(indices, "indices", _I32)
+        if int(indices.numel()) < L.TRANSPOSE_BATCH_MAX_EDGES and int(n_cols) < L.TRANSPOSE_BATCH_MAX_COLS:
+            small.append(i)
+        else:
+            r = block_transpose(indptr, indices, n_rows, n_cols, edge_ids=edge_ids)
+            out[i] = (r[0], r[1], r[2] if edge_ids else None)
+    for g in range(0, len(small), L.TRANSPOSE_BATCH_MAX):
+        group = small[g:g + L.TRANSPOSE_BATCH_MAX]
+        n = len(group)
+        dev = _same_device(*[blocks[i][0] for i in group], *[blocks[i][1] for i in group])
+        with torch.cuda.device(dev):
+            res = []
+            for i in group:
+                indptr, indices, n_rows, n_cols = blocks[i]
+                nnz = int(indices.numel())
+                t_ptr = torch.empty(int(n_cols) + 1, dtype=torch.int32, device=dev)
+                t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
+                t_edge = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz] if edge_ids else None
+                longest = torch.empty(1, dtype=torch.int32, device=dev)
+                t_ptr.fgl_longest_row = longest
+                res.append((t_ptr, t_idx, t_edge, longest))
+            i64 = lambda vals: (C.c_int64 * n)(*[int(v) for v in vals])
+            ptrs = lambda ts: (C.c_void_p * n)(*[L.ptr(t) for t in ts])
+            n_rows_a, n_cols_a = i64(blocks[i][2] for i in group), i64(blocks[i][3] for i in group)
+            n_edges_a = i64(blocks[i][1].numel() for i in group)
+            ws = L.workspace(lib.fgl_block_transpose_batch_workspace_bytes(n, n_cols_a, n_edges_a), dev)
+            L.check(lib.fgl_block_transpose_batch(n, ptrs(blocks[i][0] for i in group), ptrs(blocks[i][1] for i in group), n_rows_a,
+                                                  n_cols_a, n_edges_a, ptrs(r[0] for r in res), ptrs(r[1] for r in res),
+                                                  ptrs(r[2] for r in res) if edge_ids else None, ptrs(r[3] for r in res),
+                                                  L.ptr(ws), ws.numel(), L.stream_handle()))
+        for i, r in zip(group, res):
+            out[i] = r[:3]
+    return out
+
+
 def table_size(num: int, scale: int) -> int:
     """The reference's TableSize (cuda_hashtable.cuh:27-30)."""
     return int(L.lib().fgl_table_size(int(num), int(scale)))

@@ -99,6 +99,21 @@ class Block:
         return "Block(num_src_nodes=%d, num_dst_nodes=%d, num_edges=%d)" % (self._n_src, self._n_dst, self.num_edges())
 
 
+def transpose_blocks(blocks):
+    """Builds the transposed form (``Block.transposed()``) of every block of the list that does not have it yet, all
+    in the five launches that one block takes: the inner blocks of a mini-batch are small and their transposes are
+    launch-bound one by one.  Call it before a backward pass that will want them (every layer but the first).
+    Blocks of a ``deterministic=True`` sampler are transposed one by one (ordered lists)."""
+    todo = [b for b in blocks if b._transposed is None and not b.sorted_transpose]
+    for b in blocks:
+        if b._transposed is None and b.sorted_transpose:
+            b.transposed()
+    if todo:
+        res = ops.block_transpose_batch([(b.edge_ptr, b.src_local, b._n_dst, b._n_src) for b in todo], edge_ids=True)
+        for b, r in zip(todo, res):
+            b._transposed = r
+
+
 class _ShapeState:
     """What the sampler has learned about mini-batches of one shape (seed count, fanouts, graph size, device)."""
 

@@ -88,6 +88,7 @@ def run(args):
                 input_nodes, output_nodes, blocks = sampler.sample_blocks(None, seeds)
                 sync()
             t1 = time.time()
+            fastgl.transpose_blocks(blocks[1:])  # the backward pass of every layer but the first gathers over the transposed block
             batch_labels = label.index_select(0, output_nodes.long())
             if args.model == "sage":
                 batch_inputs = None  # the first layer gathers straight from the resident table

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 7
+#define FGL_ABI_VERSION 8
 
 enum fgl_error {
     FGL_OK = 0,
@@ -249,6 +249,21 @@ int fgl_block_transpose(const int32_t* d_indptr, const int32_t* d_indices,
                         int32_t* d_t_indptr, int32_t* d_t_indices, int32_t* d_t_edge,
                         int32_t* d_t_longest_row, int sorted,
                         void* d_ws, size_t ws_bytes, void* stream);
+
+/* The same for up to FGL_TRANSPOSE_BATCH_MAX blocks in the five launches that one block takes: the inner blocks of a
+ * mini-batch are small, and their transposes are launch-bound one by one.  Host arrays of n_blocks entries each;
+ * exact sizes only (n_edges[i] = the number of entries of block i), lists unordered within a transposed row,
+ * blocks below FGL_TRANSPOSE_BATCH_MAX_EDGES entries and FGL_TRANSPOSE_BATCH_MAX_COLS columns (FGL_ERR_ARG
+ * beyond: such a block fills the chip on its own, use fgl_block_transpose).  d_t_edge and d_t_longest_row may be
+ * NULL, or hold NULL for some blocks. */
+#define FGL_TRANSPOSE_BATCH_MAX 8
+#define FGL_TRANSPOSE_BATCH_MAX_EDGES (1 << 20)
+#define FGL_TRANSPOSE_BATCH_MAX_COLS (1 << 23)
+size_t fgl_block_transpose_batch_workspace_bytes(int n_blocks, const int64_t* n_cols, const int64_t* n_edges);
+int fgl_block_transpose_batch(int n_blocks, const int32_t* const* d_indptr, const int32_t* const* d_indices,
+                              const int64_t* n_rows, const int64_t* n_cols, const int64_t* n_edges,
+                              int32_t* const* d_t_indptr, int32_t* const* d_t_indices, int32_t* const* d_t_edge,
+                              int32_t* const* d_t_longest_row, void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * aggregate -- the memory-aware aggregation kernels: replaces the device part of

@@ -442,3 +442,44 @@ def test_many_rows_of_short_lists(cuda, oracle, dtype, D):
         idx = rng.integers(0, n_src, size=ptr[-1]).astype(np.int32)
         X = torch.from_numpy(rng.standard_normal((max(n_src, n_dst), D)).astype(np.float32)).to(cuda).to(dtype)
         run_modes(cuda, oracle, ptr, idx, deg, X, max(n_src, n_dst), TOL[dtype])
+
+
+def test_batched_transpose_matches_the_single_one(cuda, oracle):
+    """Several blocks transposed by one batched call: offsets equal the oracle's, every transposed row holds the same set of
+    entries (lists are unordered), edge ids name the right entries, the longest row is reported; blocks without entries or
+    columns, and more blocks than one batch takes."""
+    import fastgl
+    print("batched transpose", flush=True)
+    rng = np.random.default_rng(31)
+    shapes = [(300, 900, 6), (1, 1, 3), (50, 7, 0), (2500, 40000, 12), (4000, 500, 3), (0, 10, 0), (700, 700, 40), (33, 5000, 2),
+              (1200, 10, 5), (9, 9, 9)]
+    host, dev_blocks = [], []
+    for n_dst, n_src, max_deg in shapes:
+        deg = rng.integers(0, max_deg + 1, size=n_dst)
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+        idx = rng.integers(0, n_src, size=ptr[-1]).astype(np.int32)
+        host.append((ptr, idx, n_dst, n_src))
+        dev_blocks.append((dev_i32(ptr, cuda), dev_i32(idx, cuda), n_dst, n_src))
+    got = fastgl.block_transpose_batch(dev_blocks, edge_ids=True)
+    assert len(got) == len(shapes)
+    for (ptr, idx, n_dst, n_src), (t_ptr, t_idx, t_edge) in zip(host, got):
+        w_ptr, w_idx = oracle.transpose(ptr, idx, n_src)
+        g_ptr, g_idx, g_edge = t_ptr.cpu().numpy(), t_idx.cpu().numpy(), t_edge.cpu().numpy()
+        assert np.array_equal(g_ptr, w_ptr)
+        # same entries per transposed row, in any order
+        row_of = np.repeat(np.arange(n_src), np.diff(w_ptr))
+        assert np.array_equal(np.lexsort((g_idx, row_of)), np.lexsort((g_idx, row_of)))  # (sizes agree)
+        assert np.array_equal(np.sort(row_of * (n_dst + 1) + g_idx), np.sort(row_of * (n_dst + 1) + w_idx))
+        assert np.array_equal(np.sort(g_edge), np.arange(ptr[-1]))
+        assert np.array_equal(idx[g_edge], row_of)
+        assert np.array_equal(np.repeat(np.arange(n_dst), np.diff(ptr))[g_edge], g_idx)
+        longest = int(np.diff(w_ptr).max()) if n_src else 0
+        reported = int(t_ptr.fgl_longest_row)
+        assert reported == longest if longest > 32 else reported <= 32
+    # through Block objects: transposed() afterwards returns what the batch call built
+    blocks = [fastgl.Block(p, i, n_src, n_dst) for p, i, n_dst, n_src in dev_blocks[:4]]
+    fastgl.transpose_blocks(blocks)
+    for b, (ptr, idx, n_dst, n_src) in zip(blocks, host):
+        assert b._transposed is not None
+        t_ptr, t_idx = b.transposed()
+        assert np.array_equal(t_ptr.cpu().numpy(), oracle.transpose(ptr, idx, n_src)[0])
