@@ -876,7 +876,11 @@ def main():
         "dtype": w["dtype"],
         "data": "synthetic",
         "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
-                   "sampled_edges_per_step": tot_edges / K, "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
+                   "sampled_edges_per_step": tot_edges / K,
+                   "note": "seeds are drawn uniformly from an R-MAT graph without degree noise, so most of them have degree 0-1 "
+                           "(the first hop expands 8192 seeds to ~10 K edges): a mini-batch samples ~1.6 M edges, not the "
+                           "8.6 M that the fanouts would allow",
+                   "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
                    "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
                            "feature table); block transpose + bwd gather on the inner blocks; no dense layers",
                    "readback": ("the batch's sizes reach the host on a second stream while the outermost aggregation runs "
@@ -896,7 +900,8 @@ def main():
                      "frac": agg_gbps / HBM_PEAK_GBPS,
                      "traffic": traffic_from_profile(args.workload, bytes_agg0 / K),
                      "achieved_is": "algorithmic bytes (every sampled edge counted as one row fetch) / kernel time; "
-                                    "traffic = HBM bytes per launch from rocprofv3 counters (repeated rows that hit in cache are not in it)",
+                                    "traffic = bytes per launch that the L2s fetch and write (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled): "
+                                    "repeated rows that hit in L2 are not in it, hits in the memory-side Infinity Cache still are",
                      "kernel": "aggregate_kernel<float,4,32,MEAN> (outermost block, forward)",
                      "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_kernel0 / K * 1e3},
         "cpu_baseline": cpu,

@@ -237,6 +237,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     const int n_counts = 2 * n_hops + 2;
     uint32_t* d_status = reinterpret_cast<uint32_t*>(d_counts + 2 * n_hops + 1);
     FGL_REQUIRE(valid_slots(table_slots), "sample_blocks: slot count %lld is not a power of two in [64, 2^31]", (long long)table_slots);
+    FGL_REQUIRE(((uintptr_t)d_table & 15) == 0 && ((uintptr_t)d_ws & 15) == 0, "sample_blocks: table and workspace must be 16-byte aligned");
     BlocksScratch ws;
     carve_scratch(p, d_ws, &ws);
     const TableRef t = make_ref(d_table, table_slots);

@@ -253,26 +253,32 @@ constexpr int kSelfTilesPerLane = 8;
 #endif
 constexpr int kIdmapSelfPrefixTiles = kBlock * kSelfTilesPerLane;
 
-// A node that has just been given position `local` in the unique list is a seed of the next hop: its row start
-// and degree go to that position.  Returns its min(fanout, degree), which the caller adds to the next hop's
-// per-tile edge counts (entry local / tile_seeds).  An id outside the graph is marked for the next hop's
-// sampling kernel to report.
-__device__ __forceinline__ int prepare_next_hop(const NextHop& next, int32_t id, int64_t local)
+// A node that has just been given a position in the unique list is a seed of the next hop: its row start and
+// degree go to that position (store_next_hop), and its min(fanout, degree) to the next hop's per-tile edge counts.
+// The two graph offsets are read by load_row_of, which callers issue early -- for every edge that may turn out to
+// be a first mention -- so that the reads overlap the pass's own chain of loads.  An id outside the graph is
+// marked for the next hop's sampling kernel to report.
+__device__ __forceinline__ void load_row_of(const NextHop& next, int32_t id, int64_t* a, int64_t* deg)
 {
-    int64_t a = kRowBadId, deg = 0;
+    *a = kRowBadId;
+    *deg = 0;
     if (id >= 0 && (int64_t)id < next.n_nodes) {
         if (next.is64) {
             const int64_t* p = static_cast<const int64_t*>(next.indptr);
-            a = p[id];
-            deg = p[id + 1] - a;
+            *a = p[id];
+            *deg = p[id + 1] - *a;
         } else {
             const int32_t* p = static_cast<const int32_t*>(next.indptr);
-            a = p[id];
-            deg = (int64_t)p[id + 1] - a;
+            *a = p[id];
+            *deg = (int64_t)p[id + 1] - *a;
         }
-        if (deg < 0) deg = 0;
-        if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
+        if (*deg < 0) *deg = 0;
+        if (*deg > 0x7FFFFFFF) *deg = 0x7FFFFFFF;
     }
+}
+
+__device__ __forceinline__ int store_next_hop(const NextHop& next, int64_t local, int64_t a, int64_t deg)
+{
     next.row_start[local] = a;
     next.deg[local] = (int32_t)deg;
     return deg < next.fanout ? (int)deg : next.fanout;
@@ -364,6 +370,12 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
         const int64_t e = base + threadIdx.x;
         int next_k = 0, next_tile = 0;
         const uint32_t p = e < n_e ? slot_of[e] : kDone;
+        int32_t id = 0;
+        int64_t row_a = kRowBadId, row_deg = 0;
+        if (next.row_start != nullptr && p < kDone) {  // most such edges are first mentions: fetch their node's row now
+            id = src[e];
+            load_row_of(next, id, &row_a, &row_deg);
+        }
         if (p != kDone) {
             int64_t local = -1;
             if (p != kEmpty) {
@@ -375,11 +387,11 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                 }
                 if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
                 if (ef == e && local >= 0) {
-                    const int32_t id = src[e];
+                    if (next.row_start == nullptr) id = src[e];
                     uniq[local] = id;
                     if (WRITE_BACK) t.words[2 * (size_t)(p & ~kHolderBit) + 1] = (uint32_t)local;
                     if (next.row_start != nullptr) {
-                        next_k = prepare_next_hop(next, id, local);
+                        next_k = store_next_hop(next, local, row_a, row_deg);
                         next_tile = (int)(local / next.tile_seeds);
                     }
                 }
@@ -501,7 +513,9 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                     out[e] = (int32_t)local;
                     if (next.row_start != nullptr) {
                         // (the tile's new nodes have consecutive positions: few next-hop tiles, summed in LDS first)
-                        const int k = prepare_next_hop(next, (int32_t)id[j], local);
+                        int64_t row_a, row_deg;
+                        load_row_of(next, (int32_t)id[j], &row_a, &row_deg);
+                        const int k = store_next_hop(next, local, row_a, row_deg);
                         if (k != 0) atomicAdd(&s_next[(int)(local / next.tile_seeds - base / next.tile_seeds)], k);
                     }
                 } else {
