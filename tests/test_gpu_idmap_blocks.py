@@ -44,9 +44,9 @@ def test_hand_fixture(cuda):
 
 @pytest.mark.parametrize("n_ids,n_dst,n_edges", [(50, 10, 4000), (100_000, 1000, 15_000), (2**31 - 1, 64, 50_000),
                                                  (3_000_000, 8192, 1_000_000), (7, 7, 0), (1000, 1, 2049),
-                                                 # 1024 tiles of 2048 edges: up to there the numbering pass scans the
+                                                 # 2048 tiles of 2048 edges: up to there the numbering pass scans the
                                                  # tile counts itself, beyond a scan launch does
-                                                 (5_000_000, 4096, 2_097_152), (5_000_000, 4096, 2_097_153),
+                                                 (5_000_000, 4096, 2_097_153), (5_000_000, 4096, 4_194_304), (5_000_000, 4096, 4_194_305),
                                                  (40_000_000, 100, 2_500_000)])
 def test_transfer_edge_id_vs_oracle(cuda, oracle, n_ids, n_dst, n_edges):
     print("idmap %d %d %d" % (n_ids, n_dst, n_edges), flush=True)
@@ -537,3 +537,36 @@ def test_a_short_last_batch_keeps_what_the_full_batches_learned(cuda, oracle, sm
         # the full-size shape's sized-by-experience plan of batch 2 is still the one in use at the end
         sized = [k for k in plans_full[2] if k is not None]
         assert sized and all(plans_full[j].get(sized[0]) == plans_full[2][sized[0]] for j in range(3, len(sizes)))
+
+
+@pytest.mark.parametrize("id_order", ["first", "arrival"])
+@pytest.mark.parametrize("fanouts,n_seeds", [([64, 3], 3000), ([2, 50], 3000), ([33, 20], 700), ([192, 1], 2000), ([3, 3, 3, 3, 3], 4000),
+                                             ([4, 2], 70_000), ([49, 2], 70_000), ([15, 10, 5], 1), ([1], 5000)])
+def test_hops_of_mixed_shapes_chain_correctly(cuda, oracle, small_graph, id_order, fanouts, n_seeds):
+    """Each hop's passes prepare the next hop's sampling (row starts, degrees, per-tile edge counts): fanouts on both sides
+    of the tile-size rules (256-seed tiles only beyond 65 536 seeds and up to fanout 48), of the register-held picks (32)
+    and of the small-hop threshold, so that consecutive hops use different tile sizes and kernels; one to five hops."""
+    import fastgl
+    print("sample_blocks hops %s seeds %d %s" % (fanouts, n_seeds, id_order), flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    rng = np.random.default_rng(len(fanouts) * 1000 + n_seeds)
+    sampler = fastgl.FusedMapSampler(fanouts, rng_seed=12, id_order=id_order).set_graph(ptr, idx)
+    for batch in range(2):  # worst-case buffers first, then sized by experience (and the table left empty by the first)
+        seeds = rng.permutation(indptr.size - 1)[:n_seeds].astype(np.int32)
+        got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        if id_order == "first":
+            check_blocks(oracle, indptr, indices, seeds, fanouts, got, 12, 64 * batch)
+            continue
+        inp, _, blocks = got
+        w_inp, w_blocks = oracle.sample_blocks(indptr, indices, seeds, fanouts, 12, 64 * batch)
+        inp_h = inp.cpu().numpy().astype(np.int64)
+        assert inp_h.size == w_inp.size and np.array_equal(inp_h[:n_seeds], seeds)
+        for b, w in zip(blocks, w_blocks):
+            nd, ns = w["n_dst"], w["n_src"]
+            assert (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()) == (ns, nd, int(w["src_local"].size))
+            assert np.array_equal(np.sort(inp_h[nd:ns]), np.sort(w_inp[nd:ns]))
+            a_src, a_dst = (t.cpu().numpy() for t in b.edges())
+            w_dst = np.repeat(np.arange(nd), np.diff(w["indptr"]))
+            assert np.array_equal(np.sort((inp_h[a_dst] << 32) | inp_h[a_src]),
+                                  np.sort((w_inp[w_dst].astype(np.int64) << 32) | w["src_global"].astype(np.int64)))
