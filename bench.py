@@ -81,6 +81,7 @@ WORKLOADS = {
     "ceiling": None,  # random row gathers from a 48 GB table, see run_ceiling
     "reuse_ab": None,  # outermost block in one launch vs two passes by source id, see run_reuse_ab
     "idmap_stats": None,  # intra-tile repeats and probes per lookup on real mini-batches, see run_idmap_stats
+    "table_access": None,  # random loads and atomics into a hash-table-sized array, whole table vs one eighth per XCD
 }
 DESCRIPTIONS = {
     "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
@@ -96,6 +97,8 @@ DESCRIPTIONS = {
     "reuse_ab": "outermost block of c3 mini-batches (1.5 M gathered rows of 512 B, 1.0 M distinct, 57 GB table): one launch vs "
                 "two launches cut by a source-id threshold",
     "idmap_stats": "c3 mini-batches: ids repeated within a 2048-edge tile per hop; slots probed per lookup in the id-map's table",
+    "table_access": "1.5 M random 8-byte accesses (loads, compare-and-swaps, adds) into tables of 16-128 MB: anywhere, or each XCD "
+                    "inside its own eighth of the table",
     "c4": "aggregation microbench: 8192 dst x exactly 25 src out of 200K rows (int32 CSR), D in {64,128,256,602}, fp32 and bf16, "
           "sum and mean, forward and backward",
 }
@@ -439,6 +442,55 @@ def run_idmap_stats(args):
                       "hops": hops, "probing": stats}), flush=True)
 
 
+def run_table_access(args):
+    """What the memory system gives the id-map's insert pass: 1.5 M random 8-byte accesses (the edges of an outermost hop)
+    into a table of the size the sampler uses, as loads, 64-bit compare-and-swaps, load-then-compare-and-swap and adds --
+    anywhere in the table, and with the workgroups that run on one XCD (every eighth workgroup) confined to one eighth
+    of the table, so that the XCD's L2 holds all that they touch.  Each figure is the best of five launches after a
+    refill of the table, timed with HIP events."""
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n_ops = 1536 * 1024
+    hist = fastgl.probe_xcc_of_workgroups(6144, dev).cpu()
+    on_diagonal = int(hist.diagonal().sum())
+    log("workgroup index % 8 (rows) against the hardware XCC id (columns) for a launch of 6144 workgroups:")
+    for r in range(8):
+        log("   " + " ".join("%5d" % int(v) for v in hist[r, :8]))
+    rows = []
+    for log2_slots in (21, 22, 24):
+        table = torch.empty(1 << log2_slots, dtype=torch.int64, device=dev)
+        for op in fastgl.ops.PROBE_OPS:
+            rec = {"slots_log2": log2_slots, "table_MB": (8 << log2_slots) >> 20, "op": op}
+            for pattern in fastgl.ops.PROBE_PATTERNS:
+                best = None
+                for rep in range(5):
+                    table.fill_(-1)
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    fastgl.probe_table_access(table, n_ops, pattern, op, salt=rep)
+                    e1.record()
+                    e1.synchronize()
+                    us = e0.elapsed_time(e1) * 1e3
+                    best = us if best is None or us < best else best
+                rec[pattern + "_us"] = best
+                rec[pattern + "_Gps"] = n_ops / best / 1e3
+            rows.append(rec)
+            log("table %4d MB  %-20s whole table %6.1f us (%5.1f G/s) | own eighth per XCD %6.1f us (%5.1f G/s) | eighths not aligned %6.1f us"
+                % (rec["table_MB"], op, rec["whole_table_us"], rec["whole_table_Gps"], rec["eighth_of_own_xcd_us"],
+                   rec["eighth_of_own_xcd_Gps"], rec["eighth_not_aligned_us"]))
+        del table
+    cas = [r for r in rows if r["op"] == "cas" and r["slots_log2"] == 22][0]
+    print(json.dumps({"metric": "random 8-byte accesses into a 32 MB table: 64-bit compare-and-swaps per second", "value": cas["whole_table_Gps"] * 1e9,
+                      "unit": "atomics/s", "n_gpus": 1, "steps": 5, "warmup": 0, "ms_per_step": cas["whole_table_us"] / 1e3,
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u64", "data": "synthetic",
+                      "config": {"workload": DESCRIPTIONS["table_access"]}, "roofline": None, "cpu_baseline": None,
+                      "workgroups_on_the_xcd_of_their_index_mod_8": on_diagonal, "workgroups": 6144, "accesses": n_ops, "cases": rows}), flush=True)
+
+
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
@@ -510,6 +562,8 @@ def main():
         return run_reuse_ab(args)
     if args.workload == "idmap_stats":
         return run_idmap_stats(args)
+    if args.workload == "table_access":
+        return run_table_access(args)
     w = WORKLOADS[args.workload]
     N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
     fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16

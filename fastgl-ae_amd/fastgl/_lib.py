@@ -19,7 +19,7 @@ CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
 F32, BF16 = 0, 1
 AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE = 0, 1, 2, 3, 4
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
-ABI_VERSION = 8  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
+ABI_VERSION = 9  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL = 0, 1, 2
 BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
@@ -57,6 +57,8 @@ SIGNATURES = {
                              _vp, _i64, _vp]),
     "fgl_edge_softmax": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, C.c_float, _vp, _vp]),
     "fgl_rmat_keys": (_i32, [_i64, _i64, _i32, _i64, _u64, _vp, _vp]),
+    "fgl_probe_table_access": (_i32, [_vp, _i64, _i64, _i32, _i32, _u32, _vp, _vp]),
+    "fgl_probe_xcc_of_workgroups": (_i32, [_vp, _i32, _vp]),
 }
 
 _lib = None

@@ -549,3 +549,25 @@ def rmat_keys(first_edge: int, n_edges: int, scale: int, n_nodes: int, seed: int
         L.check(L.lib().fgl_rmat_keys(int(first_edge), int(n_edges), int(scale), int(n_nodes),
                                       int(seed) & 0xFFFFFFFFFFFFFFFF, L.ptr(keys), L.stream_handle()))
     return keys
+
+
+PROBE_OPS = {"load": 0, "cas": 1, "load_then_cas": 2, "add": 3, "cas_workgroup_scope": 4}
+PROBE_PATTERNS = {"whole_table": 0, "eighth_of_own_xcd": 1, "eighth_not_aligned": 2}
+
+
+def probe_table_access(table: torch.Tensor, n_ops: int, pattern: str, op: str, salt: int = 0) -> None:
+    """One pseudo-random 8-byte access per lane into ``table`` (int64, a power of two of entries); see
+    ``fgl_probe_table_access`` in include/fastgl_hip.h.  Enqueues on the current stream."""
+    _check_input(table, "table", (torch.int64,))
+    with torch.cuda.device(table.device):
+        sink = torch.zeros(1, dtype=torch.int64, device=table.device)
+        L.check(L.lib().fgl_probe_table_access(L.ptr(table), int(table.numel()), int(n_ops), PROBE_PATTERNS[pattern],
+                                               PROBE_OPS[op], int(salt) & 0xFFFFFFFF, L.ptr(sink), L.stream_handle()))
+
+
+def probe_xcc_of_workgroups(n_workgroups: int, device) -> torch.Tensor:
+    """8 x 16 counts: entry [w % 8, x] = workgroups of index w that ran on the XCD whose hardware id is x."""
+    with torch.cuda.device(device):
+        hist = torch.zeros((8, 16), dtype=torch.int32, device=device)
+        L.check(L.lib().fgl_probe_xcc_of_workgroups(L.ptr(hist), int(n_workgroups), L.stream_handle()))
+    return hist

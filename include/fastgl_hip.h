@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 8
+#define FGL_ABI_VERSION 9
 
 enum fgl_error {
     FGL_OK = 0,
@@ -319,6 +319,26 @@ int fgl_edge_softmax(const int32_t* d_indptr, const int32_t* d_indices, int64_t 
  * ------------------------------------------------------------------------------- */
 int fgl_rmat_keys(int64_t first_edge, int64_t n_edges, int scale, int64_t n_nodes, uint64_t seed,
                   int64_t* d_keys, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * Probes of the memory system behind the id-map's design.  No counterpart in the reference; they exist so
+ * that the figures the design rests on can be re-measured on any box (bench.py --workload table_access).
+ *
+ * fgl_probe_table_access: n_ops lanes each make one access to a pseudo-random 8-byte slot of d_table
+ * (`slots` of them, a power of two; fill it with 0xFF bytes first).
+ *   pattern  0 anywhere; 1 inside the eighth of the table numbered (workgroup index % 8) -- workgroups are
+ *            dealt to the 8 XCDs in turn, so that is "each XCD on its own eighth"; 2 inside the eighth
+ *            ((workgroup index / 8) % 8): as partitioned, but every XCD touches every eighth
+ *   op       0 load; 1 64-bit compare-and-swap of an empty slot; 2 load, then that compare-and-swap if the slot
+ *            was empty; 3 32-bit add without a return value; 4 the compare-and-swap at workgroup scope
+ * d_sink: 8 bytes that the kernel may write (keeps the loads alive).
+ *
+ * fgl_probe_xcc_of_workgroups: launches n_workgroups workgroups; d_hist (8 x 16 uint32, zeroed by the caller)
+ * [(workgroup index % 8) * 16 + hardware XCC id] counts them.
+ * ------------------------------------------------------------------------------- */
+int fgl_probe_table_access(void* d_table, int64_t slots, int64_t n_ops, int pattern, int op, uint32_t salt,
+                           uint64_t* d_sink, void* stream);
+int fgl_probe_xcc_of_workgroups(uint32_t* d_hist, int n_workgroups, void* stream);
 
 #ifdef __cplusplus
 }

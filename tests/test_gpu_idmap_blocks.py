@@ -570,3 +570,30 @@ def test_hops_of_mixed_shapes_chain_correctly(cuda, oracle, small_graph, id_orde
             w_dst = np.repeat(np.arange(nd), np.diff(w["indptr"]))
             assert np.array_equal(np.sort((inp_h[a_dst] << 32) | inp_h[a_src]),
                                   np.sort((w_inp[w_dst].astype(np.int64) << 32) | w["src_global"].astype(np.int64)))
+
+
+def test_memory_probes_touch_what_they_say(cuda):
+    """The two diagnostic entry points behind `bench.py --workload table_access`."""
+    import fastgl
+    print("probe_table_access / probe_xcc_of_workgroups", flush=True)
+    n_ops = 100_000
+    table = torch.zeros(1 << 16, dtype=torch.int64, device=cuda)
+    fastgl.probe_table_access(table, n_ops, "whole_table", "add")
+    assert int(table.sum()) == n_ops  # one 32-bit add per lane, nothing lost
+    # a single workgroup (index 0) confined to its eighth of the table
+    table.fill_(-1)
+    fastgl.probe_table_access(table, 256, "eighth_of_own_xcd", "cas")
+    touched = torch.nonzero(table != -1).flatten()
+    assert 0 < touched.numel() <= 256 and int(touched.max()) < (1 << 16) // 8
+    assert int(table[touched].max()) < 256 and int(table[touched].min()) >= 0  # the lane index that won the slot
+    # workgroup 8 + k of the other partitioned pattern uses eighth 1
+    table.fill_(-1)
+    fastgl.probe_table_access(table, 16 * 256, "eighth_not_aligned", "cas_workgroup_scope")
+    touched = torch.nonzero(table != -1).flatten()
+    assert int(touched.max()) < 2 * ((1 << 16) // 8)
+    for op in ("load", "load_then_cas"):
+        fastgl.probe_table_access(table, n_ops, "whole_table", op, salt=3)
+    hist = fastgl.probe_xcc_of_workgroups(800, cuda).cpu()
+    assert int(hist.sum()) == 800 and hist.sum(dim=1).tolist() == [100] * 8
+    with pytest.raises(RuntimeError, match="power of two"):
+        fastgl.probe_table_access(torch.zeros(1000, dtype=torch.int64, device=cuda), 10, "whole_table", "load")
