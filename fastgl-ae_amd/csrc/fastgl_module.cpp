@@ -99,6 +99,8 @@ struct Transposed {
 Transposed transpose(const torch::Tensor& indptr, const torch::Tensor& indices, int64_t n_rows, int64_t n_cols, bool edge_ids)
 {
     const int64_t nnz = indices.numel();
+    TORCH_CHECK(n_rows >= 0 && n_rows <= indptr.numel() - 1, "row count ", n_rows, " does not match the offsets (", indptr.numel(), " entries)");
+    TORCH_CHECK(n_cols >= 0, "negative node count");
     auto opt = indptr.options();
     Transposed t;
     t.ptr = torch::empty({n_cols + 1}, opt);

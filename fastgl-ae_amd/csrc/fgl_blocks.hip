@@ -119,6 +119,8 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
         FGL_REQUIRE(fanouts[h] >= 1 && fanouts[h] <= FGL_MAX_FANOUT, "sample_blocks: fanout %d outside [1, %d]", fanouts[h], FGL_MAX_FANOUT);
         if (node_capacity) {
             FGL_REQUIRE(node_capacity[h] >= n_seeds, "sample_blocks: node_capacity[%d] = %lld is below the seed count", h, (long long)node_capacity[h]);
+            // (a hop's nodes are a prefix of the next hop's: the bounds must not shrink, the workspace layout relies on it)
+            FGL_REQUIRE(h == 0 || node_capacity[h] >= p->cap_dst[h - 1], "sample_blocks: node_capacity[%d] is below an earlier entry", h);
             if (cur > node_capacity[h]) cur = node_capacity[h];
         }
         p->cap_dst[h] = cur;

@@ -189,7 +189,8 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * passes them already reversed.)
  *
  * node_capacity (optional, n_hops+1 host entries, NULL = none): the caller's own limit on the
- * number of nodes before hop h (last entry: after the last hop).  Worst-case bounds assume
+ * number of nodes before hop h (last entry: after the last hop); every entry at least the seed
+ * count and none below the one before it.  Worst-case bounds assume
  * that no neighbour ever repeats; for deep fanouts they reach the size of the graph, so a
  * caller that knows its batches may size its buffers by experience instead.  A batch that
  * grows past a limit sets FGL_STATUS_UNIQ_OVERFLOW (its outputs are then invalid, nothing is

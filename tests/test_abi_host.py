@@ -56,6 +56,10 @@ def test_plan_matches_the_worst_case_table():
     assert list(cd) == [100, 300, 400] and list(ce) == [500, 3000, 6000] and cu.value == 500
     bad = (C.c_int64 * 4)(50, 300, 400, 500)
     assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, bad, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
+    # limits that shrink from one hop to the next are refused (a hop's nodes are a prefix of the next hop's)
+    shrinking = (C.c_int64 * 4)(100, 400, 300, 500)
+    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, shrinking, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
+    assert b"below an earlier entry" in fastgl.lib().fgl_last_error()
 
 
 def test_argument_errors_are_reported_not_launched():
