@@ -597,3 +597,72 @@ def test_memory_probes_touch_what_they_say(cuda):
     assert int(hist.sum()) == 800 and hist.sum(dim=1).tolist() == [100] * 8
     with pytest.raises(RuntimeError, match="power of two"):
         fastgl.probe_table_access(torch.zeros(1000, dtype=torch.int64, device=cuda), 10, "whole_table", "load")
+
+
+def _csr_from_rows(rows, ptr_dtype=np.int64):
+    indptr = np.zeros(len(rows) + 1, dtype=ptr_dtype)
+    indptr[1:] = np.cumsum([len(r) for r in rows])
+    return indptr, np.asarray([v for r in rows for v in r], dtype=np.int32)
+
+
+@pytest.mark.parametrize("id_order", ["first", "arrival"])
+def test_hand_built_graphs_with_repeated_neighbours_self_loops_and_a_hub(cuda, oracle, id_order):
+    """Graphs that an R-MAT generator never makes: rows that list a neighbour several times and themselves (the
+    sampler draws positions, so such rows give repeated sources within one seed), rows of exactly fanout - 1,
+    fanout and fanout + 1 entries, isolated nodes -- and a star: every node lists the hub, so the hub's row of the
+    transposed block holds one entry per seed (far beyond the 128 entries that the backward gather leaves to its
+    hub-row launch).  Sampling, id-map, forward and backward gathers against the oracle."""
+    import fastgl
+    print("hand-built graphs, id_order=%s" % id_order, flush=True)
+    rng = np.random.default_rng(17)
+    n = 3000
+    rows = []
+    for v in range(n):
+        kind = v % 6
+        if kind == 0:
+            row = []                                             # isolated
+        elif kind == 1:
+            row = [v, v, (v + 1) % n]                            # self loops, one of them twice
+        elif kind == 2:
+            row = [(v + 7) % n] * 9                              # one neighbour nine times
+        else:
+            row = rng.integers(0, n, size=(3, 4, 5)[kind - 3]).tolist()  # fanout - 1, fanout, fanout + 1 entries
+        rows.append([0] + row if v != 0 else row)                # the star: everyone lists node 0 first
+    indptr, indices = _csr_from_rows(rows)
+    ptr, idx = load_graph(cuda, indptr, indices)
+    fanouts = [4, 4]
+    seeds = rng.permutation(n)[:2000].astype(np.int32)
+    sampler = fastgl.FusedMapSampler(fanouts, rng_seed=9, id_order=id_order).set_graph(ptr, idx)
+    for batch in range(2):
+        got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        inp, _, blocks = got
+        w_inp, w_blocks = oracle.sample_blocks(indptr, indices, seeds, fanouts, 9, batch * 64)
+        if id_order == "first":
+            check_blocks(oracle, indptr, indices, seeds, fanouts, got, 9, batch * 64)
+        else:  # any numbering of the new ids is a valid map: compare the edges in graph ids, hop by hop
+            uniq = inp.cpu().numpy()
+            for b, w in zip(blocks, w_blocks):
+                assert (b.num_src_nodes(), b.num_dst_nodes()) == (w["n_src"], w["n_dst"])
+                src, dst = b.edges()
+                got_keys = np.sort(uniq[dst.cpu().numpy()].astype(np.int64) << 32 | uniq[src.cpu().numpy()])
+                want_keys = np.sort(w_inp[np.repeat(np.arange(w["n_dst"]), np.diff(w["indptr"]))].astype(np.int64) << 32 | w["src_global"])
+                assert np.array_equal(got_keys, want_keys)
+            assert np.array_equal(np.sort(uniq), np.sort(w_inp))
+    # the outermost block: forward mean, then the backward gather over its transpose, whose hub row is long
+    b = blocks[0]
+    n_src, n_dst = b.num_src_nodes(), b.num_dst_nodes()
+    ptr_h, src_h = b.edge_ptr.cpu().numpy(), b.src_local.cpu().numpy()
+    hub_local = int(np.flatnonzero(inp.cpu().numpy() == 0)[0])
+    assert int((src_h == hub_local).sum()) > 1000
+    X = torch.from_numpy(rng.standard_normal((n_src, 48)).astype(np.float32)).to(cuda)
+    out = fastgl.aggregate(b.edge_ptr, b.src_local, X, mode="mean", zero_policy="zeros", n_rows=n_dst)
+    want = oracle.aggregate(ptr_h, src_h, X.cpu().numpy(), "mean", 1)
+    assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * max(np.abs(want).max(), 1.0)
+    t_ptr, t_idx = b.transposed()[:2]
+    assert int(torch.diff(t_ptr).max()) > 1000  # the hub
+    d_out = torch.from_numpy(rng.standard_normal((n_dst, 48)).astype(np.float32)).to(cuda)
+    d_x = fastgl.aggregate(t_ptr, t_idx, d_out, mode="colmean", zero_policy="zeros", col_norm=b.in_degrees().contiguous(), n_rows=n_src)
+    tp, ti = oracle.transpose(ptr_h, src_h, n_src)
+    deg = np.maximum(np.diff(ptr_h), 1).astype(np.int32)
+    want = oracle.aggregate(tp, ti, d_out.cpu().numpy(), "colmean", 1, None, deg)
+    assert np.abs(d_x.cpu().numpy() - want).max() <= 1e-5 * max(np.abs(want).max(), 1.0)
