@@ -378,7 +378,6 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
     using IO = RowIO<T, VEC>;
     constexpr int kGroups = kBlock / LPR;
     const int32_t* __restrict__ indptr = g.indptr;
-    const int32_t* __restrict__ indices = g.indices;
     const T* __restrict__ X = static_cast<const T*>(g.x);
     T* __restrict__ out = static_cast<T*>(g.out);
     const int64_t ldx = g.ldx, ldo = g.ldo;

@@ -42,19 +42,23 @@ __global__ __launch_bounds__(TS) void blocks_prepare_kernel(TableRef t, const vo
             if (uniq != seeds) uniq[i] = s;
             int64_t a = kRowBadId, deg = 0;
             if (s >= 0 && (int64_t)s < n_nodes) {
+                int64_t b;
                 if (is64) {
                     const int64_t* p = static_cast<const int64_t*>(indptr);
                     a = p[s];
-                    deg = p[s + 1] - a;
+                    b = p[s + 1];
                 } else {
                     const int32_t* p = static_cast<const int32_t*>(indptr);
                     a = p[s];
-                    deg = (int64_t)p[s + 1] - a;
+                    b = p[s + 1];
                 }
+                // (the table probe goes out before the two offsets are looked at: one wait for both)
+                uint32_t seen;
+                const bool full = find_or_insert(t, (uint32_t)s, (uint32_t)i, &seen) == kEmpty;  // a repeated seed keeps its first position
+                deg = b - a;
                 if (deg < 0) deg = 0;
                 if (deg > 0x7FFFFFFF) deg = 0x7FFFFFFF;
-                uint32_t seen;
-                if (find_or_insert(t, (uint32_t)s, (uint32_t)i, &seen) == kEmpty) {  // a repeated seed keeps its first position
+                if (full) {
                     a = kRowTableFull;
                     deg = 0;
                 }

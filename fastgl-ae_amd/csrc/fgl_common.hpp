@@ -110,11 +110,19 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* smem, int* total
 // of tile t derive its own exclusive prefix from the per-tile sums of an earlier launch, which
 // saves the single-workgroup scan launch in between while the tile count is small.
 template <int NT>
-__device__ __forceinline__ int block_sum_before(const int32_t* __restrict__ v, int64_t count, int* smem)
+__device__ __forceinline__ int lane_sum_before(const int32_t* __restrict__ v, int64_t count)
 {
-    constexpr int NW = NT / kWave;
     int s = 0;
     for (int64_t i = threadIdx.x; i < count; i += NT) s += v[i];
+    return s;
+}
+
+// (lane_sum_before, then this: a caller with other loads to wait for issues those between the two, so that both
+// sets are in flight together)
+template <int NT>
+__device__ __forceinline__ int block_sum_of_lanes(int s, int* smem)
+{
+    constexpr int NW = NT / kWave;
 #pragma unroll
     for (int d = kWave / 2; d >= 1; d >>= 1) s += __shfl_xor(s, d, kWave);
     if (lane_id() == 0) smem[threadIdx.x / kWave] = s;
@@ -124,6 +132,12 @@ __device__ __forceinline__ int block_sum_before(const int32_t* __restrict__ v, i
     for (int w = 0; w < NW; ++w) sum += smem[w];
     __syncthreads();
     return sum;
+}
+
+template <int NT>
+__device__ __forceinline__ int block_sum_before(const int32_t* __restrict__ v, int64_t count, int* smem)
+{
+    return block_sum_of_lanes<NT>(lane_sum_before<NT>(v, count), smem);
 }
 
 // Philox4x32-10 (Salmon et al., SC'11): the counter-based generator the reference uses

@@ -337,6 +337,19 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
     __shared__ int smem[kBlock / kWave + 1];
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    // What the first trip of the loop below reads about its edge is fetched now, so that it travels together with
+    // the tile counts that the scan waits for (a small hop is one trip per workgroup: a chain of memory latencies).
+    uint32_t p_ahead = kDone, first_ahead = 0;
+    int32_t id_ahead = 0;
+    {
+        const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+        if (e < n_e) {
+            p_ahead = slot_of[e];
+            first_ahead = first_of[e];
+            id_ahead = src[e];
+        }
+    }
     if constexpr (SELF) {
         const int n_tiles = (int)tiles_of(n_e);  // <= kIdmapSelfPrefixTiles: the launcher checks the bound
         int v[kSelfTilesPerLane];
@@ -357,7 +370,6 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
         __syncthreads();
         if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status);
     }
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
     // the last pass of a mini-batch, which no longer reads the table, can leave it empty for the next one
     // (first, so that the stores drain while the edges are being numbered)
     if (!WRITE_BACK && clear_words != nullptr) {
@@ -369,17 +381,18 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
     for (int64_t base = (int64_t)blockIdx.x * kBlock; base < n_e; base += stride) {
         const int64_t e = base + threadIdx.x;
         int next_k = 0, next_tile = 0;
-        const uint32_t p = e < n_e ? slot_of[e] : kDone;
-        int32_t id = 0;
+        const bool first_trip = base == (int64_t)blockIdx.x * kBlock;
+        const uint32_t p = first_trip ? p_ahead : (e < n_e ? slot_of[e] : kDone);
+        int32_t id = first_trip ? id_ahead : 0;
         int64_t row_a = kRowBadId, row_deg = 0;
         if (next.row_start != nullptr && p < kDone) {  // most such edges are first mentions: fetch their node's row now
-            id = src[e];
+            if (!first_trip) id = src[e];
             load_row_of(next, id, &row_a, &row_deg);
         }
         if (p != kDone) {
             int64_t local = -1;
             if (p != kEmpty) {
-                const int64_t ef = (int64_t)(first_of[e] & ~kPending);  // first edge of this edge's id (ef <= e)
+                const int64_t ef = (int64_t)((first_trip ? first_ahead : first_of[e]) & ~kPending);  // first edge of this edge's id (ef <= e)
                 if (ef < n_e) {
                     const int64_t tile = ef / kTile;
                     const int before_tile = SELF ? s_prefix[tile] : tile_prefix[tile];
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                 }
                 if (local >= capacity) local = -1;  // the unique list is full (reported with the node total)
                 if (ef == e && local >= 0) {
-                    if (next.row_start == nullptr) id = src[e];
+                    if (next.row_start == nullptr && !first_trip) id = src[e];
                     uniq[local] = id;
                     if (WRITE_BACK) t.words[2 * (size_t)(p & ~kHolderBit) + 1] = (uint32_t)local;
                     if (next.row_start != nullptr) {

@@ -103,12 +103,12 @@ __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restric
 // count is small) the workgroup sums the earlier tiles' sums itself, and the workgroup of the last
 // tile also publishes the edge total: block_ptr[n] and *n_edges_out.
 template <int TS>
-__device__ __forceinline__ int tile_base(const int32_t* __restrict__ tile_sums, const int32_t* __restrict__ tile_prefix,
-                                         int64_t tile, int64_t n_tiles, int64_t n, int tile_total, int* smem,
+__device__ __forceinline__ int tile_base(int lane_sum_of_earlier_tiles, const int32_t* __restrict__ tile_prefix, int64_t tile,
+                                         int64_t n_tiles, int64_t n, int tile_total, int* smem,
                                          int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
 {
     if (tile_prefix) return tile_prefix[tile];
-    const int base = block_sum_before<TS>(tile_sums, tile, smem);
+    const int base = block_sum_of_lanes<TS>(lane_sum_of_earlier_tiles, smem);
     if (tile == n_tiles - 1 && threadIdx.x == 0) {
         block_ptr[n] = base + tile_total;
         if (n_edges_out) *n_edges_out = base + tile_total;
@@ -190,11 +190,13 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
             row = row_start[i];
             seed = seeds[i];
         }
+        // (the earlier tiles' sums are fetched while the seed's own three loads are still under way)
+        const int sum_before = tile_prefix ? 0 : lane_sum_before<TS>(tile_sums, tile);
         seed_checks_and_next_hop<TS>(i < n, tile, row, deg, d_status, next_fanout, next_tile_seeds, next_tile_sums);
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_base<TS>(tile_sums, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
+        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
         s_off[tid] = ex;
         if (tid == 0) s_off[TS] = total;
         s_row[tid] = row;
@@ -291,11 +293,13 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
             row = row_start[i];
             seed = seeds[i];
         }
+        // (the earlier tiles' sums are fetched while the seed's own three loads are still under way)
+        const int sum_before = tile_prefix ? 0 : lane_sum_before<TS>(tile_sums, tile);
         seed_checks_and_next_hop<TS>(i < n, tile, row, deg, d_status, next_fanout, next_tile_seeds, next_tile_sums);
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_base<TS>(tile_sums, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
+        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
         if (i < n) block_ptr[i] = base + ex;
 
         uint32_t sel[F];
