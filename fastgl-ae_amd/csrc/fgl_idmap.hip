@@ -508,6 +508,13 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                 }
             }
         }
+        // the new nodes' rows in the graph (for the next hop) are fetched while the workgroup takes its numbers
+        int64_t row_a[ITEMS], row_deg[ITEMS];
+        if (next.row_start != nullptr) {
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j)
+                if ((won >> j) & 1u) load_row_of(next, (int32_t)id[j], &row_a[j], &row_deg[j]);
+        }
         int total;
         int rank = block_exclusive_scan<kBlock>(__popc(won), smem, &total);
         if (threadIdx.x == 0) s_base = total ? atomicAdd(counter, total) : 0;
@@ -526,9 +533,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                     out[e] = (int32_t)local;
                     if (next.row_start != nullptr) {
                         // (the tile's new nodes have consecutive positions: few next-hop tiles, summed in LDS first)
-                        int64_t row_a, row_deg;
-                        load_row_of(next, (int32_t)id[j], &row_a, &row_deg);
-                        const int k = store_next_hop(next, local, row_a, row_deg);
+                        const int k = store_next_hop(next, local, row_a[j], row_deg[j]);
                         if (k != 0) atomicAdd(&s_next[(int)(local / next.tile_seeds - base / next.tile_seeds)], k);
                     }
                 } else {
