@@ -179,3 +179,41 @@ def test_traffic_record_is_only_used_while_it_matches(tmp_path, monkeypatch, cap
     assert bench.traffic_from_profile("c3", 800e6) is None       # the kernel has changed since
     monkeypatch.setattr(bench, "TRAFFIC_PROFILE", str(tmp_path / "missing.md"))
     assert bench.traffic_from_profile("c3", 800e6) is None
+
+
+def test_size_limits_are_stated_before_anything_is_launched():
+    """Sizes that would overflow the library's 32-bit offsets come back as errors with the limit in the message."""
+    lib = fastgl.lib()
+    fake = C.c_void_p(0x1000)  # never dereferenced: every call below fails its size checks first
+    # seeds x fanout beyond int32 edge offsets
+    assert lib.fgl_sample_node(fake, 1, fake, 10, fake, 20_000_000, None, 192, 0, 0, fake, None, fake, None, None, fake, 1 << 40, None) == 1
+    assert b"overflows int32" in lib.fgl_last_error()
+    # a hop of the all-hops plan that could produce more than 2^31 edges
+    fan = (C.c_int32 * 2)(192, 192)
+    assert lib.fgl_sample_blocks_plan(1 << 30, 20_000_000, fan, 2, None, None, None, None, None, None) == 1
+    assert b"beyond int32" in lib.fgl_last_error()
+    # hop counts and fanouts outside the supported range
+    fan1 = (C.c_int32 * 1)(193)
+    assert lib.fgl_sample_blocks_plan(100, 10, fan1, 1, None, None, None, None, None, None) == 1
+    assert b"fanout" in lib.fgl_last_error()
+    fan33 = (C.c_int32 * 33)(*([2] * 33))
+    assert lib.fgl_sample_blocks_plan(100, 10, fan33, 33, None, None, None, None, None, None) == 1
+    assert b"hops" in lib.fgl_last_error()
+    # an id-map call whose local ids would not fit 31 bits next to the pending marker
+    assert lib.fgl_idmap_map_src(fake, 64, fake, fake, (1 << 31) - 1, None, 10, None, None, fake, 100, 0, None, fake, 1 << 40, None) == 1
+    assert b"31 bits" in lib.fgl_last_error()
+    # a table that is not a power of two
+    assert lib.fgl_idmap_insert_dst(fake, 1000, fake, 10, None, None, None, None) == 1
+    assert b"power of two" in lib.fgl_last_error()
+    # more ids than a table takes at load 1/2
+    assert lib.fgl_idmap_insert_dst(fake, 64, fake, 33, None, None, None, None) == 1
+    assert b"load 1/2" in lib.fgl_last_error()
+    # a transpose of more than 2^31 - 1 entries, and a batched one of a block that is too large for it
+    assert lib.fgl_block_transpose(fake, fake, 10, None, 10, None, 1 << 31, fake, fake, None, None, 0, fake, 1 << 40, None) == 1
+    assert b"int32 offsets" in lib.fgl_last_error()
+    one = lambda v: (C.c_int64 * 1)(v)
+    pp = (C.c_void_p * 1)(0x1000)
+    assert lib.fgl_block_transpose_batch(1, pp, pp, one(10), one(10), one(1 << 20), pp, pp, None, None, fake, 1 << 40, None) == 1
+    assert b"too large" in lib.fgl_last_error()
+    assert lib.fgl_block_transpose_batch(9, pp, pp, one(10), one(10), one(10), pp, pp, None, None, fake, 1 << 40, None) == 1
+    assert b"blocks outside" in lib.fgl_last_error()
