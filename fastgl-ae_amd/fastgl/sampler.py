@@ -74,7 +74,11 @@ class Block:
 
     def out_degrees(self):
         if self._src_deg is None:
-            self._src_deg = ops.cal_deg(self.src_local, self._n_src)
+            if self._transposed is not None:  # the transposed block's row lengths: no histogram pass
+                t_ptr = self._transposed[0]
+                self._src_deg = t_ptr[1:] - t_ptr[:-1]
+            else:
+                self._src_deg = ops.cal_deg(self.src_local, self._n_src)
         return self._src_deg
 
     def transposed(self, edge_ids=False):

@@ -666,3 +666,22 @@ def test_hand_built_graphs_with_repeated_neighbours_self_loops_and_a_hub(cuda, o
     deg = np.maximum(np.diff(ptr_h), 1).astype(np.int32)
     want = oracle.aggregate(tp, ti, d_out.cpu().numpy(), "colmean", 1, None, deg)
     assert np.abs(d_x.cpu().numpy() - want).max() <= 1e-5 * max(np.abs(want).max(), 1.0)
+
+
+def test_block_degrees_with_and_without_the_transpose(cuda, oracle, small_graph):
+    """``Block.out_degrees()`` counts with a histogram pass, or reads the transposed block's row lengths if the
+    transpose is already there: the same numbers either way."""
+    import fastgl
+    print("Block.in_degrees / out_degrees", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    seeds = np.random.default_rng(2).permutation(indptr.size - 1)[:2048].astype(np.int32)
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=1).set_graph(ptr, idx)
+    for transposed_first in (False, True):
+        _, _, blocks = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+        if transposed_first:
+            fastgl.transpose_blocks(blocks)
+        for b in blocks:
+            src = b.src_local.cpu().numpy()
+            assert np.array_equal(b.out_degrees().cpu().numpy(), np.bincount(src, minlength=b.num_src_nodes()))
+            assert np.array_equal(b.in_degrees().cpu().numpy(), np.diff(b.edge_ptr.cpu().numpy()))
