@@ -500,6 +500,37 @@ def run_table_access(args):
                       "workgroups_on_the_xcd_of_their_index_mod_8": on_diagonal, "workgroups": 6144, "accesses": n_ops, "cases": rows}), flush=True)
 
 
+def time_dgl_cpu_path(h_ptr, h_src, train, B, fanouts, n_batches):
+    """The reference's own CPU sampling path -- DGL's `sample_neighbors` + `to_block` per hop, as its
+    DGLNeighborSampler drives them (FusedMapSampler.py:130-148) -- timed on the same mini-batches, if a DGL
+    happens to be importable on this box.  It is not part of the image this library is built and tested in, so
+    this leg normally reports that it was skipped; nothing is ever installed or downloaded for it."""
+    try:
+        import dgl  # noqa: F401
+        import torch
+    except Exception as exc:  # not installed: the usual case
+        return {"timed": False, "why": "dgl is not importable here (%s)" % type(exc).__name__}
+    try:
+        n = int(h_ptr.shape[0]) - 1
+        g = dgl.graph(("csc", (torch.from_numpy(h_ptr.astype("int64")), torch.from_numpy(h_src.astype("int64")), torch.tensor([], dtype=torch.int64))),
+                      num_nodes=n)
+        edges, t = 0, 0.0
+        for i in range(n_batches):
+            seeds = train[i * B:(i + 1) * B].cpu().long()
+            t0 = time.perf_counter()
+            for fanout in reversed(fanouts):
+                frontier = g.sample_neighbors(seeds, fanout, edge_dir="in", replace=False)
+                block = dgl.to_block(frontier, seeds)
+                seeds = block.srcdata[dgl.NID]
+                edges += int(block.num_edges())
+            t += time.perf_counter() - t0
+        log("DGL %s on the host: %.3g sampled edges/s" % (dgl.__version__, edges / t))
+        return {"timed": True, "version": dgl.__version__, "value": edges / t, "unit": "sampled edges/s",
+                "threads": torch.get_num_threads(), "sample": "%d mini-batches of %d seeds" % (n_batches, B)}
+    except Exception as exc:
+        return {"timed": False, "why": "dgl is importable but the run failed: %r" % (exc,)}
+
+
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
@@ -923,6 +954,7 @@ def main():
                "value_sequential_idmap": cpu_edges / cpu_t_seq,
                "aggregation_GBps": agg_bytes / agg_t / 1e9, "host_cpus": os.cpu_count()}
         log("cpu baseline: %.3g edges/s (%d threads), aggregation %.1f GB/s" % (cpu["value"], cpu["cores"], cpu["aggregation_GBps"]))
+        cpu["dgl"] = time_dgl_cpu_path(h_ptr, h_src, train, B, w["fanouts"], min(args.cpu_batches, 16))
 
     out = {
         "metric": "sampled edges/s (sample+id_map) + aggregation HBM GB/s (% peak), 1 MI355X",
