@@ -81,7 +81,6 @@ WORKLOADS = {
     "ceiling": None,  # random row gathers from a 48 GB table, see run_ceiling
     "reuse_ab": None,  # outermost block in one launch vs two passes by source id, see run_reuse_ab
     "idmap_stats": None,  # intra-tile repeats and probes per lookup on real mini-batches, see run_idmap_stats
-    "table_access": None,  # random loads and atomics into a hash-table-sized array, whole table vs one eighth per XCD
 }
 DESCRIPTIONS = {
     "c1": "R-MAT 100K nodes / ~2.5M edges, feat 128 fp32, batch 1024, fanout [15,10,5]",
@@ -97,20 +96,22 @@ DESCRIPTIONS = {
     "reuse_ab": "outermost block of c3 mini-batches (1.5 M gathered rows of 512 B, 1.0 M distinct, 57 GB table): one launch vs "
                 "two launches cut by a source-id threshold",
     "idmap_stats": "c3 mini-batches: ids repeated within a 2048-edge tile per hop; slots probed per lookup in the id-map's table",
-    "table_access": "1.5 M random 8-byte accesses (loads, compare-and-swaps, adds) into tables of 16-128 MB: anywhere, or each XCD "
-                    "inside its own eighth of the table",
     "c4": "aggregation microbench: 8192 dst x exactly 25 src out of 200K rows (int32 CSR), D in {64,128,256,602}, fp32 and bf16, "
           "sum and mean, forward and backward",
 }
 
 
-def run_c4(args):
+def run_c4(args, edge_weighted=True):
     """Aggregation-only microbench.  Forward = gather over the block, backward = gather over the
     transposed block; every case is 50 back-to-back launches between two HIP events ("cold" = the
-    same launches rotating over copies of the table that do not fit the Infinity Cache together)."""
+    same launches rotating over copies of the tables -- the gathered one and, for the backward pass, the written
+    one as well -- that do not fit the Infinity Cache together, so that the figures are HBM figures).  Returns the
+    record; `launch_floor_us` is a launch of the library that moves a few hundred bytes, timed the same way."""
     import torch
 
     import fastgl
+
+    last_mapping = lambda: fastgl.lib().fgl_aggregate_last_mapping().decode()
 
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
@@ -158,6 +159,14 @@ def run_c4(args):
         del graph
         return best  # us
 
+    # what a launch costs in this harness when there is next to nothing to move: one row of one entry
+    tiny_ptr = torch.tensor([0, 1], dtype=torch.int32, device=dev)
+    tiny_idx = torch.zeros(1, dtype=torch.int32, device=dev)
+    tiny_x = torch.zeros((1, 64), device=dev)
+    tiny_o = torch.empty((1, 64), device=dev)
+    launch_floor_us = timed(lambda: fastgl.aggregate(tiny_ptr, tiny_idx, tiny_x, mode="sum", zero_policy="zeros", out=tiny_o, longest_row=1))
+    log("launch floor (one row of one entry, same harness): %.2f us" % launch_floor_us)
+
     rows = []
     for dt, name, esz in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
         for D in (64, 128, 256, 602):
@@ -177,32 +186,47 @@ def run_c4(args):
                 turn[0] = (turn[0] + 1) % n_copies
                 fastgl.aggregate(ptr, idx, Xs[turn[0]], mode=mode, zero_policy="zeros", out=of, longest_row=k)
 
+            # cold backward: the gathered table (upstream gradients, 8192 rows) is small, the written one
+            # (200 K rows) is what would otherwise sit in the cache from one launch to the next: rotate both
+            dOs = [dO] + [dO.clone() for _ in range(n_copies - 1)]
+            obs = [ob] + [torch.empty_like(ob) for _ in range(n_copies - 1)]
+
+            def bwd_cold(bmode):
+                turn[0] = (turn[0] + 1) % n_copies
+                fastgl.aggregate(t_ptr, t_idx, dOs[turn[0]], mode=bmode, zero_policy="zeros", col_norm=deg, out=obs[turn[0]],
+                                 longest_row=t_longest)
+
             for mode, bmode in (("sum", "sum"), ("mean", "colmean")):
                 # longest_row: every row holds exactly k entries (a sampler knows its fanout the same way)
                 uf = timed(lambda: fastgl.aggregate(ptr, idx, X, mode=mode, zero_policy="zeros", out=of, longest_row=k))
+                kf = last_mapping()
                 uc = timed(lambda: fwd_cold(mode), reps=5 * n_copies)
+                ubc = timed(lambda: bwd_cold(bmode), reps=5 * n_copies)
                 ub = timed(lambda: fastgl.aggregate(t_ptr, t_idx, dO, mode=bmode, zero_policy="zeros", col_norm=deg, out=ob))
                 uk = timed(lambda: fastgl.aggregate(t_ptr, t_idx, dO, mode=bmode, zero_policy="zeros", col_norm=deg, out=ob,
                                                     longest_row=t_longest))
-                rows.append({"dtype": name, "D": D, "mode": mode, "fwd_us": uf, "fwd_GBps": bf / uf / 1e3,
+                kb = last_mapping()
+                rows.append({"dtype": name, "D": D, "mode": mode, "fwd_kernel": kf, "bwd_kernel": kb,
+                             "bwd_cold_us": ubc, "bwd_cold_GBps": bb / ubc / 1e3, "bwd_cold_frac_peak": bb / ubc / 1e3 / HBM_PEAK_GBPS,
+                             "fwd_us": uf, "fwd_GBps": bf / uf / 1e3,
                              "bwd_known_longest_us": uk, "bwd_known_longest_GBps": bb / uk / 1e3,
                              "bwd_known_longest_frac_peak": bb / uk / 1e3 / HBM_PEAK_GBPS,
                              "fwd_frac_peak": bf / uf / 1e3 / HBM_PEAK_GBPS, "fwd_cold_us": uc,
                              "fwd_cold_GBps": bf / uc / 1e3, "fwd_cold_frac_peak": bf / uc / 1e3 / HBM_PEAK_GBPS, "bwd_us": ub, "bwd_GBps": bb / ub / 1e3,
                              "bwd_frac_peak": bb / ub / 1e3 / HBM_PEAK_GBPS})
                 log("%-4s D=%-3d %-4s fwd %6.1f us %5.0f GB/s (%4.1f%%) | cold fwd %6.1f us %5.0f GB/s (%4.1f%%) | "
-                    "bwd %6.1f us %5.0f GB/s (%4.1f%%) | bwd, longest row (%d) known to the host %6.1f us (%4.1f%%)"
+                    "bwd %6.1f us %5.0f GB/s (%4.1f%%) | bwd, longest row (%d) known to the host %6.1f us (%4.1f%%) | cold %6.1f us (%4.1f%%)"
                     % (name, D, mode, uf, bf / uf / 1e3, bf / uf / 1e3 / HBM_PEAK_GBPS * 100, uc, bf / uc / 1e3,
                        bf / uc / 1e3 / HBM_PEAK_GBPS * 100, ub, bb / ub / 1e3, bb / ub / 1e3 / HBM_PEAK_GBPS * 100, t_longest, uk,
-                       bb / uk / 1e3 / HBM_PEAK_GBPS * 100))
-            del Xs
+                       bb / uk / 1e3 / HBM_PEAK_GBPS * 100, ubc, bb / ubc / 1e3 / HBM_PEAK_GBPS * 100))
+            del Xs, dOs, obs
     # attention-weighted aggregation (GAT): one float per (entry, head) on top of the row gather
     gat_rows = []
     n_heads = 4
     alpha = torch.rand((E, n_heads), generator=g).to(dev)
     t_ptr3, t_idx3, t_edge3 = fastgl.block_transpose(ptr, idx, n_dst, n_src, edge_ids=True)
     for dt, name, esz in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
-        for D in (128, 256):
+        for D in (128, 256) if edge_weighted else ():
             X = torch.randn(n_src, D, generator=g).to(dt).to(dev)
             dO = torch.randn(n_dst, D, generator=g).to(dt).to(dev)
             of = torch.empty((n_dst, D), dtype=dt, device=dev)
@@ -222,13 +246,41 @@ def run_c4(args):
                 % (name, D, n_heads, uf, bf / uf / 1e3, bf / uf / 1e3 / HBM_PEAK_GBPS * 100, us, bs / us / 1e3, ub, bb / ub / 1e3,
                    bb / ub / 1e3 / HBM_PEAK_GBPS * 100))
     head = [r for r in rows if r["dtype"] == "f32" and r["D"] == 128 and r["mode"] == "mean"][0]
-    print(json.dumps({
+    return {
         "metric": "aggregation HBM GB/s (% peak), 1 MI355X", "value": head["fwd_GBps"], "unit": "GB/s", "n_gpus": 1,
         "steps": 50, "warmup": 5, "ms_per_step": head["fwd_us"] / 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": DESCRIPTIONS["c4"]},
         "roofline": {"bound": "hbm", "achieved": head["fwd_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": head["fwd_frac_peak"], "traffic": None, "kernel": "aggregate_kernel (D=128 fp32 mean forward)"},
-        "cpu_baseline": None, "cases": rows, "edge_weighted_cases": gat_rows}), flush=True)
+        "cpu_baseline": None, "launch_floor_us": launch_floor_us, "transposed_longest_row": t_longest, "cases": rows,
+        "edge_weighted_cases": gat_rows}
+
+
+def c4_compact(rec):
+    """The microbench's record cut down to what rides on the default benchmark line: per case the time and
+    fraction of the HBM peak of the forward gather, the backward gather (longest transposed row known to the
+    host, as the sampler hands it over) and their cold-cache forms, with the kernel that ran; the worst
+    forward and the worst backward case named."""
+    cases = []
+    for r in rec["cases"]:
+        cases.append({"case": "%s D=%d %s" % (r["dtype"], r["D"], r["mode"]),
+                      "fwd_us": round(r["fwd_us"], 2), "fwd_frac": round(r["fwd_frac_peak"], 3),
+                      "fwd_cold_us": round(r["fwd_cold_us"], 2), "fwd_cold_frac": round(r["fwd_cold_frac_peak"], 3),
+                      "bwd_us": round(r["bwd_known_longest_us"], 2), "bwd_frac": round(r["bwd_known_longest_frac_peak"], 3),
+                      "bwd_cold_us": round(r["bwd_cold_us"], 2), "bwd_cold_frac": round(r["bwd_cold_frac_peak"], 3),
+                      "fwd_kernel": r["fwd_kernel"], "bwd_kernel": r["bwd_kernel"]})
+    worst = lambda key: min(cases, key=lambda c: c[key])
+    return {"workload": DESCRIPTIONS["c4"],
+            "timing": "50 launches replayed from a captured HIP graph between two HIP events, best of 3; frac = algorithmic bytes / time / 8 TB/s; "
+                      "warm = the same tables every launch (a 200K-row table of <= 481 MB partly stays in the 256 MB Infinity Cache; the backward "
+                      "pass gathers from an 8192-row table that always does, so its warm figures are not HBM figures); cold = rotating over "
+                      "copies that exceed the cache several times",
+            "launch_floor_us": round(rec["launch_floor_us"], 2), "transposed_longest_row": rec["transposed_longest_row"],
+            "worst_fwd": {k: worst("fwd_frac")[k] for k in ("case", "fwd_us", "fwd_frac", "fwd_kernel")},
+            "worst_fwd_cold": {k: worst("fwd_cold_frac")[k] for k in ("case", "fwd_cold_us", "fwd_cold_frac", "fwd_kernel")},
+            "worst_bwd": {k: worst("bwd_frac")[k] for k in ("case", "bwd_us", "bwd_frac", "bwd_kernel")},
+            "worst_bwd_cold": {k: worst("bwd_cold_frac")[k] for k in ("case", "bwd_cold_us", "bwd_cold_frac", "bwd_kernel")},
+            "cases": cases}
 
 
 
@@ -451,55 +503,6 @@ def run_idmap_stats(args):
                       "hops": hops, "probing": stats}), flush=True)
 
 
-def run_table_access(args):
-    """What the memory system gives the id-map's insert pass: 1.5 M random 8-byte accesses (the edges of an outermost hop)
-    into a table of the size the sampler uses, as loads, 64-bit compare-and-swaps, load-then-compare-and-swap and adds --
-    anywhere in the table, and with the workgroups that run on one XCD (every eighth workgroup) confined to one eighth
-    of the table, so that the XCD's L2 holds all that they touch.  Each figure is the best of five launches after a
-    refill of the table, timed with HIP events."""
-    import torch
-
-    import fastgl
-
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    n_ops = 1536 * 1024
-    hist = fastgl.probe_xcc_of_workgroups(6144, dev).cpu()
-    on_diagonal = int(hist.diagonal().sum())
-    log("workgroup index % 8 (rows) against the hardware XCC id (columns) for a launch of 6144 workgroups:")
-    for r in range(8):
-        log("   " + " ".join("%5d" % int(v) for v in hist[r, :8]))
-    rows = []
-    for log2_slots in (21, 22, 24):
-        table = torch.empty(1 << log2_slots, dtype=torch.int64, device=dev)
-        for op in fastgl.ops.PROBE_OPS:
-            rec = {"slots_log2": log2_slots, "table_MB": (8 << log2_slots) >> 20, "op": op}
-            for pattern in fastgl.ops.PROBE_PATTERNS:
-                best = None
-                for rep in range(5):
-                    table.fill_(-1)
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    fastgl.probe_table_access(table, n_ops, pattern, op, salt=rep)
-                    e1.record()
-                    e1.synchronize()
-                    us = e0.elapsed_time(e1) * 1e3
-                    best = us if best is None or us < best else best
-                rec[pattern + "_us"] = best
-                rec[pattern + "_Gps"] = n_ops / best / 1e3
-            rows.append(rec)
-            log("table %4d MB  %-20s whole table %6.1f us (%5.1f G/s) | own eighth per XCD %6.1f us (%5.1f G/s) | eighths not aligned %6.1f us"
-                % (rec["table_MB"], op, rec["whole_table_us"], rec["whole_table_Gps"], rec["eighth_of_own_xcd_us"],
-                   rec["eighth_of_own_xcd_Gps"], rec["eighth_not_aligned_us"]))
-        del table
-    cas = [r for r in rows if r["op"] == "cas" and r["slots_log2"] == 22][0]
-    print(json.dumps({"metric": "random 8-byte accesses into a 32 MB table: 64-bit compare-and-swaps per second", "value": cas["whole_table_Gps"] * 1e9,
-                      "unit": "atomics/s", "n_gpus": 1, "steps": 5, "warmup": 0, "ms_per_step": cas["whole_table_us"] / 1e3,
-                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u64", "data": "synthetic",
-                      "config": {"workload": DESCRIPTIONS["table_access"]}, "roofline": None, "cpu_baseline": None,
-                      "workgroups_on_the_xcd_of_their_index_mod_8": on_diagonal, "workgroups": 6144, "accesses": n_ops, "cases": rows}), flush=True)
-
-
 def time_dgl_cpu_path(h_ptr, h_src, train, B, fanouts, n_batches):
     """The reference's own CPU sampling path -- DGL's `sample_neighbors` + `to_block` per hop, as its
     DGLNeighborSampler drives them (FusedMapSampler.py:130-148) -- timed on the same mini-batches, if a DGL
@@ -529,6 +532,40 @@ def time_dgl_cpu_path(h_ptr, h_src, train, B, fanouts, n_batches):
                 "threads": torch.get_num_threads(), "sample": "%d mini-batches of %d seeds" % (n_batches, B)}
     except Exception as exc:
         return {"timed": False, "why": "dgl is importable but the run failed: %r" % (exc,)}
+
+
+def compare_with_oracle(O, np, g_inp, g_blocks, w_inp, w_blocks, exact_order=True):
+    """None if the sampler's output equals the oracle's, else a short description of the first difference."""
+    g_inp = g_inp.cpu().numpy()
+    if exact_order:
+        if not np.array_equal(g_inp, w_inp):
+            return "unique list differs (%d vs %d ids)" % (g_inp.size, w_inp.size)
+    elif not np.array_equal(np.sort(g_inp), np.sort(w_inp)):
+        return "unique ids differ as a set"
+    if len(g_blocks) != len(w_blocks):
+        return "block count"
+    for k, (b, w) in enumerate(zip(g_blocks, w_blocks)):
+        if (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()) != (w["n_src"], w["n_dst"], int(w["src_local"].size)):
+            return "block %d: sizes %s vs %s" % (k, (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()),
+                                                  (w["n_src"], w["n_dst"], int(w["src_local"].size)))
+        ptr_h, src_h = b.edge_ptr.cpu().numpy(), b.src_local.cpu().numpy()
+        if not np.array_equal(ptr_h, w["indptr"]):
+            return "block %d: row offsets" % k
+        if exact_order and not np.array_equal(src_h, w["src_local"]):
+            return "block %d: local ids" % k
+        if not exact_order and not np.array_equal(g_inp[src_h], w["src_global"]):
+            return "block %d: edges in graph ids" % k
+        if b.src_global is not None and not np.array_equal(b.src_global.cpu().numpy(), w["src_global"]):
+            return "block %d: graph ids" % k
+        if b._transposed is not None:
+            t_ptr, t_dst = (t.cpu().numpy() for t in b.transposed())
+            w_ptr, w_dst = O.transpose(ptr_h, src_h, b.num_src_nodes())
+            if not np.array_equal(t_ptr, w_ptr):
+                return "block %d: transposed row offsets" % k
+            row_of = np.repeat(np.arange(b.num_src_nodes(), dtype=np.int64), np.diff(w_ptr))
+            if not np.array_equal(np.sort(row_of * (b.num_dst_nodes() + 1) + t_dst), np.sort(row_of * (b.num_dst_nodes() + 1) + w_dst)):
+                return "block %d: transposed entries" % k
+    return None
 
 
 def log(*a):
@@ -569,6 +606,9 @@ def main():
     ap.add_argument("--other-forms", choices=["on", "off"], default="on",
                     help="also time sample_blocks() with its read-back (value_sample_blocks) and the reference's per-hop call "
                          "pattern through the compiled extension module (value_drop_in_api)")
+    ap.add_argument("--extras", choices=["on", "off"], default="on",
+                    help="workload c3 only: also run the aggregation microbench (key c4) and the very large shape (key c5) and "
+                         "attach their compact records to the line")
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
     ap.add_argument("--c4-eager", action="store_true",
@@ -595,16 +635,61 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload == "c4":
-        return run_c4(args)
+        print(json.dumps(run_c4(args)), flush=True)
+        return
     if args.workload == "ceiling":
         return run_ceiling(args)
     if args.workload == "reuse_ab":
         return run_reuse_ab(args)
     if args.workload == "idmap_stats":
         return run_idmap_stats(args)
-    if args.workload == "table_access":
-        return run_table_access(args)
-    w = WORKLOADS[args.workload]
+    out = run_graph_workload(args, args.workload)
+    if args.workload == "c3" and args.extras == "on":
+        # Two more configurations ride on the default line, each a compact object: the aggregation microbench
+        # (seconds) and, now that this workload's tensors are freed, the very large shape with bf16 features.
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            out["c4"] = c4_compact(run_c4(args, edge_weighted=False))
+        except Exception as exc:  # noqa: BLE001 -- context figures: reported, never fatal to the headline line
+            out["c4"] = {"error": repr(exc)}
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            out["c5"] = light_summary(run_graph_workload(args, "c5", light=True))
+        except Exception as exc:  # noqa: BLE001
+            out["c5"] = {"error": repr(exc)}
+    print(json.dumps(out), flush=True)
+    parity = out.get("parity_checked")
+    if parity is not None and not parity["ok"]:
+        print("bench.py: the timed mini-batches differ from the oracle's: %s" % parity.get("first_difference"), file=sys.stderr)
+        sys.exit(1)
+
+
+def light_summary(rec):
+    """A workload's record cut down to what rides on another workload's line."""
+    r = rec["roofline"]
+    return {"workload": rec["config"]["workload"], "value": rec["value"], "unit": rec["unit"], "dtype": rec["dtype"],
+            "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"], "stages_ms": rec["stages_ms"],
+            "sampled_edges_per_step": rec["config"]["sampled_edges_per_step"], "graph_edges": rec["config"]["graph_edges"],
+            "roofline": {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "kernel", "bytes_per_launch", "us_per_launch")},
+            "random_read_Gps": rec["random_read_Gps"]}
+
+
+def run_graph_workload(args, workload, light=False):
+    """One of the graph workloads (c1, c2, c3, c5, c5deep): builds the synthetic inputs on the device, times the steps and
+    returns the record.  light: the steps and the dominant kernel only (no other forms of the sampler, no CPU leg)."""
+    import numpy as np
+    import torch
+
+    import fastgl
+
+    dev = torch.device("cuda:0")
+    other_order_on = args.other_order == "on" and not light
+    other_forms_on = args.other_forms == "on" and not light
+    cpu_batches = 0 if light else args.cpu_batches
+    w = WORKLOADS[workload]
     N, D, H, B = w["nodes"], w["dim"], w["hidden"], w["batch"]
     fdtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16
     esz = 4 if fdtype == torch.float32 else 2
@@ -650,6 +735,7 @@ def main():
             log("graph-replay sampler abandoned: %s" % exc)
             sampler_mode = "eager (graph replay abandoned: %s)" % exc
             sampler = make_sampler(0)
+    main_sampler = sampler
     L = len(w["fanouts"])
     # hidden activations / upstream gradients of the inner layers: synthetic; sized from a probe
     # batch with head-room (the worst-case bound would be tens of GB for deep fanouts) and grown on demand
@@ -668,8 +754,12 @@ def main():
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
 
+    parity_keep = []  # (seed batch, random stream, outputs) of the first timed steps, compared with the oracle in the CPU leg
+    N_PARITY = 4
+
     def step(i, rec=None, sampler=sampler):
         seeds = train[(i % n_batches) * B:(i % n_batches) * B + B]
+        stream_base = (sampler.batches * 64) & 0xFFFFFFFF  # the Philox streams this mini-batch draws from
         e0, e1, e2, e3, e4 = ev(), ev(), ev(), ev(), ev()
         e0.record()
         if args.readback == "hidden":
@@ -699,13 +789,20 @@ def main():
         fastgl.transpose_blocks(blocks[1:])  # all inner blocks in the launches that one transpose takes
         for b in blocks[1:]:
             t_ptr, t_idx = b.transposed()
-            outs.append(fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",
-                                         col_norm=b.in_degrees().contiguous()))
+            outs.append(fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean_ptr", zero_policy="zeros",
+                                         col_norm=b.edge_ptr))
         e4.record()
         if rec is not None:
             rec.append(((sum(b.num_edges() for b in blocks), b0.num_edges(), b0.num_dst_nodes()), (e0, e1, e2, e3, e4)))
             keep.append(b0.clone() if sampler.graph_slots else b0)  # (a graph-replay slot is overwritten two batches on)
             del keep[:-4]  # a few outermost blocks are kept for the kernel-time replay below
+            if sampler is main_sampler and len(parity_keep) < N_PARITY and cpu_batches > 0:
+                # what this timed step produced, kept as it is (references, or copies where a replay slot would be
+                # overwritten) for the comparison with the oracle after the timing
+                if sampler.graph_slots:
+                    parity_keep.append((i % n_batches, stream_base, input_nodes.clone(), [b.clone() for b in blocks]))
+                else:
+                    parity_keep.append((i % n_batches, stream_base, input_nodes, blocks))
         return blocks
 
     for i in range(args.warmup):
@@ -722,7 +819,7 @@ def main():
     # ---- the same steps with the other numbering rule of the id-map (context for `value`) ----------------
     other_order = "arrival" if args.id_order == "first" else "first"
     value_other = None
-    if sampler_mode == "eager" and args.other_order == "on":
+    if sampler_mode == "eager" and other_order_on:
         keep_main = list(keep)
         alt = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=other_order).set_graph(edge_ptr, edge_src)
         for i in range(args.warmup):
@@ -761,7 +858,7 @@ def main():
         return edges / (ms * 1e-3), ms / args.steps
 
     value_sample_blocks = value_drop_in = None
-    if args.other_forms == "on":
+    if other_forms_on:
         plain = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
         value_sample_blocks, ms_sb = time_sampler(lambda seeds: sum(b.num_edges() for b in plain.sample_blocks(None, seeds)[2]))
         log("sample_blocks() with its read-back: %.3g sampled edges/s (%.3f ms per mini-batch)" % (value_sample_blocks, ms_sb))
@@ -793,7 +890,7 @@ def main():
 
     # ---- optional: the same steps with sampling of batch i+1 overlapped with aggregation of batch i ----
     ms_overlapped = None
-    if args.overlap:
+    if args.overlap and not light:
         def aggregate_only(blocks):
             b0 = blocks[0]
             fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
@@ -803,8 +900,8 @@ def main():
             fastgl.transpose_blocks(blocks[1:])
             for b in blocks[1:]:
                 t_ptr, t_idx = b.transposed()
-                fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean", zero_policy="zeros",
-                                 col_norm=b.in_degrees().contiguous())
+                fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean_ptr", zero_policy="zeros",
+                                 col_norm=b.edge_ptr)
         batches = [train[(i % n_batches) * B:(i % n_batches) * B + B] for i in range(args.warmup + args.steps)]
         torch.cuda.synchronize()
         for i, (_, _, blocks) in enumerate(sampler.iter_batches(batches)):
@@ -924,13 +1021,14 @@ def main():
 
     # ---- CPU baseline: the oracle on a bounded sample of the same workload ------------
     cpu = None
-    if args.cpu_batches > 0:
+    parity = None
+    if cpu_batches > 0:
         from oracle import oracle as O
         t0 = time.time()
         h_ptr, h_src = edge_ptr.cpu().numpy(), edge_src.cpu().numpy()
         log("graph copied to the host in %.1fs; oracle threads: %d" % (time.time() - t0, O.num_threads()))
         cpu_edges, cpu_t, cpu_t_seq, agg_t, agg_bytes = 0, 0.0, 0.0, 0.0, 0
-        for i in range(args.cpu_batches):
+        for i in range(cpu_batches):
             seeds = train[i * B:(i + 1) * B].cpu().numpy()
             t0 = time.perf_counter()
             inp, oblocks = O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, i * 64, parallel_idmap=True)
@@ -950,11 +1048,32 @@ def main():
                "sample": "%d mini-batches of %d seeds of the same workload through the CPU oracle "
                          "(OpenMP sampling + OpenMP id-map: CAS insert, first-occurrence numbering by prefix sum; "
                          "value_sequential_idmap = the same with a single-threaded hash-map id-map); "
-                         "aggregation = fp32 OpenMP row gather of the outermost block" % (args.cpu_batches, B),
+                         "aggregation = fp32 OpenMP row gather of the outermost block" % (cpu_batches, B),
                "value_sequential_idmap": cpu_edges / cpu_t_seq,
                "aggregation_GBps": agg_bytes / agg_t / 1e9, "host_cpus": os.cpu_count()}
         log("cpu baseline: %.3g edges/s (%d threads), aggregation %.1f GB/s" % (cpu["value"], cpu["cores"], cpu["aggregation_GBps"]))
-        cpu["dgl"] = time_dgl_cpu_path(h_ptr, h_src, train, B, w["fanouts"], min(args.cpu_batches, 16))
+        # ---- parity of the timed path: the first timed steps' own outputs against the oracle on the same seeds and
+        # random streams -- unique list, every block's offsets and local ids, the outermost block's graph ids, and the
+        # transposed inner blocks (offsets, and each row's entries as a set) -- bit for bit
+        t0 = time.time()
+        first_difference = None
+        for bi, sb, g_inp, g_blocks in parity_keep:
+            seeds = train[bi * B:(bi + 1) * B].cpu().numpy()
+            w_inp, w_blocks = O.sample_blocks(h_ptr, h_src, seeds, w["fanouts"], 0, sb)
+            first_difference = compare_with_oracle(O, np, g_inp, g_blocks, w_inp, w_blocks, exact_order=args.id_order == "first")
+            if first_difference is not None:
+                first_difference = "seed batch %d, stream %d: %s" % (bi, sb, first_difference)
+                break
+        parity = {"batches": len(parity_keep), "ok": first_difference is None,
+                  "what": "the first timed steps' outputs (the steady-state path: learned buffer sizes, small table, no fill, "
+                          "begin_sample/finish) vs the CPU oracle on the same seeds and Philox streams: unique list, block offsets, "
+                          "local ids, outermost graph ids, transposed inner blocks; bit-exact"
+                          + ("" if args.id_order == "first" else " after sorting the new ids (arrival order)")}
+        if first_difference is not None:
+            parity["first_difference"] = first_difference
+        log("parity of %d timed mini-batches against the oracle: %s (%.1fs)"
+            % (len(parity_keep), "ok" if first_difference is None else "MISMATCH " + first_difference, time.time() - t0))
+        cpu["dgl"] = time_dgl_cpu_path(h_ptr, h_src, train, B, w["fanouts"], min(cpu_batches, 16))
 
     out = {
         "metric": "sampled edges/s (sample+id_map) + aggregation HBM GB/s (% peak), 1 MI355X",
@@ -970,7 +1089,7 @@ def main():
         "vs_baseline": None,
         "dtype": w["dtype"],
         "data": "synthetic",
-        "config": {"workload": DESCRIPTIONS[args.workload], "graph_edges": n_graph_edges,
+        "config": {"workload": DESCRIPTIONS[workload], "graph_edges": n_graph_edges,
                    "sampled_edges_per_step": tot_edges / K,
                    "note": "seeds are drawn uniformly from an R-MAT graph without degree noise, so most of them have degree 0-1 "
                            "(the first hop expands 8192 seeds to ~10 K edges): a mini-batch samples ~1.6 M edges, not the "
@@ -993,15 +1112,20 @@ def main():
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
-                     "traffic": traffic_from_profile(args.workload, bytes_agg0 / K),
-                     "achieved_is": "algorithmic bytes (every sampled edge counted as one row fetch) / kernel time; "
+                     "traffic": traffic_from_profile(workload, bytes_agg0 / K),
+                     "achieved_is": "an effective rate: algorithmic bytes (every sampled edge counted as one row fetch) / kernel time; "
+                                    "frac_of_peak_by_traffic = the counter-derived bytes / the same time / peak; "
                                     "traffic = bytes per launch that the L2s fetch and write (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled): "
                                     "repeated rows that hit in L2 are not in it, hits in the memory-side Infinity Cache still are",
                      "kernel": "aggregate_kernel<float,4,32,MEAN> (outermost block, forward)",
                      "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_kernel0 / K * 1e3},
         "cpu_baseline": cpu,
+        "parity_checked": parity,
     }
-    print(json.dumps(out), flush=True)
+    r = out["roofline"]
+    # the same launch priced by what the counters saw move instead of by the algorithmic bytes
+    r["frac_of_peak_by_traffic"] = None if r["traffic"] is None else r["traffic"] / (r["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBPS
+    return out
 
 
 if __name__ == "__main__":

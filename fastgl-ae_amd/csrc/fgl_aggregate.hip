@@ -143,15 +143,17 @@ struct AggArgs {
     int skip_rows_longer_than;  // aggregate_kernel leaves rows with more entries to aggregate_long_rows_kernel
     int n_heads;
     int unit_dim;               // D / n_heads
+    int col_norm_is_ptr;        // FGL_AGG_COLMEAN: col_norm is an offsets array, the counts are its differences
 };
 
 // per-edge weight, evaluated by the lane that loaded the neighbour id
 template <int MODE>
-__device__ __forceinline__ float edge_weight(int col, float row_factor, const int32_t* __restrict__ col_norm)
+__device__ __forceinline__ float edge_weight(int col, float row_factor, const int32_t* __restrict__ col_norm, int col_norm_is_ptr)
 {
     if (MODE == FGL_AGG_GCN) return row_factor * (1.0f / sqrtf((float)col_norm[col]));
     if (MODE == FGL_AGG_COLMEAN) {
-        const int c = col_norm[col];
+        // (the columns' entry counts, or the offsets array they are the differences of)
+        const int c = col_norm_is_ptr ? col_norm[col + 1] - col_norm[col] : col_norm[col];
         return 1.0f / (float)(c > 1 ? c : 1);
     }
     return row_factor;  // SUM: 1, MEAN: 1/deg(row)
@@ -232,7 +234,7 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
         float my_w = 0.0f;
         if (gl < cnt) {
             my_col = indices[base + gl];
-            my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+            my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm, g.col_norm_is_ptr);
         }
         // four row loads are issued before the first FMA; the tail of the list goes one by one
         // (measured: longer or predicated unrolls gain nothing on long lists and lose up to 2x
@@ -462,7 +464,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_split_kernel(const AggArgs g
             float my_w = 0.0f;
             if (q < cnt) {
                 my_col = indices[base + q];
-                my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm, g.col_norm_is_ptr);
             }
             float sum[VEC];  // this chunk's share of the row (two-level summation, as in gather_row)
 #pragma unroll
@@ -576,7 +578,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_bundle_kernel(const AggArgs 
                 float row_factor = 1.0f;
                 if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(end_j - begin_j);
                 if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[r0 + j]);
-                if (MODE != FGL_AGG_EDGE) my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                if (MODE != FGL_AGG_EDGE) my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm, g.col_norm_is_ptr);
                 my_tag = j | (e + 1 == end_j ? 256 : 0);
             }
             for (int t = 0; t < cnt; t += 4) {
@@ -701,8 +703,8 @@ __global__ __launch_bounds__(kBlock) void aggregate_flat_kernel(const AggArgs g,
             int e = base;
             for (; e + 4 <= end; e += 4) {
                 const int c0 = indices[e], c1 = indices[e + 1], c2 = indices[e + 2], c3 = indices[e + 3];
-                const float w0 = edge_weight<MODE>(c0, row_factor, g.col_norm), w1 = edge_weight<MODE>(c1, row_factor, g.col_norm);
-                const float w2 = edge_weight<MODE>(c2, row_factor, g.col_norm), w3 = edge_weight<MODE>(c3, row_factor, g.col_norm);
+                const float w0 = edge_weight<MODE>(c0, row_factor, g.col_norm, g.col_norm_is_ptr), w1 = edge_weight<MODE>(c1, row_factor, g.col_norm, g.col_norm_is_ptr);
+                const float w2 = edge_weight<MODE>(c2, row_factor, g.col_norm, g.col_norm_is_ptr), w3 = edge_weight<MODE>(c3, row_factor, g.col_norm, g.col_norm_is_ptr);
                 const typename IO::Raw r0 = load(X + (int64_t)c0 * ldx + col0);
                 const typename IO::Raw r1 = load(X + (int64_t)c1 * ldx + col0);
                 const typename IO::Raw r2 = load(X + (int64_t)c2 * ldx + col0);
@@ -717,9 +719,9 @@ __global__ __launch_bounds__(kBlock) void aggregate_flat_kernel(const AggArgs g,
                 const int c0 = indices[e];
                 const int c1 = indices[rem > 1 ? e + 1 : e];
                 const int c2 = indices[rem > 2 ? e + 2 : e];
-                const float w0 = edge_weight<MODE>(c0, row_factor, g.col_norm);
-                const float w1 = edge_weight<MODE>(c1, row_factor, g.col_norm);
-                const float w2 = edge_weight<MODE>(c2, row_factor, g.col_norm);
+                const float w0 = edge_weight<MODE>(c0, row_factor, g.col_norm, g.col_norm_is_ptr);
+                const float w1 = edge_weight<MODE>(c1, row_factor, g.col_norm, g.col_norm_is_ptr);
+                const float w2 = edge_weight<MODE>(c2, row_factor, g.col_norm, g.col_norm_is_ptr);
                 const typename IO::Raw r0 = load(X + (int64_t)c0 * ldx + col0);
                 typename IO::Raw r1 = r0, r2 = r0;
                 if (rem > 1) r1 = load(X + (int64_t)c1 * ldx + col0);
@@ -802,7 +804,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_flat_bundle_kernel(const Agg
                 float row_factor = 1.0f;
                 if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(end_j - begin_j);
                 if (MODE == FGL_AGG_GCN && cb + j < total) row_factor = 1.0f / sqrtf((float)g.row_norm[r0 + row_j]);
-                w[j] = cb + j < total ? edge_weight<MODE>(c[j], row_factor, g.col_norm) : 0.0f;
+                w[j] = cb + j < total ? edge_weight<MODE>(c[j], row_factor, g.col_norm, g.col_norm_is_ptr) : 0.0f;
                 tag[j] = row_j | (e + 1 == end_j ? 256 : 0);
             }
 #pragma unroll
@@ -850,7 +852,7 @@ __global__ __launch_bounds__(kBlock) void aggregate_flat_bundle_kernel(const Agg
                 for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
                 for (int e = base; e < end; ++e) {
                     const int c0 = indices[e];
-                    IO::fma(part, edge_weight<MODE>(c0, row_factor, g.col_norm), load(X + (int64_t)c0 * ldx + col0));
+                    IO::fma(part, edge_weight<MODE>(c0, row_factor, g.col_norm, g.col_norm_is_ptr), load(X + (int64_t)c0 * ldx + col0));
                 }
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) acc[i] += part[i];
@@ -923,7 +925,7 @@ __global__ __launch_bounds__(kLongBlock) void aggregate_long_rows_kernel(const A
                 if (gl < cnt) {
                     my_col = indices[base + gl];
                     if (MODE == FGL_AGG_EDGE) my_eid = g.edge_index ? g.edge_index[base + gl] : (int)(base + gl);
-                    else my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm);
+                    else my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm, g.col_norm_is_ptr);
                 }
                 float part[VEC];  // two-level summation, as in gather_row
 #pragma unroll
@@ -1096,6 +1098,14 @@ size_t transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int so
 }
 
 // ---- dispatch ----------------------------------------------------------------------
+// Which lane mapping the calling thread's last fgl_aggregate call chose (for benchmarks and bug reports).
+static thread_local char g_mapping[96] = "";
+static void note_mapping(const char* kernel, int lpr, int extra, bool second_pass)
+{
+    snprintf(g_mapping, sizeof(g_mapping), "%s lanes/row=%d%s%s", kernel, lpr,
+             extra > 1 ? (extra >= 100 ? " (rows bundled by 4)" : " (groups/row>1)") : "", second_pass ? " + long_rows" : "");
+}
+
 // Workgroups of the long-row pass: each looks through an equal share of the row offsets.
 constexpr int kLongRowBlocks = 1021;  // a prime: rows are dealt round robin, and ids that agree in their low bits are
                                        // alike in synthetic (R-MAT) graphs -- a power of two would hand all hubs to a few workgroups
@@ -1105,6 +1115,7 @@ static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStre
 {
     const bool second_pass = long_rows_possible;
     g.skip_rows_longer_than = second_pass ? kLongRowEntries : 0x7FFFFFFF;
+    note_mapping("aggregate_kernel", LPR, 1, second_pass);
 #define FGL_LAUNCH_MODE(M)                                                                                         \
     do {                                                                                                           \
         hipLaunchKernelGGL((aggregate_kernel<T, VEC, LPR, M>), grid, dim3(kBlock), 0, stream, g);                  \
@@ -1132,6 +1143,7 @@ template <typename T, int VEC>
 static int launch_agg_flat(int mode, bool long_rows_possible, int lanes, bool bundle, hipStream_t stream, AggArgs g)
 {
     g.skip_rows_longer_than = long_rows_possible ? kLongRowEntries : 0x7FFFFFFF;
+    note_mapping(bundle ? "aggregate_flat_bundle_kernel" : "aggregate_flat_kernel", lanes, bundle ? 100 : 1, long_rows_possible);
     const int64_t blocks = ceil_div((bundle ? ceil_div(g.n_rows_max, kBundleRows) : g.n_rows_max) * lanes, kBlock);
     if (blocks > 0x7FFFFFFF) {
         set_error("aggregate: grid too large (%lld workgroups)", (long long)blocks);
@@ -1184,6 +1196,7 @@ template <typename T, int VEC, int LPR, int S>
 static int launch_agg_split(int mode, unsigned gy, hipStream_t stream, AggArgs g)
 {
     g.skip_rows_longer_than = 0x7FFFFFFF;
+    note_mapping("aggregate_split_kernel", LPR, S, false);
     const int64_t gx = ceil_div(g.n_rows_max, kBlock / (S * LPR));
 #define FGL_LAUNCH_SPLIT(M) \
     hipLaunchKernelGGL((aggregate_split_kernel<T, VEC, LPR, S, M>), dim3((unsigned)gx, gy), dim3(kBlock), 0, stream, g)
@@ -1197,6 +1210,7 @@ template <typename T, int VEC, int LPR>
 static int launch_agg_bundle(int mode, bool long_rows_possible, unsigned gy, hipStream_t stream, AggArgs g)
 {
     g.skip_rows_longer_than = long_rows_possible ? kLongRowEntries : 0x7FFFFFFF;
+    note_mapping("aggregate_bundle_kernel", LPR, 100, long_rows_possible);
     const int64_t gx = ceil_div(ceil_div(g.n_rows_max, kBundleRows), kBlock / LPR);
 #define FGL_LAUNCH_BUNDLE(M)                                                                                          \
     do {                                                                                                              \
@@ -1307,7 +1321,9 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     FGL_REQUIRE(D >= 1, "aggregate: feature length %d < 1", D);
     FGL_REQUIRE(ldx >= D && ldo >= D, "aggregate: row stride smaller than the row length");
     FGL_REQUIRE(dtype == FGL_F32 || dtype == FGL_BF16, "aggregate: unknown dtype %d", dtype);
-    FGL_REQUIRE(mode >= FGL_AGG_SUM && mode <= FGL_AGG_EDGE, "aggregate: unknown mode %d", mode);
+    FGL_REQUIRE(mode >= FGL_AGG_SUM && mode <= FGL_AGG_COLMEAN_PTR, "aggregate: unknown mode %d", mode);
+    const int col_norm_is_ptr = mode == FGL_AGG_COLMEAN_PTR;
+    if (col_norm_is_ptr) mode = FGL_AGG_COLMEAN;
     FGL_REQUIRE(zero_policy == FGL_ZERO_COPY_SELF || zero_policy == FGL_ZERO_ZEROS, "aggregate: unknown zero policy %d", zero_policy);
     FGL_REQUIRE(mode != FGL_AGG_GCN || (d_row_norm && d_col_norm), "aggregate: gcn mode needs row_norm and col_norm");
     FGL_REQUIRE(mode != FGL_AGG_COLMEAN || d_col_norm, "aggregate: colmean mode needs col_norm");
@@ -1320,12 +1336,14 @@ FGL_EXPORT int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices, 
     g.indptr = d_indptr; g.indices = d_indices; g.n_rows_max = n_rows_max; g.d_n_rows = d_n_rows;
     g.x = d_x; g.ldx = ldx; g.D = D; g.zero_policy = zero_policy; g.row_norm = d_row_norm; g.col_norm = d_col_norm;
     g.out = d_out; g.ldo = ldo; g.edge_w = d_edge_w; g.edge_index = d_edge_index; g.longest_row = d_longest_row;
-    g.n_heads = n_heads > 0 ? n_heads : 1; g.unit_dim = D / g.n_heads;
+    g.n_heads = n_heads > 0 ? n_heads : 1; g.unit_dim = D / g.n_heads; g.col_norm_is_ptr = col_norm_is_ptr;
     hipStream_t s = as_stream(stream);
     if (dtype == FGL_F32) return launch_agg_vec<float, 4>(mode, longest_row_max, n_entries_max, s, g);
     if (bf16_rows_dword_aligned(ldx, ldo, d_x, d_out)) return launch_agg_vec<uint16_t, 8>(mode, longest_row_max, n_entries_max, s, g);
     return launch_agg_vec<uint16_t, 1>(mode, longest_row_max, n_entries_max, s, g);
 }
+
+FGL_EXPORT const char* fgl_aggregate_last_mapping(void) { return g_mapping; }
 
 FGL_EXPORT size_t fgl_block_transpose_workspace_bytes(int64_t n_cols_max, int64_t n_edges_max, int sorted)
 {

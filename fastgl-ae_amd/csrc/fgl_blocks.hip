@@ -9,6 +9,7 @@
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 #include "fgl_table.hpp"
+#include "fgl_transpose_job.hpp"
 
 namespace fgl {
 
@@ -31,7 +32,7 @@ __global__ __launch_bounds__(TS) void blocks_prepare_kernel(TableRef t, const vo
     __shared__ int smem[TS / kWave + 1];
     const int64_t first = (int64_t)blockIdx.x * TS + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * TS;
-    if (first < n_counts) counts[first] = (first == 0) ? (int32_t)n_seeds : 0;
+    for (int64_t i = first; i < n_counts; i += stride) counts[i] = (i == 0) ? (int32_t)n_seeds : 0;
     for (int64_t i = first; i < n_later_sums; i += stride) later_sums[i] = 0;
     const int64_t n_tiles = (n_seeds + TS - 1) / TS;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -85,6 +86,10 @@ struct BlocksPlan {
     int64_t max_tiles;
     int64_t max_edges;
     size_t idmap_bytes;
+    // transposed blocks built inside the call (bit h of transpose_hops: hop h's)
+    uint32_t transpose_hops;
+    int64_t cap_src[32];  // max source nodes (= columns) of hop h
+    int split[32];        // counters per column while hop h's transposed rows are being counted
 };
 
 struct BlocksScratch {
@@ -94,6 +99,10 @@ struct BlocksScratch {
     int32_t* tile_prefix;
     uint8_t* lowered;  // one byte per edge of a hop: cleared by the hop's sampling kernel, used by its id-map passes
     char* idmap_ws;
+    // per hop whose transposed block is wanted (null otherwise)
+    int32_t* t_rank[32];
+    int32_t* t_tile_sums[32];
+    int32_t* t_split_cnt[32];  // split counters (hops that count with several counters per column)
 };
 
 static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
@@ -105,14 +114,39 @@ static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
     int32_t* tile_prefix = c.take<int32_t>((size_t)p.max_tiles);
     uint8_t* lowered = c.take<uint8_t>((size_t)p.max_edges);
     char* idmap_ws = c.take<char>(p.idmap_bytes);
-    if (out) *out = BlocksScratch{row_start, deg, tile_sums, tile_prefix, lowered, idmap_ws};
+    if (out) {
+        memset(out, 0, sizeof(*out));
+        out->row_start = row_start;
+        out->deg = deg;
+        out->tile_sums = tile_sums;
+        out->tile_prefix = tile_prefix;
+        out->lowered = lowered;
+        out->idmap_ws = idmap_ws;
+    }
+    for (int h = 0; h < 32; ++h) {
+        if (!((p.transpose_hops >> h) & 1u)) continue;
+        const int64_t counters = p.cap_src[h] * p.split[h] + 1;
+        int32_t* rank = c.take<int32_t>((size_t)p.cap_edges[h]);
+        int32_t* sums = c.take<int32_t>((size_t)ceil_div(counters, kTjobTile));
+        int32_t* cnt = p.split[h] > 1 ? c.take<int32_t>((size_t)counters) : nullptr;
+        if (out) {
+            out->t_rank[h] = rank;
+            out->t_tile_sums[h] = sums;
+            out->t_split_cnt[h] = cnt;
+        }
+    }
     return c.used();
 }
 
 // node_capacity (optional, n_hops+1 entries): the caller's own limit on the number of nodes before
 // hop h (entry n_hops: after the last hop).  The plan is the worst case clipped to it.
+// Hops of at least this many edges (by the plan's bound) count their transposed rows with kTransposeSplit
+// counters per column: a hub column of such a hop is mentioned thousands of times.
+constexpr int64_t kTransposeSplitMinEdges = (int64_t)1 << 20;
+constexpr int kTransposeSplit = 8;
+
 static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops, const int64_t* node_capacity,
-                     BlocksPlan* p)
+                     uint32_t transpose_hops, BlocksPlan* p)
 {
     FGL_REQUIRE(n_hops >= 1 && n_hops <= 32, "sample_blocks: %d hops outside [1, 32]", n_hops);
     FGL_REQUIRE(n_nodes >= 0 && n_seeds >= 0 && fanouts != nullptr, "sample_blocks: bad sizes");
@@ -148,6 +182,14 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
         if (cur > node_capacity[n_hops]) cur = node_capacity[n_hops];
     }
     p->cap_uniq = cur;
+    FGL_REQUIRE(n_hops == 32 || (transpose_hops >> n_hops) == 0, "sample_blocks: transpose_hops names a hop beyond the %d of the call", n_hops);
+    p->transpose_hops = transpose_hops;
+    for (int h = 0; h < 32; ++h) {
+        p->cap_src[h] = h < n_hops ? (h + 1 < n_hops ? p->cap_dst[h + 1] : cur) : 0;
+        p->split[h] = (h < n_hops && p->cap_edges[h] >= kTransposeSplitMinEdges) ? kTransposeSplit : 1;
+        if (h < n_hops && ((transpose_hops >> h) & 1u))
+            FGL_REQUIRE(p->cap_src[h] * p->split[h] + 1 <= 0x7FFFFFFF, "sample_blocks: hop %d has too many columns to transpose", h);
+    }
     p->table_slots = fgl_idmap_slots(cur);
     FGL_REQUIRE(p->table_slots <= ((int64_t)1 << 31), "sample_blocks: table too large");
     p->n_positions = p->cap_dst[n_hops - 1] > 0 ? p->cap_dst[n_hops - 1] : 1;
@@ -156,6 +198,16 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
     p->idmap_bytes = idmap_ws;
     p->ws_bytes = carve_scratch(*p, nullptr, nullptr);
     return FGL_OK;
+}
+
+// The three closing steps of a transposed block as launches of their own: for the last hop of a call, which has no
+// later hop whose launches could carry them.
+template <int STEP>
+__global__ __launch_bounds__(kBlock) void transpose_step_kernel(const TransposeJob j)
+{
+    if (STEP == 0) tjob_tile_sums<kBlock>(j);
+    if (STEP == 1) tjob_scan<kBlock>(j);
+    if (STEP == 2) tjob_fill<kBlock>(j);
 }
 
 // ---- R-MAT -------------------------------------------------------------------------
@@ -193,11 +245,11 @@ __global__ __launch_bounds__(kBlock) void rmat_keys_kernel(int64_t first_edge, i
 using namespace fgl;
 
 FGL_EXPORT int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                                      const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges,
-                                      int64_t* cap_uniq, int64_t* table_slots, size_t* ws_bytes)
+                                      const int64_t* node_capacity, uint32_t transpose_hops, int64_t* cap_dst,
+                                      int64_t* cap_edges, int64_t* cap_uniq, int64_t* table_slots, size_t* ws_bytes)
 {
     BlocksPlan p;
-    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, transpose_hops, &p);
     if (rc != FGL_OK) return rc;
     for (int h = 0; h < n_hops; ++h) {
         if (cap_dst) cap_dst[h] = p.cap_dst[h];
@@ -215,12 +267,21 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
                                  const uint32_t* d_stream_offset, int idmap_flags, void* d_table,
                                  int64_t table_slots,
                                  int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
-                                 int32_t* const* src_local, int32_t* const* src_global, int32_t* d_counts, void* d_ws,
+                                 int32_t* const* src_local, int32_t* const* src_global, int32_t* const* t_ptr,
+                                 int32_t* const* t_dst, int32_t* const* t_edge, int32_t* d_counts, void* d_ws,
                                  size_t ws_bytes, void* stream)
 {
+    // the hops whose transposed block is wanted: those with a row-pointer output
+    uint32_t transpose_hops = 0;
+    if (t_ptr != nullptr && n_hops >= 1 && n_hops <= 32)
+        for (int h = 0; h < n_hops; ++h)
+            if (t_ptr[h] != nullptr) transpose_hops |= 1u << h;
     BlocksPlan p;
-    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, &p);
+    int rc = make_plan(n_nodes, n_seeds, fanouts, n_hops, node_capacity, transpose_hops, &p);
     if (rc != FGL_OK) return rc;
+    for (int h = 0; h < n_hops; ++h)
+        if ((transpose_hops >> h) & 1u)
+            FGL_REQUIRE(t_dst != nullptr && t_dst[h] != nullptr, "sample_blocks: hop %d has a transposed row pointer but no entry array", h);
     const int order = idmap_flags & FGL_IDMAP_ARRIVAL;
     const bool table_is_empty = (idmap_flags & FGL_BLOCKS_TABLE_EMPTY) != 0;
     const bool leave_empty = (idmap_flags & FGL_BLOCKS_LEAVE_TABLE_EMPTY) != 0;
@@ -240,7 +301,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     for (int h = 0; h < n_hops; ++h) FGL_REQUIRE(block_ptr[h] && src_local[h], "sample_blocks: null output for hop %d", h);
 
     hipStream_t s = as_stream(stream);
-    const int n_counts = 2 * n_hops + 2;
+    const int n_counts = 3 * n_hops + 2;
     uint32_t* d_status = reinterpret_cast<uint32_t*>(d_counts + 2 * n_hops + 1);
     FGL_REQUIRE(valid_slots(table_slots), "sample_blocks: slot count %lld is not a power of two in [64, 2^31]", (long long)table_slots);
     FGL_REQUIRE(((uintptr_t)d_table & 15) == 0 && ((uintptr_t)d_ws & 15) == 0, "sample_blocks: table and workspace must be 16-byte aligned");
@@ -273,6 +334,30 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         FGL_CHECK_LAUNCH("blocks_prepare_kernel");
     }
 
+    auto make_job = [&](int h) {
+        TransposeJob j;
+        memset(&j, 0, sizeof(j));
+        if (!((transpose_hops >> h) & 1u)) return j;
+        j.split = p.split[h];
+        j.cnt = j.split > 1 ? ws.t_split_cnt[h] : t_ptr[h];
+        j.tile_sums = ws.t_tile_sums[h];
+        j.rank = ws.t_rank[h];
+        j.t_ptr = t_ptr[h];
+        j.t_dst = t_dst[h];
+        j.t_edge = t_edge ? t_edge[h] : nullptr;
+        j.longest = d_counts + 2 * n_hops + 2 + h;
+        j.block_ptr = block_ptr[h];
+        j.src_local = src_local[h];
+        j.d_n_rows = d_counts + h;
+        j.d_n_cols = d_counts + h + 1;
+        j.d_n_edges = d_counts + n_hops + 1 + h;
+        j.rows_max = p.cap_dst[h];
+        j.cols_max = p.cap_src[h];
+        j.edges_max = p.cap_edges[h];
+        return j;
+    };
+    TransposeJob job_before;
+    memset(&job_before, 0, sizeof(job_before));
     for (int h = 0; h < n_hops; ++h) {
         const bool last = h == n_hops - 1;
         const int32_t* hop_seeds = (h == 0) ? d_seeds : d_uniq;
@@ -293,10 +378,15 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
             next.fanout = fanouts[h + 1];
             next.tile_seeds = sample_tile_seeds(fanouts[h + 1], p.cap_dst[h + 1]);
         }
+        // transposed blocks: this hop's (if wanted) has its counters cleared by the sampling launch and its ranks
+        // taken by the id-map passes; the one of the hop before is closed by this hop's first three launches
+        TransposeSteps steps;
+        steps.before = job_before;
+        steps.zero = make_job(h);
         rc = launch_sample_edges(d_indices, hop_seeds, p.cap_dst[h], d_n_dst, fanouts[h], ws.row_start, ws.deg,
                                  ws.tile_sums + p.tile_first[h], ws.tile_prefix, rng_seed, stream_base + (uint32_t)h, sampled,
                                  nullptr, block_ptr[h], d_n_edges, d_status, s, d_stream_offset, last ? nullptr : &next,
-                                 ws.lowered);
+                                 ws.lowered, &steps);
         if (rc != FGL_OK) return rc;
         // the node count this hop may grow to: what the next hop's buffers (or the unique list) hold;
         // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped
@@ -304,8 +394,18 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
                                   d_counts + h + 1, d_uniq, grow_to, order | (last ? FGL_IDMAP_FINAL : 0), d_status,
                                   ws.idmap_ws, p.idmap_bytes, s, /*counter_is_zeroed=*/true, last ? nullptr : &next,
-                                  /*leave_table_empty=*/last && leave_empty, ws.lowered);
+                                  /*leave_table_empty=*/last && leave_empty, ws.lowered, &steps.zero, &job_before);
         if (rc != FGL_OK) return rc;
+        job_before = steps.zero;
+    }
+    if (job_before.cnt != nullptr) {  // the last hop's transposed block: no later launch to carry its closing steps
+        job_before.side_first = 0;
+        job_before.side_blocks = side_blocks_for(job_before.cols_max * job_before.split + 1, kTjobTile, 8192);
+        hipLaunchKernelGGL(transpose_step_kernel<0>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
+        hipLaunchKernelGGL(transpose_step_kernel<1>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
+        job_before.side_blocks = side_blocks_for(job_before.rows_max, kBlock / 16, 8192);
+        hipLaunchKernelGGL(transpose_step_kernel<2>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
+        FGL_CHECK_LAUNCH("transpose_step_kernel");
     }
     return FGL_OK;
 }

@@ -30,6 +30,7 @@
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 #include "fgl_table.hpp"
+#include "fgl_transpose_job.hpp"
 
 namespace fgl {
 
@@ -105,8 +106,10 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
                                                                   int64_t e_max, const int32_t* __restrict__ d_e,
                                                                   uint32_t* __restrict__ slot_of, int32_t* out,
                                                                   uint8_t* __restrict__ lowered,
-                                                                  uint32_t* __restrict__ d_status)
+                                                                  uint32_t* __restrict__ d_status, const TransposeRank tr,
+                                                                  const TransposeJob before)
 {
+    tjob_scan<kBlock>(before);  // (the hop before, if its transposed block is being built: counters -> offsets)
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
@@ -123,6 +126,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
             // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
             // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
             out[e] = (int32_t)seen;
+            take_rank(tr, e, (int32_t)seen);
             p = kDone;
         } else if (lowered != nullptr) {
             if (holder) p |= kHolderBit;
@@ -143,9 +147,10 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
                                                             const uint8_t* __restrict__ lowered,
                                                             uint32_t* __restrict__ first_of,
                                                             uint8_t* __restrict__ flags8, uint16_t* __restrict__ before8,
-                                                            int32_t* __restrict__ tile_sums)
+                                                            int32_t* __restrict__ tile_sums, const TransposeJob before)
 {
     __shared__ int smem[kBlock / kWave + 1];
+    tjob_fill<kBlock>(before);  // (the hop before, if its transposed block is being built: entries into their rows)
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t n_tiles = tiles_of(n_e);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -331,7 +336,8 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                                                               int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
                                                               int32_t* __restrict__ d_n_total_out,
                                                               uint32_t* __restrict__ d_status, const NextHop next,
-                                                              uint32_t* __restrict__ clear_words, int64_t n_clear_words)
+                                                              uint32_t* __restrict__ clear_words, int64_t n_clear_words,
+                                                              const TransposeRank tr)
 {
     __shared__ int s_prefix[SELF ? kIdmapSelfPrefixTiles : 1];
     __shared__ int smem[kBlock / kWave + 1];
@@ -410,6 +416,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                 }
             }
             out[e] = (int32_t)local;
+            take_rank(tr, e, (int32_t)local);
         }
         if (next.row_start != nullptr) add_next_tile_sums(next, next_k, next_tile);
     }
@@ -446,10 +453,12 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                                                                       int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                       uint32_t* __restrict__ slot_of, int32_t* __restrict__ counter,
                                                                       int32_t* __restrict__ uniq, int64_t capacity, int32_t* out,
-                                                                      uint32_t* __restrict__ d_status, const NextHop next)
+                                                                      uint32_t* __restrict__ d_status, const NextHop next,
+                                                                      const TransposeRank tr, const TransposeJob before)
 {
     __shared__ int smem[kBlock / kWave + 1];
     __shared__ int s_base;
+    tjob_scan<kBlock>(before);  // (the hop before, if its transposed block is being built: counters -> offsets)
     constexpr int kNextTiles = kBlock * ITEMS / kWave + 2;  // next-hop tiles (64 seeds or more each) that a tile's new nodes can touch
     __shared__ int s_next[kNextTiles];
     unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
@@ -496,6 +505,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                             p[j] = q;
                         } else {
                             out[e] = (int32_t)v;
+                            take_rank(tr, e, (int32_t)v);
                             p[j] = kDone;
                         }
                         break;
@@ -504,6 +514,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                 }
                 if (p[j] == kEmpty) {
                     out[e] = -1;
+                    take_rank(tr, e, -1);
                     if (d_status) atomicOr(d_status, (int32_t)id[j] >= 0 ? FGL_STATUS_TABLE_FULL : FGL_STATUS_BAD_ID);
                 }
             }
@@ -531,6 +542,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                     t.words[2 * (size_t)p[j] + 1] = (uint32_t)local;
                     uniq[local] = (int32_t)id[j];
                     out[e] = (int32_t)local;
+                    take_rank(tr, e, (int32_t)local);
                     if (next.row_start != nullptr) {
                         // (the tile's new nodes have consecutive positions: few next-hop tiles, summed in LDS first)
                         const int k = store_next_hop(next, local, row_a[j], row_deg[j]);
@@ -538,6 +550,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_arrival_kernel(TableRef t
                     }
                 } else {
                     out[e] = -1;  // the unique list is full (reported by the second pass); val stays "not numbered"
+                    take_rank(tr, e, -1);
                 }
                 p[j] = kDone;
             }
@@ -559,15 +572,19 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
                                                                        int32_t* __restrict__ out, const int32_t* __restrict__ counter,
                                                                        int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                        int64_t capacity, int32_t* __restrict__ d_n_total_out,
-                                                                       uint32_t* __restrict__ d_status)
+                                                                       uint32_t* __restrict__ d_status, const TransposeRank tr,
+                                                                       const TransposeJob before)
 {
+    tjob_fill<kBlock>(before);  // (the hop before, if its transposed block is being built: entries into their rows)
     const int64_t n_e = actual_count(e_max, d_e);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
         const uint32_t p = slot_of[e];
         if (p >= kDone) continue;  // relabelled by the first pass (kDone) or reported there (kEmpty)
         const uint32_t v = t.words[2 * (size_t)p + 1];
-        out[e] = (v & 0x80000000u) ? -1 : (int32_t)v;  // (still unnumbered: the unique list was full)
+        const int32_t local = (v & 0x80000000u) ? -1 : (int32_t)v;  // (still unnumbered: the unique list was full)
+        out[e] = local;
+        take_rank(tr, e, local);
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
@@ -627,7 +644,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base, int32_t* d_n_total_out,
                          int32_t* d_uniq, int64_t uniq_capacity, int flags, uint32_t* d_status, void* d_ws,
                          size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed, const NextHop* next_hop,
-                         bool leave_table_empty, uint8_t* d_lowered)
+                         bool leave_table_empty, uint8_t* d_lowered, const TransposeJob* rank_job,
+                         const TransposeJob* before_job)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
@@ -654,6 +672,19 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     const unsigned tile_blocks = stride_grid(n_edges_max, kTile);
     NextHop next{};  // all null: nothing to prepare
     if (next_hop != nullptr) next = *next_hop;
+    const TransposeRank tr = rank_of(rank_job);
+    TransposeJob before;
+    memset(&before, 0, sizeof(before));
+    if (before_job != nullptr) before = *before_job;
+    // the two passes that carry the hop before's scan and fill steps get workgroups of their own for those,
+    // behind the pass's own
+    TransposeJob scan_job = before, fill_job = before;
+    unsigned scan_blocks = 0, fill_blocks_t = 0;
+    if (before.cnt != nullptr) {
+        scan_job.side_first = fill_job.side_first = 0;
+        scan_blocks = scan_job.side_blocks = side_blocks_for(before.cols_max * before.split + 1, kTjobTile);
+        fill_blocks_t = fill_job.side_blocks = side_blocks_for(before.rows_max, kBlock / 16);
+    }
     FGL_REQUIRE(!leave_table_empty || final_call, "idmap_map_src: only a final call can leave the table empty");
 
     if (flags & FGL_IDMAP_ARRIVAL) {
@@ -666,17 +697,18 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
             if (rc0 != FGL_OK) return rc0;
         }
         if (n_edges_max > kArrivalSmallEdges)
-            hipLaunchKernelGGL(idmap_insert_arrival_kernel<kArrivalItems>, dim3(stride_grid(n_edges_max, kBlock * kArrivalItems)),
+            hipLaunchKernelGGL(idmap_insert_arrival_kernel<kArrivalItems>,
+                               dim3(stride_grid(n_edges_max, kBlock * kArrivalItems) + scan_blocks),
                                dim3(kBlock), 0, stream, t, d_src_in,
                                n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
-                               d_status, next);
+                               d_status, next, tr, scan_job);
         else
-            hipLaunchKernelGGL(idmap_insert_arrival_kernel<1>, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+            hipLaunchKernelGGL(idmap_insert_arrival_kernel<1>, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
                                n_edges_max, d_n_edges, n_base, d_n_base, slot_of, counter, d_uniq, uniq_capacity, d_src_out,
-                               d_status, next);
+                               d_status, next, tr, scan_job);
         FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
-        hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
+        hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
+                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, tr, fill_job);
         FGL_CHECK_LAUNCH("idmap_relabel_publish_kernel");
         // (the second pass reads the table, so emptying it takes a launch of its own here)
         if (leave_table_empty) return launch_fill_u32(t.words, slots * 2, kEmpty, stream);
@@ -685,16 +717,16 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
 
     // (the holder bit shares a word with the slot index: tables of 2^31 slots go without the bookkeeping)
     uint8_t* lowered = slots <= ((int64_t)1 << 30) ? d_lowered : nullptr;
-    hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,
-                       n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status);
+    hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+                       n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
-    hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                       slot_of, lowered, first_of, flags8, before8, sums);
+    hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
+                       slot_of, lowered, first_of, flags8, before8, sums, fill_job);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
 #define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS)                                                              \
     hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
-                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words)
+                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words, tr)
     // emptying the table rides on the last pass: enough workgroups for a fill of that size
     uint32_t* clear_words = leave_table_empty ? t.words : nullptr;
     const int64_t n_clear_words = leave_table_empty ? slots * 2 : 0;
@@ -763,7 +795,7 @@ FGL_EXPORT int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_
 {
     return launch_idmap_map_src(d_table, slots, d_src_in, d_src_out, n_edges_max, d_n_edges, n_base, d_n_base,
                                 d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream), false,
-                                nullptr, false, nullptr);
+                                nullptr, false, nullptr, nullptr, nullptr);
 }
 
 FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,

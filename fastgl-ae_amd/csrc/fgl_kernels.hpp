@@ -34,6 +34,53 @@ struct NextHop {
     int tile_seeds;
 };
 
+// A block's transposed form under construction inside the all-hops call (fgl_transpose_job.hpp).  cnt == nullptr:
+// no such work.
+struct TransposeJob {
+    int32_t* cnt;        // split * cols_max + 1 counters, then their prefix sums; split == 1: the same array as t_ptr
+    int32_t* tile_sums;  // one per 2048 counters
+    int32_t* rank;       // per edge: its position within its transposed row
+    int32_t* t_ptr;      // cols_max + 1
+    int32_t* t_dst;      // edges_max
+    int32_t* t_edge;     // edges_max, or null
+    int32_t* longest;    // one int, zero before the scan step: the longest transposed row if beyond FGL_SHORT_ROW_ENTRIES
+    const int32_t* block_ptr;
+    const int32_t* src_local;
+    const int32_t* d_n_rows;
+    const int32_t* d_n_cols;
+    const int32_t* d_n_edges;
+    int64_t rows_max, cols_max, edges_max;
+    int split;
+    // which workgroups of the launch at hand work on the step it carries: side_blocks of them, the last of the
+    // grid but side_first (set per launch by the launcher, which appends them to the grid)
+    int side_blocks, side_first;
+};
+// Side workgroups for a step over n_items, items_per_block at a time: never more than the work needs, and few
+// enough that they are an appendix to the launch that carries them.
+inline int side_blocks_for(int64_t n_items, int64_t items_per_block, int cap = 1024)
+{
+    int64_t b = (n_items + items_per_block - 1) / items_per_block;
+    if (b < 1) b = 1;
+    return (int)(b < cap ? b : cap);
+}
+// what the id-map passes need of it: where an edge takes its rank
+struct TransposeRank {
+    int32_t* cnt;
+    int32_t* rank;  // null: no transposed block is being built
+    int64_t cols_max;
+    int split;
+};
+inline TransposeRank rank_of(const TransposeJob* j)
+{
+    return j && j->cnt ? TransposeRank{j->cnt, j->rank, j->cols_max, j->split} : TransposeRank{nullptr, nullptr, 0, 1};
+}
+// what one launch carries along for the transposed blocks: steps of the hop before (tile sums / scan / fill, by the
+// launch's place in the hop) and the zeroing of this hop's counters (sampling launch only)
+struct TransposeSteps {
+    TransposeJob before;
+    TransposeJob zero;
+};
+
 // neighbour sampling (fgl_sample.hip)
 int sample_tile_seeds(int fanout, int64_t n_seeds_max);
 int64_t sample_tile_count(int64_t n_seeds_max, int fanout);
@@ -44,7 +91,8 @@ int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_
                         int32_t* tile_prefix, uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out,
                         int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
                         hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next,
-                        uint8_t* d_zero_per_edge = nullptr);  // (optional) one byte per output edge, cleared along with the writes
+                        uint8_t* d_zero_per_edge = nullptr,   // (optional) one byte per output edge, cleared along with the writes
+                        const TransposeSteps* steps = nullptr);  // (optional) zero this hop's counters, tile sums of the hop before
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
@@ -63,7 +111,9 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          bool counter_is_zeroed,          // arrival order: *d_n_total_out holds zero and may count the new ids
                          const NextHop* next_hop,         // (may be null) the new nodes are seeds of a next hop: prepare its sampling
                          bool leave_table_empty,          // final calls only: every slot of the table is empty when the call's work is done
-                         uint8_t* d_lowered);             // (may be null) n_edges_max bytes, zero on entry: lets the mark pass skip most table reads
+                         uint8_t* d_lowered,              // (may be null) n_edges_max bytes, zero on entry: lets the mark pass skip most table reads
+                         const TransposeJob* rank_job = nullptr,     // (may be null) the edges take their ranks in this block's transposed rows
+                         const TransposeJob* before_job = nullptr);  // (may be null) scan and fill steps of the hop before, carried by the first two passes
 
 // deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
 size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);

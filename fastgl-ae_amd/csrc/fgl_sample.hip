@@ -19,6 +19,7 @@
 
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
+#include "fgl_transpose_job.hpp"
 
 // Scratch of fgl_sample_node_static: device memory that belongs to the library, one copy per GPU, held
 // until the process ends.  In host code this name is only a handle for hipGetSymbolAddress -- it is
@@ -29,7 +30,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace fgl {
 
-constexpr int64_t kStaticMaxSeeds = (int64_t)1 << 20;  // 12.2 bytes of scratch per seed at most: fits 16 MiB
+constexpr int64_t kStaticMaxSeeds = FGL_STATIC_MAX_SEEDS;  // 12.2 bytes of scratch per seed at most: fits 16 MiB
 constexpr int kStaticMaxDevices = 64;
 
 // The calling thread's current device's copy of `scratch` (each GPU holds its own at its own address).
@@ -167,7 +168,8 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                                                           int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
                                                           int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
                                                           uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
-                                                          int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge)
+                                                          int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge,
+                                                          const TransposeSteps steps)
 {
     extern __shared__ uint32_t s_sel[];  // [fanout][TS] picked positions
     __shared__ int s_scan[TS / kWave + 1];
@@ -178,6 +180,9 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
 
     const int tid = (int)threadIdx.x;
     if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
+    // work for the transposed blocks that this launch carries along (nothing in the per-hop operator)
+    tjob_zero<TS>(steps.zero);
+    tjob_tile_sums<TS>(steps.before);
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
     publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
@@ -272,7 +277,8 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
                                                               int32_t* __restrict__ src_out, int32_t* __restrict__ dst_out,
                                                               int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
                                                               uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
-                                                              int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge)
+                                                              int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge,
+                                                              const TransposeSteps steps)
 {
     extern __shared__ int32_t s_stage[];  // [TS*fanout] sampled ids (+ [TS*fanout] seed ids when dst_out is wanted)
     __shared__ int s_scan[TS / kWave + 1];
@@ -281,6 +287,9 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
 
     const int tid = (int)threadIdx.x;
     if (d_stream_add) stream_id += *d_stream_add;  // lets a captured launch sequence advance its random stream
+    // work for the transposed blocks that this launch carries along (nothing in the per-hop operator)
+    tjob_zero<TS>(steps.zero);
+    tjob_tile_sums<TS>(steps.before);
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
     publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
@@ -373,10 +382,28 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
                            int fanout, const int64_t* row_start, const int32_t* deg, const int32_t* sums, int32_t* prefix,
                            uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                            int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, hipStream_t stream,
-                           const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge)
+                           const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge,
+                           const TransposeSteps* steps_in)
 {
     const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, TS);
-    const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    TransposeSteps steps;
+    memset(&steps, 0, sizeof(steps));
+    if (steps_in) {
+        steps = *steps_in;
+        // the carried steps get workgroups of their own behind the sampling ones: clearing this hop's counters
+        // (16 per lane), then the tile sums of the hop before
+        if (steps.zero.cnt != nullptr) {
+            steps.zero.side_first = 0;
+            steps.zero.side_blocks = side_blocks_for(steps.zero.cols_max * steps.zero.split + 1, (int64_t)TS * 16);
+            grid += (unsigned)steps.zero.side_blocks;
+        }
+        if (steps.before.cnt != nullptr) {
+            steps.before.side_first = steps.zero.cnt != nullptr ? steps.zero.side_blocks : 0;
+            steps.before.side_blocks = side_blocks_for(steps.before.cols_max * steps.before.split + 1, kTjobTile);
+            grid += (unsigned)steps.before.side_blocks;
+        }
+    }
     // few tiles: each workgroup of the edges kernel sums the earlier tile sums itself (the last one
     // publishes the totals), which saves the scan launch in between
     if (tiles > kSampleSelfPrefixTiles) {
@@ -397,7 +424,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
                        (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, \
-                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge)
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps)
         if (fanout <= 8) FGL_LAUNCH_REG(8);
         else if (fanout <= 16) FGL_LAUNCH_REG(16);
         else FGL_LAUNCH_REG(32);
@@ -409,7 +436,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
     hipLaunchKernelGGL((sample_edges_kernel<TS, 16>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,
                        (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out,
-                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge);
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps);
     FGL_CHECK_LAUNCH("sample_edges_kernel");
     return FGL_OK;
 }
@@ -418,15 +445,16 @@ int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_
                         int fanout, const int64_t* row_start, const int32_t* deg, const int32_t* tile_sums,
                         int32_t* tile_prefix, uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out,
                         int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
-                        hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge)
+                        hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge,
+                        const TransposeSteps* steps)
 {
     if (sample_tile_seeds(fanout, n_seeds_max) == 256)
         return launch_edges_ts<256>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
                                     rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
-                                    d_stream_add, next, d_zero_per_edge);
+                                    d_stream_add, next, d_zero_per_edge, steps);
     return launch_edges_ts<64>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
                                rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
-                               d_stream_add, next, d_zero_per_edge);
+                               d_stream_add, next, d_zero_per_edge, steps);
 }
 
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,

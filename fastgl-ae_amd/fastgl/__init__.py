@@ -23,8 +23,6 @@ from .ops import (  # noqa: F401
     forward_gat,
     forward_gcn,
     manual_seed,
-    probe_table_access,
-    probe_xcc_of_workgroups,
     rmat_keys,
     sample_blocks_fused,
     sample_node,

@@ -17,13 +17,14 @@ CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
 
 # enum values of include/fastgl_hip.h
 F32, BF16 = 0, 1
-AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE = 0, 1, 2, 3, 4
+AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE, AGG_COLMEAN_PTR = 0, 1, 2, 3, 4, 5
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
-ABI_VERSION = 9  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
+ABI_VERSION = 10  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL = 0, 1, 2
 BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
 MAX_FANOUT = 192
+SHORT_ROW_ENTRIES = 32
 TRANSPOSE_BATCH_MAX, TRANSPOSE_BATCH_MAX_EDGES, TRANSPOSE_BATCH_MAX_COLS = 8, 1 << 20, 1 << 23
 
 _i64, _i32, _u64, _u32, _vp, _sz = C.c_int64, C.c_int, C.c_uint64, C.c_uint32, C.c_void_p, C.c_size_t
@@ -46,19 +47,18 @@ SIGNATURES = {
     "fgl_idmap_map_src_workspace_bytes": (_sz, [_i64]),
     "fgl_idmap_map_src": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _sz, _vp]),
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
-    "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]),
     "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _vp, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
-                                 _vp, _vp, _sz, _vp]),
+                                 _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp, _sz, _vp]),
     "fgl_block_transpose_batch_workspace_bytes": (_sz, [_i32, _vp, _vp]),
     "fgl_block_transpose_batch": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_aggregate": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
                              _vp, _i64, _vp]),
+    "fgl_aggregate_last_mapping": (C.c_char_p, []),
     "fgl_edge_softmax": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, C.c_float, _vp, _vp]),
     "fgl_rmat_keys": (_i32, [_i64, _i64, _i32, _i64, _u64, _vp, _vp]),
-    "fgl_probe_table_access": (_i32, [_vp, _i64, _i64, _i32, _i32, _u32, _vp, _vp]),
-    "fgl_probe_xcc_of_workgroups": (_i32, [_vp, _i32, _vp]),
 }
 
 _lib = None

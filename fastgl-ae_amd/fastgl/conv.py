@@ -349,8 +349,9 @@ class MA_Function_Mean(torch.autograd.Function):
             return None, None, None
         block = ctx.block
         t_ptr, t_idx = block.transposed()
-        d_feat = ops.aggregate(t_ptr, t_idx, d_out.contiguous(), mode="colmean", zero_policy="zeros",
-                               col_norm=block.in_degrees().contiguous(), n_rows=ctx.n_src)
+        # (the destination rows' entry counts are the differences of the block's own row pointer: no degree array)
+        d_feat = ops.aggregate(t_ptr, t_idx, d_out.contiguous(), mode="colmean_ptr", zero_policy="zeros",
+                               col_norm=block.edge_ptr, n_rows=ctx.n_src)
         return None, d_feat, None
 
 

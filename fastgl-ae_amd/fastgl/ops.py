@@ -281,14 +281,16 @@ def backward_gat(edge_ptr, edge_data, src_edges, d_input, src_nodes, num_heads):
 # ---------------------------------------------------------------------------------------
 # extensions
 # ---------------------------------------------------------------------------------------
-_MODES = {"sum": L.AGG_SUM, "mean": L.AGG_MEAN, "gcn": L.AGG_GCN, "colmean": L.AGG_COLMEAN, "edge": L.AGG_EDGE}
+_MODES = {"sum": L.AGG_SUM, "mean": L.AGG_MEAN, "gcn": L.AGG_GCN, "colmean": L.AGG_COLMEAN, "edge": L.AGG_EDGE,
+          "colmean_ptr": L.AGG_COLMEAN_PTR}
 _ZERO = {"self": L.ZERO_COPY_SELF, "zeros": L.ZERO_ZEROS}
 
 
 def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=None, col_norm=None, n_rows=None,
               out=None, edge_weight=None, n_heads=1, edge_index=None, longest_row=None, n_rows_dev=None, mapping="auto"):
     """``out[r] = sum_e w(r, indices[e]) * feat[indices[e]]`` over the CSR rows (fp32
-    accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge;
+    accumulation; fp32 or bf16 storage).  ``mode``: sum | mean | gcn | colmean | edge | colmean_ptr (colmean with
+    ``col_norm`` holding the offsets array whose differences are the counts: a block's ``edge_ptr``);
     ``zero_policy``: what a row without entries gets -- ``self`` (``feat[r]``) or ``zeros``.
     ``longest_row``: what is known about the longest row's entry count -- an ``int`` bound (the fanout of a
     sampled block) or a one-element int32 device tensor (as ``block_transpose`` makes).  Speed only: hub rows
@@ -466,9 +468,11 @@ def table_size(num: int, scale: int) -> int:
 class BlocksPlan:
     """Bounds and persistent scratch for sampling mini-batches of one shape."""
 
-    def __init__(self, n_nodes: int, n_seeds: int, hop_fanouts, device, node_capacity=None):
+    def __init__(self, n_nodes: int, n_seeds: int, hop_fanouts, device, node_capacity=None, transpose_hops=()):
         """``node_capacity`` (optional, ``n_hops + 1`` ints): the caller's own limit on the node count
-        before each hop / after the last; the worst-case bounds are clipped to it."""
+        before each hop / after the last; the worst-case bounds are clipped to it.
+        ``transpose_hops``: the hops (sampling order, negative = from the end) whose transposed block
+        ``sample_blocks_fused`` is to build along the way."""
         lib = L.lib()
         self.n_nodes, self.n_seeds = int(n_nodes), int(n_seeds)
         self.hop_fanouts = [int(f) for f in hop_fanouts]
@@ -479,11 +483,14 @@ class BlocksPlan:
         cap_dst = (C.c_int64 * self.n_hops)()
         cap_edges = (C.c_int64 * self.n_hops)()
         cap_uniq, slots, ws_bytes = C.c_int64(), C.c_int64(), C.c_size_t()
-        L.check(lib.fgl_sample_blocks_plan(self.n_nodes, self.n_seeds, self._fan, self.n_hops, self._node_cap, cap_dst, cap_edges,
-                                           C.byref(cap_uniq), C.byref(slots), C.byref(ws_bytes)))
+        self.transpose_hops = sorted({(int(h) + self.n_hops) % self.n_hops for h in transpose_hops})
+        self.transpose_mask = sum(1 << h for h in self.transpose_hops)
+        L.check(lib.fgl_sample_blocks_plan(self.n_nodes, self.n_seeds, self._fan, self.n_hops, self._node_cap, self.transpose_mask,
+                                           cap_dst, cap_edges, C.byref(cap_uniq), C.byref(slots), C.byref(ws_bytes)))
         self.cap_dst = list(cap_dst)
         self.cap_edges = list(cap_edges)
         self.cap_uniq, self.slots, self.ws_bytes = cap_uniq.value, slots.value, ws_bytes.value
+        self.cap_src = self.cap_dst[1:] + [self.cap_uniq]  # source nodes (columns) of each hop's block
         self.table = torch.empty(self.slots, dtype=torch.int64, device=self.device)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=self.device)
         # the slot count that the last call on this plan's table left empty (None: unknown contents)
@@ -495,9 +502,12 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
-    src_global[h] or None, counts)``; hop 0 expands the raw seeds.  ``counts`` (int32,
-    ``2*n_hops + 2``) holds the node count before each hop and after the last, then the
-    edge count of each hop, then the status word; the caller reads it once per batch.
+    src_global[h] or None, counts, transposed[h])``; hop 0 expands the raw seeds.  ``counts`` (int32,
+    ``3*n_hops + 2``) holds the node count before each hop and after the last, then the
+    edge count of each hop, then the status word, then per hop the longest row of its transposed block
+    (zero where none was built); the caller reads it once per batch.
+    For the hops in ``plan.transpose_hops`` the call also builds the transposed block:
+    ``transposed[h] = (t_ptr, t_dst, t_edge)`` (bound-sized; ``None`` for the other hops).
     ``keep_global`` lists the hops (negative = from the end) whose pre-relabel source ids are kept.
     ``table_slots`` (a power of two, default the plan's worst case) uses only that much of the
     hash table; a batch that outgrows it is reported in the status word (FGL_STATUS_TABLE_FULL).
@@ -524,8 +534,14 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         src_local = [torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev) for h in range(H)]
         src_global = [torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev) if h in keep else None
                       for h in range(H)]
-        counts = torch.empty(2 * H + 2, dtype=torch.int32, device=dev)
+        counts = torch.empty(3 * H + 2, dtype=torch.int32, device=dev)
         arr = lambda ts: (C.c_void_p * H)(*[L.ptr(t) for t in ts])
+        transposed = [None] * H
+        for h in plan.transpose_hops:
+            transposed[h] = (torch.empty(plan.cap_src[h] + 1, dtype=torch.int32, device=dev),
+                             torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev),
+                             torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev))
+        t_arr = lambda k: arr([None if t is None else t[k] for t in transposed]) if plan.transpose_hops else None
         # every call leaves the table empty for the next one (its last pass no longer reads it), so only a
         # plan's first call -- or the first after a failed one, or with another slot count -- pays for a fill
         flags = {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order] | L.BLOCKS_LEAVE_TABLE_EMPTY
@@ -536,10 +552,10 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF, L.ptr(stream_offset),
                                       flags, L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
-                                      arr(src_local), arr(src_global), L.ptr(counts), L.ptr(plan.ws), plan.ws.numel(),
-                                      L.stream_handle()))
+                                      arr(src_local), arr(src_global), t_arr(0), t_arr(1), t_arr(2), L.ptr(counts), L.ptr(plan.ws),
+                                      plan.ws.numel(), L.stream_handle()))
         plan.empty_slots = slots
-    return uniq, block_ptr, src_local, src_global, counts
+    return uniq, block_ptr, src_local, src_global, counts, transposed
 
 
 def rmat_keys(first_edge: int, n_edges: int, scale: int, n_nodes: int, seed: int, device) -> torch.Tensor:
@@ -550,24 +566,3 @@ def rmat_keys(first_edge: int, n_edges: int, scale: int, n_nodes: int, seed: int
                                       int(seed) & 0xFFFFFFFFFFFFFFFF, L.ptr(keys), L.stream_handle()))
     return keys
 
-
-PROBE_OPS = {"load": 0, "cas": 1, "load_then_cas": 2, "add": 3, "cas_workgroup_scope": 4}
-PROBE_PATTERNS = {"whole_table": 0, "eighth_of_own_xcd": 1, "eighth_not_aligned": 2}
-
-
-def probe_table_access(table: torch.Tensor, n_ops: int, pattern: str, op: str, salt: int = 0) -> None:
-    """One pseudo-random 8-byte access per lane into ``table`` (int64, a power of two of entries); see
-    ``fgl_probe_table_access`` in include/fastgl_hip.h.  Enqueues on the current stream."""
-    _check_input(table, "table", (torch.int64,))
-    with torch.cuda.device(table.device):
-        sink = torch.zeros(1, dtype=torch.int64, device=table.device)
-        L.check(L.lib().fgl_probe_table_access(L.ptr(table), int(table.numel()), int(n_ops), PROBE_PATTERNS[pattern],
-                                               PROBE_OPS[op], int(salt) & 0xFFFFFFFF, L.ptr(sink), L.stream_handle()))
-
-
-def probe_xcc_of_workgroups(n_workgroups: int, device) -> torch.Tensor:
-    """8 x 16 counts: entry [w % 8, x] = workgroups of index w that ran on the XCD whose hardware id is x."""
-    with torch.cuda.device(device):
-        hist = torch.zeros((8, 16), dtype=torch.int32, device=device)
-        L.check(L.lib().fgl_probe_xcc_of_workgroups(L.ptr(hist), int(n_workgroups), L.stream_handle()))
-    return hist

@@ -134,7 +134,7 @@ class PendingBatch:
 
     def __init__(self, sampler, pending):
         self._sampler, self._pending = sampler, pending
-        _, bptr, _, src_g, counts = pending["out"]
+        _, bptr, _, src_g, counts, _ = pending["out"]
         H = len(sampler.fanouts)
         self.outer_edge_ptr = bptr[H - 1]        # int32[bound + 1]: row offsets of the outermost block
         self.outer_src_global = src_g[H - 1]     # int32[edge bound]: its neighbour lists in graph ids
@@ -169,7 +169,7 @@ class PendingBatch:
 class FusedMapSampler:
     def __init__(self, fanouts, edge_dir='in', prob=None, mask=None, replace=False, prefetch_node_feats=None,
                  prefetch_labels=None, prefetch_edge_feats=None, output_device=None, fused=True, rng_seed=0,
-                 id_order="first", deterministic=False, graph_slots=0):
+                 id_order="first", deterministic=False, graph_slots=0, transposed="inner"):
         if mask is not None and prob is not None:
             raise ValueError('Mask and probability arguments are mutually exclusive. '
                              'Consider multiplying the probability with the mask to achieve the same goal.')
@@ -199,6 +199,13 @@ class FusedMapSampler:
         # are hidden behind the previous step's kernels anyway.  The price: outputs live in R fixed slots used in
         # turn, so the tensors of a mini-batch are overwritten when the R-th mini-batch after it is sampled --
         # consume (or clone) them before that.
+        # transposed: which blocks come with their transposed form (what the backward pass of a layer gathers over),
+        # built inside the fused sampling call at next to no cost: "inner" = every block but the outermost (the first
+        # layer's input needs no gradient), "all", or "none" (built on demand, Block.transposed()).  A deterministic
+        # sampler orders its transposed lists and builds them on demand.
+        if transposed not in ("inner", "all", "none"):
+            raise ValueError("transposed must be 'inner', 'all' or 'none'")
+        self.transposed = "none" if self.deterministic else transposed
         self.graph_slots = int(graph_slots)
         if self.graph_slots < 0 or self.graph_slots == 1:
             raise ValueError("graph_slots must be 0 (off) or at least 2")
@@ -266,7 +273,9 @@ class FusedMapSampler:
         caps = None if worst_case else self._caps(state, n_seeds)
         plan = state.plans.get(caps)
         if plan is None:
-            plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps)
+            n_hops = len(hop_fanouts)
+            hops = {"inner": range(n_hops - 1), "all": range(n_hops), "none": ()}[self.transposed]
+            plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps, transpose_hops=hops)
             state.plans = {k: v for k, v in state.plans.items() if k is None}  # keep the worst-case plan only
             state.plans[caps] = plan
         slots = plan.slots
@@ -292,7 +301,14 @@ class FusedMapSampler:
         slot = ring[turn]
         slot["seeds"].copy_(seeds)
         slot["offset"].fill_(stream_base - (1 << 32) if stream_base >= (1 << 31) else stream_base)  # uint32 bits in an int32
+        # A captured sequence holds no table fill: it was recorded behind a call that left the table empty, and
+        # leaves it empty itself.  If anything since then may have left entries behind (a call on this plan that
+        # failed half-way), the table is emptied here, eagerly, before the replay.
+        if plan.empty_slots != slots:
+            ops.L.check(ops.L.lib().fgl_idmap_reset(ops.L.ptr(plan.table), slots, ops.L.stream_handle()))
+        plan.empty_slots = None
         slot["graph"].replay()
+        plan.empty_slots = slots
         return slot["out"]
 
     def _capture(self, plan, slots, dev):
@@ -338,14 +354,21 @@ class FusedMapSampler:
             state.nodes_seen = seen
         elif any(a > 1.25 * b for a, b in zip(seen, state.nodes_seen)):
             state.nodes_seen = [max(a, b) for a, b in zip(seen, state.nodes_seen)]
-        uniq, bptr, src_l, src_g, _ = pending["out"]
+        uniq, bptr, src_l, src_g, _, transposed = pending["out"]
         blocks = []
         for h in range(H):
             n_dst, n_src, n_e = c[h], c[h + 1], c[H + 1 + h]
             block_ptr = bptr[h][:n_dst + 1]
             block_ptr.fgl_longest_row = int(self.fanouts[H - 1 - h])  # no row exceeds the fanout (read by ops.aggregate)
-            blocks.insert(0, Block(block_ptr, src_l[h][:n_e], n_src, n_dst,
-                                   None if src_g[h] is None else src_g[h][:n_e], sorted_transpose=self.deterministic))
+            block = Block(block_ptr, src_l[h][:n_e], n_src, n_dst, None if src_g[h] is None else src_g[h][:n_e],
+                          sorted_transpose=self.deterministic)
+            if transposed[h] is not None:
+                # built by the same call; its longest row came back with the sizes, so the backward gather knows
+                # on the host whether any row needs the hub-row launch
+                t_ptr = transposed[h][0][:n_src + 1]
+                t_ptr.fgl_longest_row = max(int(c[2 * H + 2 + h]), ops.L.SHORT_ROW_ENTRIES)
+                block._transposed = (t_ptr, transposed[h][1][:n_e], transposed[h][2][:n_e])
+            blocks.insert(0, block)
         return uniq[:c[H]], pending["seeds"], blocks
 
     def begin_sample(self, seed_nodes):
@@ -393,7 +416,7 @@ class FusedMapSampler:
             side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
             with torch.cuda.stream(side):
                 pending = self._launch_fused(seeds, stream_base)
-                host = torch.empty(2 * H + 2, dtype=torch.int32, pin_memory=True)
+                host = torch.empty(3 * H + 2, dtype=torch.int32, pin_memory=True)
                 host.copy_(pending["out"][4], non_blocking=True)
                 done = torch.cuda.Event()
                 done.record(side)

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 9
+#define FGL_ABI_VERSION 10
 
 enum fgl_error {
     FGL_OK = 0,
@@ -50,7 +50,10 @@ enum fgl_agg_mode {
     FGL_AGG_MEAN = 1,    /* w = 1 / deg(row)                                  (SAGE) */
     FGL_AGG_GCN = 2,     /* w = (1/sqrt(row_norm[row])) * (1/sqrt(col_norm[col]))    */
     FGL_AGG_COLMEAN = 3, /* w = 1 / max(col_norm[col], 1)   (backward of MEAN)        */
-    FGL_AGG_EDGE = 4     /* w = edge_w[entry_id * n_heads + column / (D / n_heads)]  (GAT) */
+    FGL_AGG_EDGE = 4,    /* w = edge_w[entry_id * n_heads + column / (D / n_heads)]  (GAT) */
+    FGL_AGG_COLMEAN_PTR = 5 /* FGL_AGG_COLMEAN with the columns' entry counts given as an offsets array:
+                               col_norm[col+1] - col_norm[col] -- the row pointer of the block whose transpose is
+                               being gathered, so the backward of MEAN needs no degree array */
 };
 
 /* what an output row with no entries gets */
@@ -211,21 +214,36 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  *
  * Outputs (device): block_ptr[h] int32[cap_dst[h]+1], src_local[h] int32[cap_edges[h]],
  * src_global[h] int32[cap_edges[h]] or NULL; d_uniq int32[cap_uniq];
- * d_counts int32[2*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
- * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word.
+ * d_counts int32[3*n_hops+2]: [0..n_hops] node count before hop h / after the last hop,
+ * [n_hops+1 .. 2*n_hops] edges of hop h, [2*n_hops+1] the status word, [2*n_hops+2+h] the entry count of the
+ * longest row of hop h's transposed block if that exceeds FGL_SHORT_ROW_ENTRIES, else some value not above it
+ * (zero for hops whose transposed block is not built) -- read back with the sizes, it is the host bound that
+ * fgl_aggregate's longest_row_max wants.
+ *
+ * Transposed blocks (the column-major companions that the backward kernels gather over, see fgl_block_transpose):
+ * t_ptr / t_dst / t_edge are NULL, or arrays of n_hops pointers of which any may be NULL.  Where t_ptr[h] is given
+ * (int32[cap_src[h]+1], cap_src[h] = cap_dst[h+1], or cap_uniq for the last hop) the call also builds hop h's
+ * transposed block: t_ptr[h] = row pointer over the hop's source nodes, t_dst[h] int32[cap_edges[h]] (required
+ * then) = the destination rows each source node feeds, unordered within a row, t_edge[h] (optional) = the
+ * position in src_local[h] of every transposed entry.  Sizes are the call's own device-side counts, so nothing
+ * waits for the host.  The work rides on launches the call makes anyway -- a hop's edges take their place in their
+ * transposed rows as the id-map numbers them, and the next hop's launches turn the counts into offsets and
+ * fill the rows -- except for the last hop, whose transposed block costs three short launches of its own.
+ * fgl_sample_blocks_plan takes the same choice as a bit mask (bit h: hop h), since the workspace depends on it.
  * The table is scratch: after the call it holds the local ids of the nodes of every hop but the
  * last (whose new nodes keep a transient value there) -- or nothing, with FGL_BLOCKS_LEAVE_TABLE_EMPTY;
  * d_uniq is the complete map local -> global.
  * ------------------------------------------------------------------------------- */
 int fgl_sample_blocks_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops,
-                           const int64_t* node_capacity, int64_t* cap_dst, int64_t* cap_edges, int64_t* cap_uniq,
-                           int64_t* table_slots, size_t* ws_bytes);
+                           const int64_t* node_capacity, uint32_t transpose_hops, int64_t* cap_dst, int64_t* cap_edges,
+                           int64_t* cap_uniq, int64_t* table_slots, size_t* ws_bytes);
 int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                       const int32_t* d_seeds, int64_t n_seeds, const int32_t* fanouts, int n_hops,
                       const int64_t* node_capacity, uint64_t rng_seed, uint32_t stream_base,
                       const uint32_t* d_stream_offset, int idmap_flags,
                       void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
                       int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
+                      int32_t* const* t_ptr, int32_t* const* t_dst, int32_t* const* t_edge,
                       int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
@@ -297,6 +315,11 @@ int fgl_aggregate(const int32_t* d_indptr, const int32_t* d_indices,
                   const float* d_edge_w, int n_heads, const int32_t* d_edge_index,
                   int64_t longest_row_max, const int32_t* d_longest_row, int64_t n_entries_max,
                   void* d_out, int64_t ldo, void* stream);
+/* Which kernel and lane mapping the calling thread's last fgl_aggregate call launched, as text ("aggregate_kernel
+ * lanes/row=32", "aggregate_bundle_kernel lanes/row=64 (rows bundled by 4) + long_rows", ...): for benchmark
+ * records and bug reports.  No counterpart in the reference, whose kernels have one fixed mapping
+ * (aggregate_acc_kernel.cu:238-247). */
+const char* fgl_aggregate_last_mapping(void);
 
 /* ---------------------------------------------------------------------------------
  * Attention coefficients of a GAT layer over a block CSR -- replaces the three DGL calls of
@@ -320,26 +343,6 @@ int fgl_edge_softmax(const int32_t* d_indptr, const int32_t* d_indices, int64_t 
  * ------------------------------------------------------------------------------- */
 int fgl_rmat_keys(int64_t first_edge, int64_t n_edges, int scale, int64_t n_nodes, uint64_t seed,
                   int64_t* d_keys, void* stream);
-
-/* ---------------------------------------------------------------------------------
- * Probes of the memory system behind the id-map's design.  No counterpart in the reference; they exist so
- * that the figures the design rests on can be re-measured on any box (bench.py --workload table_access).
- *
- * fgl_probe_table_access: n_ops lanes each make one access to a pseudo-random 8-byte slot of d_table
- * (`slots` of them, a power of two; fill it with 0xFF bytes first).
- *   pattern  0 anywhere; 1 inside the eighth of the table numbered (workgroup index % 8) -- workgroups are
- *            dealt to the 8 XCDs in turn, so that is "each XCD on its own eighth"; 2 inside the eighth
- *            ((workgroup index / 8) % 8): as partitioned, but every XCD touches every eighth
- *   op       0 load; 1 64-bit compare-and-swap of an empty slot; 2 load, then that compare-and-swap if the slot
- *            was empty; 3 32-bit add without a return value; 4 the compare-and-swap at workgroup scope
- * d_sink: 8 bytes that the kernel may write (keeps the loads alive).
- *
- * fgl_probe_xcc_of_workgroups: launches n_workgroups workgroups; d_hist (8 x 16 uint32, zeroed by the caller)
- * [(workgroup index % 8) * 16 + hardware XCC id] counts them.
- * ------------------------------------------------------------------------------- */
-int fgl_probe_table_access(void* d_table, int64_t slots, int64_t n_ops, int pattern, int op, uint32_t salt,
-                           uint64_t* d_sink, void* stream);
-int fgl_probe_xcc_of_workgroups(uint32_t* d_hist, int n_workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_pure_host_entry_points():
     lib = fastgl.lib()
-    assert lib.fgl_abi_version() == 9
+    assert lib.fgl_abi_version() == 10
     assert fastgl.table_size(40960, 2) == 131072
     assert fastgl.table_size(8110080, 2) == 16777216
     assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25
@@ -38,34 +38,44 @@ def test_pure_host_entry_points():
     assert lib.fgl_exclusive_sum_workspace_bytes(10) > 0
 
 
+def test_static_scratch_holds_the_workspace_of_its_largest_call():
+    # fgl_sample_node_static's 16 MiB array against what the workspace formula asks for at the stated seed limit
+    lib = fastgl.lib()
+    text = open(os.path.join(ROOT, "include", "fastgl_hip.h")).read()
+    max_seeds = int(re.search(r"#define FGL_STATIC_MAX_SEEDS (\d+)", text).group(1))
+    assert max_seeds == 1 << 20
+    for fanout in (1, 48, 49, L.MAX_FANOUT):
+        assert 0 < lib.fgl_sample_workspace_bytes(max_seeds, fanout) <= 16 << 20
+
+
 def test_plan_matches_the_worst_case_table():
     # batch 8192, hops expanded with 5, 10, 15 on the 111M-node graph
     fan = (C.c_int32 * 3)(5, 10, 15)
     cd, ce = (C.c_int64 * 3)(), (C.c_int64 * 3)()
     cu, sl, ws = C.c_int64(), C.c_int64(), C.c_size_t()
-    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 8192, fan, 3, None, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 8192, fan, 3, None, 0, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
     assert list(cd) == [8192, 49152, 540672]
     assert list(ce) == [40960, 491520, 8110080]
     assert cu.value == 8650752 and sl.value == 1 << 25 and ws.value > 0
     # a small graph caps the bounds
-    L.check(fastgl.lib().fgl_sample_blocks_plan(1000, 100, fan, 3, None, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    L.check(fastgl.lib().fgl_sample_blocks_plan(1000, 100, fan, 3, None, 0, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
     assert list(cd) == [100, 600, 1100] and cu.value == 1100
     # the caller's own limits clip the plan
     lim = (C.c_int64 * 4)(100, 300, 400, 500)
-    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, lim, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
+    L.check(fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, lim, 0, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)))
     assert list(cd) == [100, 300, 400] and list(ce) == [500, 3000, 6000] and cu.value == 500
     bad = (C.c_int64 * 4)(50, 300, 400, 500)
-    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, bad, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
+    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, bad, 0, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
     # limits that shrink from one hop to the next are refused (a hop's nodes are a prefix of the next hop's)
     shrinking = (C.c_int64 * 4)(100, 400, 300, 500)
-    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, shrinking, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
+    assert fastgl.lib().fgl_sample_blocks_plan(111_000_000, 100, fan, 3, shrinking, 0, cd, ce, C.byref(cu), C.byref(sl), C.byref(ws)) == 1
     assert b"below an earlier entry" in fastgl.lib().fgl_last_error()
 
 
 def test_argument_errors_are_reported_not_launched():
     lib = fastgl.lib()
     fan = (C.c_int32 * 1)(0)
-    assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, None, None, None, None, None) == 1
+    assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, 0, None, None, None, None, None) == 1
     assert b"fanout" in lib.fgl_last_error()
     assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
     assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table
@@ -190,15 +200,19 @@ def test_size_limits_are_stated_before_anything_is_launched():
     assert b"overflows int32" in lib.fgl_last_error()
     # a hop of the all-hops plan that could produce more than 2^31 edges
     fan = (C.c_int32 * 2)(192, 192)
-    assert lib.fgl_sample_blocks_plan(1 << 30, 20_000_000, fan, 2, None, None, None, None, None, None) == 1
+    assert lib.fgl_sample_blocks_plan(1 << 30, 20_000_000, fan, 2, None, 0, None, None, None, None, None) == 1
     assert b"beyond int32" in lib.fgl_last_error()
     # hop counts and fanouts outside the supported range
     fan1 = (C.c_int32 * 1)(193)
-    assert lib.fgl_sample_blocks_plan(100, 10, fan1, 1, None, None, None, None, None, None) == 1
+    assert lib.fgl_sample_blocks_plan(100, 10, fan1, 1, None, 0, None, None, None, None, None) == 1
     assert b"fanout" in lib.fgl_last_error()
     fan33 = (C.c_int32 * 33)(*([2] * 33))
-    assert lib.fgl_sample_blocks_plan(100, 10, fan33, 33, None, None, None, None, None, None) == 1
+    assert lib.fgl_sample_blocks_plan(100, 10, fan33, 33, None, 0, None, None, None, None, None) == 1
     assert b"hops" in lib.fgl_last_error()
+    # a transposed block asked for a hop that the call does not have
+    fan2 = (C.c_int32 * 2)(5, 5)
+    assert lib.fgl_sample_blocks_plan(100, 10, fan2, 2, None, 0b100, None, None, None, None, None) == 1
+    assert b"beyond the 2" in lib.fgl_last_error()
     # an id-map call whose local ids would not fit 31 bits next to the pending marker
     assert lib.fgl_idmap_map_src(fake, 64, fake, fake, (1 << 31) - 1, None, 10, None, None, fake, 100, 0, None, fake, 1 << 40, None) == 1
     assert b"31 bits" in lib.fgl_last_error()

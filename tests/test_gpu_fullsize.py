@@ -147,7 +147,8 @@ def _resident_features(n, dim, dtype, cuda, seed):
     return feat
 
 
-def _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, fanouts, rng_seed, tol, id_orders=("first", "arrival")):
+def _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, fanouts, rng_seed, tol, id_orders=("first", "arrival"),
+                                steady_batches=None, graph_replay=False):
     """One mini-batch of 8192 seeds: unique list, every block's offsets and local ids bit-exact against the
     oracle (first-occurrence numbering; the arrival rule after sorting the new ids per hop), then the outermost
     block's mean aggregation from the resident table against the fp64 oracle on the rows it gathers."""
@@ -158,15 +159,60 @@ def _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, fano
     w_inp, w_blocks = oracle.sample_blocks(h_ptr, h_src, h_seeds, fanouts, rng_seed, 0)
     print("oracle blocks:", [(b["n_src"], b["n_dst"], int(b["src_local"].size)) for b in w_blocks], flush=True)
 
+    from test_gpu_idmap_blocks import check_transposed
+
+    def same_as_oracle(got, want, want_seeds):
+        g_inp, g_out, g_blocks = got
+        w_inp_, w_blocks_ = want
+        assert torch.equal(g_out, want_seeds)
+        assert np.array_equal(g_inp.cpu().numpy(), w_inp_)
+        for b, w in zip(g_blocks, w_blocks_):
+            assert (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()) == (w["n_src"], w["n_dst"], int(w["src_local"].size))
+            assert np.array_equal(b.edge_ptr.cpu().numpy(), w["indptr"])
+            assert np.array_equal(b.src_local.cpu().numpy(), w["src_local"])
+            if b._transposed is not None:  # the inner blocks come with their transposed form
+                check_transposed(oracle, b, w)
+        assert np.array_equal(g_blocks[0].src_global.cpu().numpy(), w_blocks_[0]["src_global"])
+        assert [b._transposed is not None for b in g_blocks] == [False] + [True] * (len(g_blocks) - 1)
+
     sampler = fastgl.FusedMapSampler(fanouts, rng_seed=rng_seed).set_graph(ptr, src)
     input_nodes, out_nodes, blocks = sampler.sample_blocks(None, seeds)
-    assert torch.equal(out_nodes, seeds)
-    assert np.array_equal(input_nodes.cpu().numpy(), w_inp)
-    for b, w in zip(blocks, w_blocks):
-        assert (b.num_src_nodes(), b.num_dst_nodes(), b.num_edges()) == (w["n_src"], w["n_dst"], int(w["src_local"].size))
-        assert np.array_equal(b.edge_ptr.cpu().numpy(), w["indptr"])
-        assert np.array_equal(b.src_local.cpu().numpy(), w["src_local"])
-    assert np.array_equal(blocks[0].src_global.cpu().numpy(), w_blocks[0]["src_global"])
+    same_as_oracle((input_nodes, out_nodes, blocks), (w_inp, w_blocks), seeds)
+
+    # The steady state, which is what a training loop and the benchmark run: the same sampler's next mini-batches use
+    # buffers and a hash table sized from the batches before (a fraction of the worst case), skip the table fill
+    # (the batch before left the table empty), and may be enqueued ahead of their read-back (begin_sample / finish)
+    # or replayed from a captured graph.  Each form, on fresh seeds, bit for bit against the oracle.
+    pool = torch.randperm(n, device=cuda, generator=torch.Generator(device=cuda).manual_seed(rng_seed + 100))
+    n_extra = 3 if steady_batches is None else steady_batches
+    first_state = sampler._state_for(seeds)
+    assert first_state.nodes_seen is not None
+    for i in range(1, 1 + n_extra):
+        s_i = pool[i * 8192:(i + 1) * 8192].int()
+        want = oracle.sample_blocks(h_ptr, h_src, s_i.cpu().numpy(), fanouts, rng_seed, 64 * i)
+        if i == n_extra:  # the last of them through the two-phase form
+            pend = sampler.begin_sample(s_i)
+            got = pend.finish()
+            assert not pend.redone
+        else:
+            got = sampler.sample_blocks(None, s_i)
+        (plan,) = [v for k, v in first_state.plans.items() if k is not None]  # the plan sized by experience
+        worst = first_state.plans[None]
+        assert plan.cap_uniq < worst.cap_uniq and sum(plan.cap_edges) < sum(worst.cap_edges)
+        assert plan.empty_slots is not None and plan.empty_slots < worst.slots  # a small table, left empty by the batch
+        same_as_oracle(got, want, s_i)
+        print("steady-state batch %d ok (%d edges)" % (i, sum(b.num_edges() for b in got[2])), flush=True)
+    if graph_replay:
+        gs = fastgl.FusedMapSampler(fanouts, rng_seed=rng_seed, graph_slots=2).set_graph(ptr, src)
+        for i in range(4):  # batch 0 eager (worst-case plan); 1 and 2 capture the two slots; 3 replays slot 0
+            s_i = pool[i * 8192:(i + 1) * 8192].int() if i else seeds
+            want = oracle.sample_blocks(h_ptr, h_src, s_i.cpu().numpy(), fanouts, rng_seed, 64 * i)
+            got = gs.sample_blocks(None, s_i)
+            same_as_oracle(got, want, s_i)
+        st = gs._state_for(seeds)
+        assert st.graphs is not None and all(slot is not None for slot in st.graphs[2])
+        print("graph replay ok", flush=True)
+        del gs, got
 
     if "arrival" in id_orders:
         # the reference's numbering rule: any run is a valid map -- per hop the same set of new ids (the rows of
@@ -226,7 +272,7 @@ def test_large_resident_shape_vs_oracle(cuda, oracle):
     h_ptr, h_src = ptr.cpu().numpy(), src.cpu().numpy()
     print("graph on the host: %d edges" % h_src.size, flush=True)
     feat = _resident_features(n, 128, torch.float32, cuda, seed=1)
-    _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, [15, 10, 5], rng_seed=5, tol=1e-5)
+    _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, [15, 10, 5], rng_seed=5, tol=1e-5, graph_replay=True)
     del feat, ptr, src
     torch.cuda.empty_cache()
 
@@ -246,6 +292,6 @@ def test_very_large_shape_vs_oracle(cuda, oracle):
     feat = _resident_features(n, 128, torch.bfloat16, cuda, seed=2)
     _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, [15, 10, 5], rng_seed=6, tol=1e-2)
     print("full-size: deep fanout", flush=True)
-    _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, [10, 10, 10, 10, 10], rng_seed=7, tol=1e-2)
+    _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, [10, 10, 10, 10, 10], rng_seed=7, tol=1e-2, steady_batches=2)
     del feat, ptr, src
     torch.cuda.empty_cache()

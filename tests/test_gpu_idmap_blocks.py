@@ -93,6 +93,28 @@ def check_blocks(oracle, indptr, indices, seeds, fanouts, got, rng_seed, stream_
             assert np.array_equal(b.src_global.cpu().numpy(), w["src_global"])
         src, dst = b.edges()
         assert np.array_equal(dst.cpu().numpy(), np.repeat(np.arange(w["n_dst"]), np.diff(w["indptr"])))
+        if b._transposed is not None:
+            check_transposed(oracle, b, w)
+
+
+def check_transposed(oracle, b, w):
+    """The transposed block that came with a sampled block: offsets equal to the oracle's transpose, the same set of
+    destination rows per source node (their order within a row is left to scheduling), every entry pointing back at
+    the edge it came from, and the longest row as it was read back with the sizes."""
+    t_ptr, t_dst, t_edge = (t.cpu().numpy() for t in b.transposed(edge_ids=True))
+    n_src, n_dst = w["n_src"], w["n_dst"]
+    w_ptr, w_idx = oracle.transpose(w["indptr"], w["src_local"], n_src)
+    assert t_ptr.size == n_src + 1 and np.array_equal(t_ptr, w_ptr)
+    assert t_dst.size == w_idx.size == t_edge.size
+    row_of = np.repeat(np.arange(n_src, dtype=np.int64), np.diff(w_ptr))
+    assert np.array_equal(np.sort(row_of * (n_dst + 1) + t_dst), np.sort(row_of * (n_dst + 1) + w_idx))
+    assert np.array_equal(np.sort(t_edge), np.arange(w["src_local"].size))
+    assert np.array_equal(w["src_local"][t_edge], row_of)
+    assert np.array_equal(np.repeat(np.arange(n_dst), np.diff(w["indptr"]))[t_edge], t_dst)
+    longest = int(np.diff(w_ptr).max()) if n_src else 0
+    reported = b.transposed()[0].fgl_longest_row
+    assert isinstance(reported, int) and reported == max(longest, 32)
+    assert np.array_equal(b.out_degrees().cpu().numpy(), np.diff(w_ptr))
 
 
 @pytest.mark.parametrize("fused", [True, False])
@@ -124,6 +146,41 @@ def test_sample_blocks_vs_oracle(cuda, oracle, small_graph, fused, fanouts, batc
         seeds = rng.permutation(indptr.size - 1)[:batch].astype(np.int32)
         got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
         check_blocks(oracle, indptr, indices, seeds, fanouts, got, 5, it * 64)
+
+
+@pytest.mark.parametrize("id_order", ["first", "arrival"])
+@pytest.mark.parametrize("which", ["inner", "all", "none"])
+def test_transposed_blocks_come_with_the_sample(cuda, oracle, small_graph, which, id_order):
+    """The fused call builds the transposed blocks itself (all, all but the outermost, or none): their offsets equal
+    the oracle's transpose, rows hold the same entries, edge ids point back, the longest row is right -- on a first
+    batch (worst-case bounds: the outermost hop counts with several counters per column), on batches sized by
+    experience, on hub seeds (rows of hundreds of entries), and for a single hop."""
+    import fastgl
+    print("sample_blocks transposed=%s id_order=%s" % (which, id_order), flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    n = indptr.size - 1
+    rng = np.random.default_rng(77)
+    hubs = np.argsort(-np.diff(indptr))[:1100].astype(np.int32)
+    for fanouts, batches in (([15, 10, 5], [rng.permutation(n)[:1100].astype(np.int32), rng.permutation(n)[:1100].astype(np.int32), hubs]),
+                             ([7], [rng.permutation(n)[:300].astype(np.int32)]),
+                             ([4, 4, 4, 4], [hubs[:64], hubs[64:128]])):
+        sampler = fastgl.FusedMapSampler(fanouts, rng_seed=3, transposed=which, id_order=id_order).set_graph(ptr, idx)
+        for it, seeds in enumerate(batches):
+            got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+            blocks = got[2]
+            have = [b._transposed is not None for b in blocks]
+            want = {"inner": [False] + [True] * (len(blocks) - 1), "all": [True] * len(blocks), "none": [False] * len(blocks)}[which]
+            assert have == want
+            if id_order == "first":
+                check_blocks(oracle, indptr, indices, seeds, fanouts, got, 3, it * 64)
+            else:  # arrival order: local ids differ from the oracle's, so the transposed blocks are checked against their own blocks
+                for b in blocks:
+                    if b._transposed is not None:
+                        check_transposed(oracle, b, dict(n_src=b.num_src_nodes(), n_dst=b.num_dst_nodes(),
+                                                         indptr=b.edge_ptr.cpu().numpy(), src_local=b.src_local.cpu().numpy()))
+            fastgl.transpose_blocks(blocks)  # builds only what is missing
+            assert all(b._transposed is not None for b in blocks)
 
 
 def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
@@ -195,12 +252,12 @@ def test_undersized_buffers_are_detected_and_redone(cuda, oracle, small_graph):
     seeds = dev_i32(hubs, cuda)
     plan = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda)
     out = fastgl.sample_blocks_fused(plan, ptr, idx, seeds, 9, 0, table_slots=1024)
-    assert out[4].tolist()[-1] & 1  # FGL_STATUS_TABLE_FULL
+    assert out[4].tolist()[2 * 3 + 1] & 1  # FGL_STATUS_TABLE_FULL (the status word follows the 2 x 3 + 1 sizes)
     tight = fastgl.BlocksPlan(indptr.size - 1, 512, [5, 10, 15], cuda, node_capacity=[512, 600, 700, 800])
     assert tight.cap_dst == [512, 600, 700] and tight.cap_uniq == 800
     out = fastgl.sample_blocks_fused(tight, ptr, idx, seeds, 9, 0)
     c = out[4].tolist()
-    assert c[-1] & 2 and c[1] <= 600 and c[2] <= 700 and c[3] <= 800  # FGL_STATUS_UNIQ_OVERFLOW, counts clamped
+    assert c[2 * 3 + 1] & 2 and c[1] <= 600 and c[2] <= 700 and c[3] <= 800  # FGL_STATUS_UNIQ_OVERFLOW, counts clamped
 
 
 @pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64)])
@@ -570,33 +627,6 @@ def test_hops_of_mixed_shapes_chain_correctly(cuda, oracle, small_graph, id_orde
             w_dst = np.repeat(np.arange(nd), np.diff(w["indptr"]))
             assert np.array_equal(np.sort((inp_h[a_dst] << 32) | inp_h[a_src]),
                                   np.sort((w_inp[w_dst].astype(np.int64) << 32) | w["src_global"].astype(np.int64)))
-
-
-def test_memory_probes_touch_what_they_say(cuda):
-    """The two diagnostic entry points behind `bench.py --workload table_access`."""
-    import fastgl
-    print("probe_table_access / probe_xcc_of_workgroups", flush=True)
-    n_ops = 100_000
-    table = torch.zeros(1 << 16, dtype=torch.int64, device=cuda)
-    fastgl.probe_table_access(table, n_ops, "whole_table", "add")
-    assert int(table.sum()) == n_ops  # one 32-bit add per lane, nothing lost
-    # a single workgroup (index 0) confined to its eighth of the table
-    table.fill_(-1)
-    fastgl.probe_table_access(table, 256, "eighth_of_own_xcd", "cas")
-    touched = torch.nonzero(table != -1).flatten()
-    assert 0 < touched.numel() <= 256 and int(touched.max()) < (1 << 16) // 8
-    assert int(table[touched].max()) < 256 and int(table[touched].min()) >= 0  # the lane index that won the slot
-    # workgroup 8 + k of the other partitioned pattern uses eighth 1
-    table.fill_(-1)
-    fastgl.probe_table_access(table, 16 * 256, "eighth_not_aligned", "cas_workgroup_scope")
-    touched = torch.nonzero(table != -1).flatten()
-    assert int(touched.max()) < 2 * ((1 << 16) // 8)
-    for op in ("load", "load_then_cas"):
-        fastgl.probe_table_access(table, n_ops, "whole_table", op, salt=3)
-    hist = fastgl.probe_xcc_of_workgroups(800, cuda).cpu()
-    assert int(hist.sum()) == 800 and hist.sum(dim=1).tolist() == [100] * 8
-    with pytest.raises(RuntimeError, match="power of two"):
-        fastgl.probe_table_access(torch.zeros(1000, dtype=torch.int64, device=cuda), 10, "whole_table", "load")
 
 
 def _csr_from_rows(rows, ptr_dtype=np.int64):
