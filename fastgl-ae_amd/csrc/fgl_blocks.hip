@@ -314,26 +314,8 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         rc = launch_fill_u32(t.words, table_slots * 2, kEmpty, s);
         if (rc != FGL_OK) return rc;
     }
-    // launch 2: counts, the later hops' tile sums, the seeds into the table, the first hop's rows and tile sums
-    {
-        const int ts0 = sample_tile_seeds(fanouts[0], n_seeds);
-        const int64_t tiles0 = sample_tile_count(n_seeds, fanouts[0]);
-        const int64_t n_later = p.tile_first[n_hops] - p.tile_first[1];
-        int64_t blocks = tiles0;
-        if (blocks < ceil_div(n_later, ts0)) blocks = ceil_div(n_later, ts0);
-        if (blocks > 8192) blocks = 8192;
-        if (blocks < 1) blocks = 1;
-        if (ts0 == 256)
-            hipLaunchKernelGGL(blocks_prepare_kernel<256>, dim3((unsigned)blocks), dim3(256), 0, s, t, d_indptr, indptr_is64, n_nodes,
-                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
-                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
-        else
-            hipLaunchKernelGGL(blocks_prepare_kernel<64>, dim3((unsigned)blocks), dim3(64), 0, s, t, d_indptr, indptr_is64, n_nodes,
-                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
-                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
-        FGL_CHECK_LAUNCH("blocks_prepare_kernel");
-    }
-
+    TransposeJob job_before;
+    memset(&job_before, 0, sizeof(job_before));
     auto make_job = [&](int h) {
         TransposeJob j;
         memset(&j, 0, sizeof(j));
@@ -356,8 +338,26 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         j.edges_max = p.cap_edges[h];
         return j;
     };
-    TransposeJob job_before;
-    memset(&job_before, 0, sizeof(job_before));
+    // launch 2: counts, the later hops' tile sums, the seeds into the table, the first hop's rows and tile sums
+    {
+        const int ts0 = sample_tile_seeds(fanouts[0], n_seeds);
+        const int64_t tiles0 = sample_tile_count(n_seeds, fanouts[0]);
+        const int64_t n_later = p.tile_first[n_hops] - p.tile_first[1];
+        int64_t blocks = tiles0;
+        if (blocks < ceil_div(n_later, ts0)) blocks = ceil_div(n_later, ts0);
+        if (blocks > 8192) blocks = 8192;
+        if (blocks < 1) blocks = 1;
+        if (ts0 == 256)
+            hipLaunchKernelGGL(blocks_prepare_kernel<256>, dim3((unsigned)blocks), dim3(256), 0, s, t, d_indptr, indptr_is64, n_nodes,
+                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+        else
+            hipLaunchKernelGGL(blocks_prepare_kernel<64>, dim3((unsigned)blocks), dim3(64), 0, s, t, d_indptr, indptr_is64, n_nodes,
+                               d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+        FGL_CHECK_LAUNCH("blocks_prepare_kernel");
+    }
+
     for (int h = 0; h < n_hops; ++h) {
         const bool last = h == n_hops - 1;
         const int32_t* hop_seeds = (h == 0) ? d_seeds : d_uniq;

@@ -31,6 +31,7 @@
 #include "fgl_kernels.hpp"
 #include "fgl_table.hpp"
 #include "fgl_transpose_job.hpp"
+#include "fgl_idmap_device.hpp"
 
 namespace fgl {
 
@@ -55,53 +56,19 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, co
     if (p == kEmpty && d_status) atomicOr(d_status, FGL_STATUS_TABLE_FULL);
 }
 
-constexpr uint32_t kHolderBit = 0x80000000u;  // slot_of[]: the edge was the first known mention of its id when its insert ran
-
-// find_or_insert for an edge's source id, which also says what the mark pass would otherwise have to read back
-// from the table: *holder = this edge became the first known mention of the id (it installed the key, or lowered
-// the key's first-edge index to its own); *displaced = the pending value it took that place from (kEmpty: none).
-// An edge that became holder and is never displaced is the id's first mention.
-__device__ __forceinline__ uint32_t insert_mention(const TableRef t, uint32_t id, uint32_t mine, uint32_t* seen_val,
-                                                   bool* holder, uint32_t* displaced)
-{
-    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
-    const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)mine << 32);
-    uint32_t p = (id * kHashMul) >> t.shift;
-    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
-    *holder = false;
-    *displaced = kEmpty;
-    for (uint32_t n = 0; n < limit; ++n) {
-        unsigned long long s = slots[p];
-        if ((uint32_t)s == kEmpty) {
-            const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
-            if (seen == ~0ull) {
-                *seen_val = mine;
-                *holder = true;
-                return p;
-            }
-            s = seen;
-        }
-        if ((uint32_t)s == id) {
-            const uint32_t v = (uint32_t)(s >> 32);
-            *seen_val = v;
-            if ((v & kPending) && v > mine) {
-                const uint32_t old = atomicMin(&t.words[2 * (size_t)p + 1], mine);
-                if (old > mine) {  // (else an even earlier mention got there between the load and the atomic)
-                    *holder = true;
-                    *displaced = old;
-                }
-            }
-            return p;
-        }
-        p = (p + 1) & t.mask;
-    }
-    return kEmpty;
-}
+// Edges per lane of the insert pass: the lane's first slot loads go out together, then the compare-and-swaps of
+// the edges that found their slot empty, then each sequence is finished (most are, by then).  Measured on the
+// 1.5 M-edge outer hop of a 111 M-node graph: 1 edge per lane 56 us, 2 -> 62 us, 4 -> 70 us -- the pass is bound
+// by the rate at which the chip retires atomics, and fewer, longer-lived waves only take parallelism away.
+#ifndef FGL_INSERT_ITEMS
+#define FGL_INSERT_ITEMS 1
+#endif
 
 // `src` and `out` may be the same array (relabelling in place): neither is __restrict__.
 // lowered (may be null; one byte per edge, zero on entry): lowered[e] is set when a later-running insert takes the
 // place of edge e as its id's first known mention.  Together with the holder bit in slot_of[] it tells the mark pass
 // which edges are first mentions without a look at the table.
+template <int ITEMS>
 __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, const int32_t* src,
                                                                   int64_t e_max, const int32_t* __restrict__ d_e,
                                                                   uint32_t* __restrict__ slot_of, int32_t* out,
@@ -110,30 +77,73 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
                                                                   const TransposeJob before)
 {
     tjob_scan<kBlock>(before);  // (the hop before, if its transposed block is being built: counters -> offsets)
+    unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
     const int64_t n_e = actual_count(e_max, d_e);
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < n_e; e += stride) {
-        // ids numbered earlier hold a local id (no pending bit) and stay as they are; a new id keeps
-        // the smallest pending edge index among the edges that mention it
-        uint32_t seen = 0, displaced = kEmpty;
-        bool holder = false;
-        const int32_t id = src[e];
-        uint32_t p = id >= 0 ? insert_mention(t, (uint32_t)id, kPending | (uint32_t)e, &seen, &holder, &displaced) : kEmpty;
-        if (p == kEmpty) {
-            // table full, or not a node id: reported; the edge's local id becomes -1 (written by the number pass)
-            if (d_status) atomicOr(d_status, id >= 0 ? FGL_STATUS_TABLE_FULL : FGL_STATUS_BAD_ID);
-        } else if (!(seen & kPending)) {
-            // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
-            // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
-            out[e] = (int32_t)seen;
-            take_rank(tr, e, (int32_t)seen);
-            p = kDone;
-        } else if (lowered != nullptr) {
-            if (holder) p |= kHolderBit;
-            // (a pending value left over from an earlier call's overflow may name an edge beyond this call's)
-            if ((displaced & kPending) && displaced != kEmpty && (int64_t)(displaced & ~kPending) < n_e) lowered[displaced & ~kPending] = 1;
+    constexpr int kEdges = kBlock * ITEMS;
+    const int64_t n_tiles = (n_e + kEdges - 1) / kEdges;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t first = tile * kEdges + threadIdx.x;
+        int32_t id[ITEMS];
+        uint32_t p[ITEMS];
+        unsigned long long s[ITEMS];
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int64_t e = first + (int64_t)j * kBlock;
+            id[j] = e < n_e ? src[e] : -1;
         }
-        slot_of[e] = p;
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            p[j] = ((uint32_t)id[j] * kHashMul) >> t.shift;
+            s[j] = id[j] >= 0 ? slots[p[j]] : 0ull;
+        }
+        // (the compare-and-swaps of the edges whose first slot is empty -- most edges of an outer hop -- are issued
+        // before any of their results is looked at)
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int64_t e = first + (int64_t)j * kBlock;
+            if (id[j] >= 0 && (uint32_t)s[j] == kEmpty) {
+                const unsigned long long fresh = (unsigned long long)(uint32_t)id[j] | ((unsigned long long)(kPending | (uint32_t)e) << 32);
+                const unsigned long long seen = atomicCAS(&slots[p[j]], ~0ull, fresh);
+                // what the slot held: still empty = this edge's key went in; (an installed slot is never empty again,
+                // so "our own key with our own pending index" tells the continuation below that the install is done)
+                s[j] = seen == ~0ull ? fresh : seen;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int64_t e = first + (int64_t)j * kBlock;
+            if (e >= n_e) continue;
+            // ids numbered earlier hold a local id (no pending bit) and stay as they are; a new id keeps
+            // the smallest pending edge index among the edges that mention it
+            const uint32_t mine = kPending | (uint32_t)e;
+            uint32_t seen = 0, displaced = kEmpty, q = kEmpty;
+            bool holder = false;
+            if (id[j] >= 0) {
+                if (s[j] == ((unsigned long long)(uint32_t)id[j] | ((unsigned long long)mine << 32))) {
+                    // installed by the compare-and-swap above (no other edge carries this pending index)
+                    q = p[j];
+                    seen = mine;
+                    holder = true;
+                } else {
+                    q = insert_mention_from(t, (uint32_t)id[j], mine, p[j], s[j], &seen, &holder, &displaced);
+                }
+            }
+            if (q == kEmpty) {
+                // table full, or not a node id: reported; the edge's local id becomes -1 (written by the number pass)
+                if (d_status) atomicOr(d_status, id[j] >= 0 ? FGL_STATUS_TABLE_FULL : FGL_STATUS_BAD_ID);
+            } else if (!(seen & kPending)) {
+                // numbered in an earlier hop (or a destination node): the edge is relabelled right here and
+                // takes no further part (`out` may be `src`: this lane is the only one that touches entry e)
+                out[e] = (int32_t)seen;
+                take_rank(tr, e, (int32_t)seen);
+                q = kDone;
+            } else if (lowered != nullptr) {
+                if (holder) q |= kHolderBit;
+                // (a pending value left over from an earlier call's overflow may name an edge beyond this call's)
+                if ((displaced & kPending) && displaced != kEmpty && (int64_t)(displaced & ~kPending) < n_e) lowered[displaced & ~kPending] = 1;
+            }
+            slot_of[e] = q;
+        }
     }
 }
 
@@ -257,37 +267,6 @@ constexpr int kSelfTilesPerLane = 8;
 #define FGL_NUMBER_SELF_MAX_BLOCKS 1024
 #endif
 constexpr int kIdmapSelfPrefixTiles = kBlock * kSelfTilesPerLane;
-
-// A node that has just been given a position in the unique list is a seed of the next hop: its row start and
-// degree go to that position (store_next_hop), and its min(fanout, degree) to the next hop's per-tile edge counts.
-// The two graph offsets are read by load_row_of, which callers issue early -- for every edge that may turn out to
-// be a first mention -- so that the reads overlap the pass's own chain of loads.  An id outside the graph is
-// marked for the next hop's sampling kernel to report.
-__device__ __forceinline__ void load_row_of(const NextHop& next, int32_t id, int64_t* a, int64_t* deg)
-{
-    *a = kRowBadId;
-    *deg = 0;
-    if (id >= 0 && (int64_t)id < next.n_nodes) {
-        if (next.is64) {
-            const int64_t* p = static_cast<const int64_t*>(next.indptr);
-            *a = p[id];
-            *deg = p[id + 1] - *a;
-        } else {
-            const int32_t* p = static_cast<const int32_t*>(next.indptr);
-            *a = p[id];
-            *deg = (int64_t)p[id + 1] - *a;
-        }
-        if (*deg < 0) *deg = 0;
-        if (*deg > 0x7FFFFFFF) *deg = 0x7FFFFFFF;
-    }
-}
-
-__device__ __forceinline__ int store_next_hop(const NextHop& next, int64_t local, int64_t a, int64_t deg)
-{
-    next.row_start[local] = a;
-    next.deg[local] = (int32_t)deg;
-    return deg < next.fanout ? (int)deg : next.fanout;
-}
 
 // The new nodes that the lanes of a wave number in one step have consecutive positions (a position is a count of
 // earlier new nodes, and the lanes hold consecutive edges), so their tiles of the next hop are at most two:
@@ -717,7 +696,12 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
 
     // (the holder bit shares a word with the slot index: tables of 2^31 slots go without the bookkeeping)
     uint8_t* lowered = slots <= ((int64_t)1 << 30) ? d_lowered : nullptr;
-    hipLaunchKernelGGL(idmap_insert_src_kernel, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+    // (small inputs need the workgroups more than the edges in flight per lane)
+    if (n_edges_max > kArrivalSmallEdges)
+        hipLaunchKernelGGL(idmap_insert_src_kernel<FGL_INSERT_ITEMS>, dim3(stride_grid(n_edges_max, kBlock * FGL_INSERT_ITEMS) + scan_blocks),
+                           dim3(kBlock), 0, stream, t, d_src_in, n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job);
+    else
+    hipLaunchKernelGGL(idmap_insert_src_kernel<1>, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
                        n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,

@@ -70,7 +70,7 @@ struct TransposeRank {
     int64_t cols_max;
     int split;
 };
-inline TransposeRank rank_of(const TransposeJob* j)
+__host__ __device__ inline TransposeRank rank_of(const TransposeJob* j)
 {
     return j && j->cnt ? TransposeRank{j->cnt, j->rank, j->cols_max, j->split} : TransposeRank{nullptr, nullptr, 0, 1};
 }

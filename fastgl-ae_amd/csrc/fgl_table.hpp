@@ -51,14 +51,15 @@ constexpr uint32_t kMaxProbes = 4096;
 // load is enough for the first look: a stale "empty" is settled by the 64-bit CAS, which
 // installs key and val in one atomic, and a stale val can only cause a redundant atomicMin.
 // *seen_val receives the val found with the key (val_if_new if this call installed the key).
-__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new, uint32_t* seen_val)
+// (The sequence is entered at slot p with that slot's value `s` already in hand -- loaded, or returned by a failed
+// compare-and-swap -- so that a caller can put the first loads of several keys in flight before walking any further.)
+__device__ __forceinline__ uint32_t find_or_insert_from(const TableRef t, uint32_t id, uint32_t val_if_new, uint32_t p,
+                                                        unsigned long long s, uint32_t* seen_val)
 {
     unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
     const unsigned long long fresh = (unsigned long long)id | ((unsigned long long)val_if_new << 32);
-    uint32_t p = (id * kHashMul) >> t.shift;
     const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
     for (uint32_t n = 0; n < limit; ++n) {
-        unsigned long long s = slots[p];
         if ((uint32_t)s == kEmpty) {
             const unsigned long long seen = atomicCAS(&slots[p], ~0ull, fresh);
             if (seen == ~0ull) {
@@ -73,8 +74,15 @@ __device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id
             return p;
         }
         p = (p + 1) & t.mask;
+        s = slots[p];
     }
     return kEmpty;
+}
+
+__device__ __forceinline__ uint32_t find_or_insert(const TableRef t, uint32_t id, uint32_t val_if_new, uint32_t* seen_val)
+{
+    const uint32_t p = (id * kHashMul) >> t.shift;
+    return find_or_insert_from(t, id, val_if_new, p, reinterpret_cast<unsigned long long*>(t.words)[p], seen_val);
 }
 
 // Finds the slot of `id` without inserting.  kEmpty if absent.

@@ -134,7 +134,9 @@ def test_sample_blocks_golden(cuda, oracle, fused):
 
 
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64), ([3], 1), ([64, 2], 300)])
+@pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64), ([3], 1), ([64, 2], 300),
+                                           # batches of 8192 and more seeds with small and mid fanouts (a third mini-batch is all hubs)
+                                           ([3, 16], 8192), ([3, 17], 500), ([2, 8], 8192), ([2, 5], 8193), ([4, 1], 1)])
 def test_sample_blocks_vs_oracle(cuda, oracle, small_graph, fused, fanouts, batch):
     import fastgl
     print("sample_blocks %s batch=%d fused=%s" % (fanouts, batch, fused), flush=True)
@@ -142,8 +144,9 @@ def test_sample_blocks_vs_oracle(cuda, oracle, small_graph, fused, fanouts, batc
     ptr, idx = load_graph(cuda, indptr, indices)
     sampler = fastgl.FusedMapSampler(fanouts, fused=fused, rng_seed=5).set_graph(ptr, idx)
     rng = np.random.default_rng(batch)
-    for it in range(2):  # the second mini-batch uses the next Philox streams and a reused table
-        seeds = rng.permutation(indptr.size - 1)[:batch].astype(np.int32)
+    hubs = np.argsort(-np.diff(indptr))
+    for it in range(3):  # the later mini-batches use the next Philox streams and a reused table; the last is all hubs
+        seeds = (rng.permutation(indptr.size - 1)[:batch] if it < 2 else hubs[:batch]).astype(np.int32)
         got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
         check_blocks(oracle, indptr, indices, seeds, fanouts, got, 5, it * 64)
 
