@@ -13,8 +13,13 @@
 #include <c10/hip/HIPGuard.h>
 
 #include <atomic>
+#include <map>
+#include <mutex>
 #include <string>
+#include <utility>
 #include <vector>
+
+#include <hip/hip_runtime_api.h>
 
 #include "fastgl_hip.h"
 
@@ -66,6 +71,55 @@ void manual_seed(uint64_t seed)
 {
     g_rng_seed = seed;
     g_rng_calls = 0;
+}
+
+// What sample_node and transfer_edge_id keep between calls, per (device, stream): the reference allocates, fills and
+// frees its hash table and scratch on every call (id_map.cu:45-59,408-409; sample.cu:118,151,157) and reads its sizes
+// back through pageable memory.  Here the table persists and is left empty by each call's last pass (so no call pays
+// for a fill once the largest table has been seen), the scratch persists, and the two words that the host needs --
+// a size and the status -- come back through one pinned buffer.
+struct CallState {
+    torch::Tensor table;      // int64 slots; grows to the largest table asked for
+    int64_t empty_slots = 0;  // slots [0, empty_slots) hold the empty marker (0: nothing is known)
+    torch::Tensor ws;         // uint8 scratch, grows on demand
+    torch::Tensor meta;       // device int32[2]: {size, status}; the status word is zero between calls
+    torch::Tensor host;       // pinned int32[2]
+};
+
+CallState& call_state(const torch::Tensor& like)
+{
+    static std::mutex mu;
+    static std::map<std::pair<int, void*>, CallState> states;
+    const int dev = like.get_device();
+    void* stream = c10::hip::getCurrentHIPStream(dev).stream();
+    std::lock_guard<std::mutex> lock(mu);
+    CallState& st = states[{dev, stream}];
+    if (!st.meta.defined()) {
+        st.meta = torch::zeros({2}, like.options().dtype(torch::kInt32));
+        st.host = torch::empty({2}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
+    }
+    return st;
+}
+
+void* grown(torch::Tensor& buf, size_t bytes, const torch::Tensor& like)
+{
+    if (!buf.defined() || (size_t)buf.numel() < bytes)
+        buf = torch::empty({(int64_t)std::max<size_t>(bytes, (size_t)1 << 20)}, like.options().dtype(torch::kUInt8));
+    return buf.data_ptr();
+}
+
+// {size, status} of the call that has just been enqueued: one 8-byte copy into pinned memory, one wait.  A non-zero
+// status word is cleared again (the kernels only ever or into it).
+std::pair<int64_t, uint32_t> read_back(CallState& st, void* stream)
+{
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    TORCH_CHECK(hipMemcpyAsync(st.host.data_ptr(), st.meta.data_ptr(), 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s) == hipSuccess,
+                "fastgl: the size read-back could not be enqueued");
+    TORCH_CHECK(hipStreamSynchronize(s) == hipSuccess, "fastgl: waiting for the size read-back failed");
+    const int32_t* h = st.host.data_ptr<int32_t>();
+    const std::pair<int64_t, uint32_t> out{h[0], (uint32_t)h[1]};
+    if (out.second != 0) st.meta.zero_();
+    return out;
 }
 
 int dtype_of(const torch::Tensor& t) { return t.scalar_type() == torch::kFloat32 ? FGL_F32 : FGL_BF16; }
@@ -134,17 +188,19 @@ std::vector<torch::Tensor> sample_node(torch::Tensor src_edges, torch::Tensor ds
     const int64_t cap = std::max<int64_t>((int64_t)dst_nodes * neighbor_num, 1);
     auto src_out = torch::empty({cap}, opt), dst_out = torch::empty({cap}, opt);
     auto block_ptr = torch::empty({n_seeds + 1}, opt);
-    auto meta = torch::zeros({2}, opt);  // [edge count, status]
-    auto ws = scratch(fgl_sample_workspace_bytes(n_seeds, neighbor_num), seed_nodes);
+    CallState& st = call_state(seed_nodes);
+    const size_t ws_bytes = fgl_sample_workspace_bytes(n_seeds, neighbor_num);
+    void* ws = grown(st.ws, ws_bytes, seed_nodes);
+    void* stream = stream_of(seed_nodes);
+    int32_t* meta = st.meta.data_ptr<int32_t>();
     ok(fgl_sample_node(edge_ptr.data_ptr(), edge_ptr.scalar_type() == torch::kInt64, src_edges.data_ptr<int32_t>(),
                        edge_ptr.size(0) - 1, seed_nodes.data_ptr<int32_t>(), n_seeds, nullptr, neighbor_num, g_rng_seed.load(),
                        g_rng_calls.fetch_add(1), src_out.data_ptr<int32_t>(), dst_out.data_ptr<int32_t>(), block_ptr.data_ptr<int32_t>(),
-                       meta.data_ptr<int32_t>(), reinterpret_cast<uint32_t*>(meta.data_ptr<int32_t>()) + 1, ws.data_ptr(),
-                       (size_t)ws.numel(), stream_of(seed_nodes)));
-    auto host = meta.cpu();  // the read-back of sample.cu:202
-    const int64_t n_edges = host.data_ptr<int32_t>()[0];
-    raise_status((uint32_t)host.data_ptr<int32_t>()[1], "sample_node");
-    return {src_out.slice(0, 0, n_edges), dst_out.slice(0, 0, n_edges), meta.slice(0, 0, 1)};
+                       meta, reinterpret_cast<uint32_t*>(meta) + 1, ws, (size_t)st.ws.numel(), stream));
+    const auto back = read_back(st, stream);  // the read-back of sample.cu:202
+    raise_status(back.second, "sample_node");
+    // (the edge count as a device tensor, as the reference returns it: the last entry of the block's row pointer)
+    return {src_out.slice(0, 0, back.first), dst_out.slice(0, 0, back.first), block_ptr.slice(0, n_seeds, n_seeds + 1)};
 }
 
 // aggregate_acc.cpp:467-489 (id_map.cu:386-493): in-place relabelling; uniq = cat(dst_edges_unique, new source ids
@@ -164,22 +220,35 @@ std::vector<torch::Tensor> transfer_edge_id(torch::Tensor src_edges, torch::Tens
     const int64_t capacity = n_dst + max_new;
     const int64_t slots = fgl_idmap_slots(capacity);
     auto opt = src_edges.options();
-    auto table = torch::empty({slots}, opt.dtype(torch::kInt64));
     auto uniq = torch::empty({std::max<int64_t>(capacity, 1)}, opt);
-    auto meta = torch::zeros({2}, opt);  // [node total, status]
-    auto ws = scratch(fgl_idmap_map_src_workspace_bytes(n_edges), src_edges);
-    void* st = stream_of(src_edges);
-    uint32_t* status = reinterpret_cast<uint32_t*>(meta.data_ptr<int32_t>()) + 1;
-    ok(fgl_idmap_reset(table.data_ptr(), slots, st));
-    ok(fgl_idmap_insert_dst(table.data_ptr(), slots, dst_edges_unique.data_ptr<int32_t>(), n_dst, nullptr, uniq.data_ptr<int32_t>(),
-                            status, st));
-    ok(fgl_idmap_map_src(table.data_ptr(), slots, src_edges.data_ptr<int32_t>(), src_edges.data_ptr<int32_t>(), n_edges, nullptr,
-                         n_dst, nullptr, meta.data_ptr<int32_t>(), uniq.data_ptr<int32_t>(), capacity, FGL_IDMAP_ORDERED, status,
-                         ws.data_ptr(), (size_t)ws.numel(), st));
-    ok(fgl_idmap_lookup(table.data_ptr(), slots, dst_edges.data_ptr<int32_t>(), n_edges, nullptr, status, st));
-    auto host = meta.cpu();  // the read-back of id_map.cu:454,491
-    raise_status((uint32_t)host.data_ptr<int32_t>()[1], "transfer_edge_id");
-    return {src_edges, dst_edges, uniq.slice(0, 0, host.data_ptr<int32_t>()[0])};
+    CallState& st = call_state(src_edges);
+    void* stream = stream_of(src_edges);
+    if (!st.table.defined() || st.table.numel() < slots) {
+        st.table = torch::empty({slots}, opt.dtype(torch::kInt64));
+        st.empty_slots = 0;
+    }
+    void* table = st.table.data_ptr();
+    // the table is a prefix of the persistent buffer; whatever part of it is not known to be empty is filled now
+    // (in the steady state of a training loop: never)
+    if (st.empty_slots < slots) ok(fgl_idmap_reset(table, slots, stream));
+    const int64_t known_empty = std::max(st.empty_slots, slots);
+    st.empty_slots = 0;  // (until the call's last pass has been enqueued)
+    const size_t ws_bytes = fgl_idmap_map_src_workspace_bytes(n_edges);
+    void* ws = grown(st.ws, ws_bytes, src_edges);
+    int32_t* meta = st.meta.data_ptr<int32_t>();
+    uint32_t* status = reinterpret_cast<uint32_t*>(meta) + 1;
+    ok(fgl_idmap_insert_dst(table, slots, dst_edges_unique.data_ptr<int32_t>(), n_dst, nullptr, uniq.data_ptr<int32_t>(), status, stream));
+    // the destination half first (its ids are all in the table by now) ...
+    ok(fgl_idmap_lookup(table, slots, dst_edges.data_ptr<int32_t>(), n_edges, nullptr, status, stream));
+    // ... then the source half, whose last pass neither writes the new ids' numbers back into the table (nobody
+    // will look them up: the next call brings its own destination list) nor leaves anything in it
+    ok(fgl_idmap_map_src(table, slots, src_edges.data_ptr<int32_t>(), src_edges.data_ptr<int32_t>(), n_edges, nullptr, n_dst, nullptr,
+                         meta, uniq.data_ptr<int32_t>(), capacity, FGL_IDMAP_ORDERED | FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY, status,
+                         ws, (size_t)st.ws.numel(), stream));
+    st.empty_slots = known_empty;
+    const auto back = read_back(st, stream);  // the read-back of id_map.cu:454,491
+    raise_status(back.second, "transfer_edge_id");
+    return {src_edges, dst_edges, uniq.slice(0, 0, back.first)};
 }
 
 // aggregate_acc.cpp:522-529 (utilis.cu:43-79)

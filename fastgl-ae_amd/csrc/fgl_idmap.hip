@@ -777,9 +777,11 @@ FGL_EXPORT int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_
                                  int32_t* d_n_total_out, int32_t* d_uniq, int64_t uniq_capacity, int flags,
                                  uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream)
 {
+    const bool leave_empty = (flags & FGL_IDMAP_LEAVE_TABLE_EMPTY) != 0;
+    FGL_REQUIRE(!leave_empty || (flags & FGL_IDMAP_FINAL), "idmap_map_src: FGL_IDMAP_LEAVE_TABLE_EMPTY needs FGL_IDMAP_FINAL");
     return launch_idmap_map_src(d_table, slots, d_src_in, d_src_out, n_edges_max, d_n_edges, n_base, d_n_base,
-                                d_n_total_out, d_uniq, uniq_capacity, flags, d_status, d_ws, ws_bytes, as_stream(stream), false,
-                                nullptr, false, nullptr, nullptr, nullptr);
+                                d_n_total_out, d_uniq, uniq_capacity, flags & ~FGL_IDMAP_LEAVE_TABLE_EMPTY, d_status, d_ws, ws_bytes,
+                                as_stream(stream), false, nullptr, leave_empty, nullptr, nullptr, nullptr);
 }
 
 FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,

@@ -122,20 +122,29 @@ def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_it
     capacity = n_dst + max_new
     slots = lib.fgl_idmap_slots(capacity)
     with torch.cuda.device(dev):
-        table = _table(slots, dev)
+        st = L.stream_handle()
+        key = (torch.device(dev).index, st)
+        table, known_empty = _table(slots, dev)
         uniq = torch.empty(max(capacity, 1), dtype=torch.int32, device=dev)
         meta = torch.zeros(2, dtype=torch.int32, device=dev)  # [n_total, status]
         ws_bytes = lib.fgl_idmap_map_src_workspace_bytes(n_edges)
         ws = L.workspace(ws_bytes, dev)
-        st = L.stream_handle()
         status_ptr = meta.data_ptr() + 4
-        L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+        # the table is a prefix of a persistent buffer that every call leaves empty: only slots that no call has
+        # emptied yet are filled here (in the steady state of a training loop: none)
+        if known_empty < slots:
+            L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
+        _tables[key] = (table, 0)
         L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dst_edges_unique), n_dst, None, L.ptr(uniq),
                                          status_ptr, st))
-        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(src_edges), L.ptr(src_edges), n_edges, None, n_dst,
-                                      None, meta.data_ptr(), L.ptr(uniq), capacity, L.IDMAP_ORDERED, status_ptr,
-                                      L.ptr(ws), ws.numel(), st))
+        # the destination half first (its ids are all in the table by now), then the source half, whose last pass
+        # writes nothing back into the table (no later call looks these ids up) and empties it
         L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(dst_edges), n_edges, None, status_ptr, st))
+        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(src_edges), L.ptr(src_edges), n_edges, None, n_dst,
+                                      None, meta.data_ptr(), L.ptr(uniq), capacity,
+                                      L.IDMAP_ORDERED | L.IDMAP_FINAL | L.IDMAP_LEAVE_TABLE_EMPTY, status_ptr,
+                                      L.ptr(ws), ws.numel(), st))
+        _tables[key] = (table, max(known_empty, slots))
         n_total, status = meta.tolist()  # host read-back, as id_map.cu:454,491
     _raise_status(status, "transfer_edge_id")
     return [src_edges, dst_edges, uniq[:n_total]]
@@ -144,15 +153,16 @@ def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_it
 _tables = {}
 
 
-def _table(slots: int, dev) -> torch.Tensor:
+def _table(slots: int, dev):
     """Hash-table storage, cached per (device, stream) and grown on demand (the reference
-    cudaMallocs, memsets and cudaFrees one per call, id_map.cu:45-59)."""
+    cudaMallocs, memsets and cudaFrees one per call, id_map.cu:45-59), with the number of its leading slots
+    that are known to hold the empty marker."""
     key = (torch.device(dev).index, L.stream_handle())
-    t = _tables.get(key)
+    t, known_empty = _tables.get(key, (None, 0))
     if t is None or t.numel() < slots:
-        t = torch.empty(int(slots), dtype=torch.int64, device=dev)
-        _tables[key] = t
-    return t
+        t, known_empty = torch.empty(int(slots), dtype=torch.int64, device=dev), 0
+        _tables[key] = (t, 0)
+    return t, known_empty
 
 
 def cal_deg(edges, nodes_num):

@@ -75,6 +75,9 @@ enum fgl_zero_policy {
                                tenth faster; the order of the new ids depends on scheduling */
 #define FGL_IDMAP_FINAL 2   /* (or'ed in) the table is not consulted after this call: the local ids of the
                                new ids go to the edges and the unique list, not back into the table */
+#define FGL_IDMAP_LEAVE_TABLE_EMPTY 8 /* (or'ed in, with FGL_IDMAP_FINAL only) the call's last pass, which no longer reads
+                               the table, stores the empty marker over all `slots` of it: the next call on the same slots
+                               needs no fgl_idmap_reset (same value and meaning as FGL_BLOCKS_LEAVE_TABLE_EMPTY) */
 /* fgl_sample_blocks only, or'ed into idmap_flags: */
 #define FGL_BLOCKS_TABLE_EMPTY 4       /* the caller vouches that every slot of the table is empty (as fgl_idmap_reset
                                           leaves it, or an earlier fgl_sample_blocks call with FGL_BLOCKS_LEAVE_TABLE_EMPTY
@@ -159,7 +162,8 @@ int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids,
  * n_base ids are already numbered (host value n_base, or *d_n_base when non-NULL).
  * New ids get n_base, n_base+1, ... and are appended to d_uniq -- in order of first
  * occurrence in d_src_in (flags = FGL_IDMAP_ORDERED) or of arrival (FGL_IDMAP_ARRIVAL), either
- * optionally or'ed with FGL_IDMAP_FINAL when no later call will look these ids up in the table;
+ * optionally or'ed with FGL_IDMAP_FINAL when no later call will look these ids up in the table (and then also
+ * with FGL_IDMAP_LEAVE_TABLE_EMPTY);
  * d_src_out[e] = local id of d_src_in[e] (may alias d_src_in);
  * *d_n_total_out = n_base + number of new ids (must not alias d_n_base).
  * n_base + n_edges_max must stay below 2^31 - 2. */
