@@ -83,7 +83,7 @@ struct CallState {
     int64_t empty_slots = 0;  // slots [0, empty_slots) hold the empty marker (0: nothing is known)
     torch::Tensor ws;         // uint8 scratch, grows on demand
     torch::Tensor meta;       // device int32[2]: {size, status}; the status word is zero between calls
-    torch::Tensor host;       // pinned int32[2]
+    torch::Tensor host;       // pinned int32[2] that the kernels write themselves: {size, status} of the call at hand
 };
 
 CallState& call_state(const torch::Tensor& like)
@@ -108,15 +108,14 @@ void* grown(torch::Tensor& buf, size_t bytes, const torch::Tensor& like)
     return buf.data_ptr();
 }
 
-// {size, status} of the call that has just been enqueued: one 8-byte copy into pinned memory, one wait.  A non-zero
-// status word is cleared again (the kernels only ever or into it).
+// {size, status} of the call that has just been enqueued.  The call's own launches wrote both words into the pinned
+// buffer (device-writable host memory), so there is no copy to enqueue: wait for the stream, read.  A non-zero
+// status word is cleared on the device again (the kernels only ever or into it).
+// (Polling hipStreamQuery instead of the blocking wait was measured: 0.34 -> 0.40 ms per three-hop mini-batch.)
 std::pair<int64_t, uint32_t> read_back(CallState& st, void* stream)
 {
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    TORCH_CHECK(hipMemcpyAsync(st.host.data_ptr(), st.meta.data_ptr(), 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s) == hipSuccess,
-                "fastgl: the size read-back could not be enqueued");
-    TORCH_CHECK(hipStreamSynchronize(s) == hipSuccess, "fastgl: waiting for the size read-back failed");
-    const int32_t* h = st.host.data_ptr<int32_t>();
+    TORCH_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)) == hipSuccess, "fastgl: waiting for the call's sizes failed");
+    const volatile int32_t* h = st.host.data_ptr<int32_t>();
     const std::pair<int64_t, uint32_t> out{h[0], (uint32_t)h[1]};
     if (out.second != 0) st.meta.zero_();
     return out;
@@ -196,7 +195,7 @@ std::vector<torch::Tensor> sample_node(torch::Tensor src_edges, torch::Tensor ds
     ok(fgl_sample_node(edge_ptr.data_ptr(), edge_ptr.scalar_type() == torch::kInt64, src_edges.data_ptr<int32_t>(),
                        edge_ptr.size(0) - 1, seed_nodes.data_ptr<int32_t>(), n_seeds, nullptr, neighbor_num, g_rng_seed.load(),
                        g_rng_calls.fetch_add(1), src_out.data_ptr<int32_t>(), dst_out.data_ptr<int32_t>(), block_ptr.data_ptr<int32_t>(),
-                       meta, reinterpret_cast<uint32_t*>(meta) + 1, ws, (size_t)st.ws.numel(), stream));
+                       meta, reinterpret_cast<uint32_t*>(meta) + 1, st.host.data_ptr<int32_t>(), ws, (size_t)st.ws.numel(), stream));
     const auto back = read_back(st, stream);  // the read-back of sample.cu:202
     raise_status(back.second, "sample_node");
     // (the edge count as a device tensor, as the reference returns it: the last entry of the block's row pointer)
@@ -237,14 +236,14 @@ std::vector<torch::Tensor> transfer_edge_id(torch::Tensor src_edges, torch::Tens
     void* ws = grown(st.ws, ws_bytes, src_edges);
     int32_t* meta = st.meta.data_ptr<int32_t>();
     uint32_t* status = reinterpret_cast<uint32_t*>(meta) + 1;
-    ok(fgl_idmap_insert_dst(table, slots, dst_edges_unique.data_ptr<int32_t>(), n_dst, nullptr, uniq.data_ptr<int32_t>(), status, stream));
-    // the destination half first (its ids are all in the table by now) ...
-    ok(fgl_idmap_lookup(table, slots, dst_edges.data_ptr<int32_t>(), n_edges, nullptr, status, stream));
-    // ... then the source half, whose last pass neither writes the new ids' numbers back into the table (nobody
-    // will look them up: the next call brings its own destination list) nor leaves anything in it
-    ok(fgl_idmap_map_src(table, slots, src_edges.data_ptr<int32_t>(), src_edges.data_ptr<int32_t>(), n_edges, nullptr, n_dst, nullptr,
-                         meta, uniq.data_ptr<int32_t>(), capacity, FGL_IDMAP_ORDERED | FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY, status,
-                         ws, (size_t)st.ws.numel(), stream));
+    TORCH_CHECK(n_edges == 0 || src_edges.data_ptr() != dst_edges.data_ptr(), "src_edges and dst_edges must be distinct tensors");
+    // destination ids in, then three passes over the edges (the destination half rides on the first); the last pass
+    // neither writes the new ids' numbers back into the table (nobody will look them up: the next call brings its
+    // own destination list) nor leaves anything in it
+    ok(fgl_idmap_transfer(table, slots, dst_edges_unique.data_ptr<int32_t>(), n_dst, src_edges.data_ptr<int32_t>(),
+                          dst_edges.data_ptr<int32_t>(), n_edges, uniq.data_ptr<int32_t>(), capacity,
+                          FGL_IDMAP_ORDERED | FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY, meta, status, st.host.data_ptr<int32_t>(), ws,
+                          (size_t)st.ws.numel(), stream));
     st.empty_slots = known_empty;
     const auto back = read_back(st, stream);  // the read-back of id_map.cu:454,491
     raise_status(back.second, "transfer_edge_id");

@@ -40,10 +40,13 @@ constexpr int kTile = kBlock * kItems;
 
 __global__ __launch_bounds__(kBlock) void idmap_insert_dst_kernel(TableRef t, const int32_t* __restrict__ ids,
                                                                   int64_t n_max, const int32_t* __restrict__ d_n,
-                                                                  int32_t* __restrict__ uniq, uint32_t* __restrict__ d_status)
+                                                                  int32_t* __restrict__ uniq, uint32_t* __restrict__ d_status,
+                                                                  uint32_t* __restrict__ zero_words, int64_t n_zero_words)
 {
     const int64_t n = actual_count(n_max, d_n);
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    // (scratch of the passes that follow in the same call, cleared on the way)
+    for (int64_t w = i; w < n_zero_words; w += (int64_t)gridDim.x * kBlock) zero_words[w] = 0u;
     if (i >= n) return;
     const int32_t id = ids[i];
     if (uniq != nullptr && uniq != ids) uniq[i] = id;
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
                                                                   uint32_t* __restrict__ slot_of, int32_t* out,
                                                                   uint8_t* __restrict__ lowered,
                                                                   uint32_t* __restrict__ d_status, const TransposeRank tr,
-                                                                  const TransposeJob before)
+                                                                  const TransposeJob before, int32_t* dst_inout)
 {
     tjob_scan<kBlock>(before);  // (the hop before, if its transposed block is being built: counters -> offsets)
     unsigned long long* slots = reinterpret_cast<unsigned long long*>(t.words);
@@ -95,6 +98,35 @@ __global__ __launch_bounds__(kBlock) void idmap_insert_src_kernel(TableRef t, co
         for (int j = 0; j < ITEMS; ++j) {
             p[j] = ((uint32_t)id[j] * kHashMul) >> t.shift;
             s[j] = id[j] >= 0 ? slots[p[j]] : 0ull;
+        }
+        // The destination half of transfer_edge_id (id_map.cu:377-381) rides on this pass when the caller asks: the
+        // edge's destination id -- numbered by an earlier launch -- is looked up and relabelled in place, its first
+        // probe travelling together with the source id's.
+        if (dst_inout != nullptr) {
+#pragma unroll
+            for (int j = 0; j < ITEMS; ++j) {
+                const int64_t e = first + (int64_t)j * kBlock;
+                if (e >= n_e) continue;
+                const uint32_t d = (uint32_t)dst_inout[e];
+                int32_t local = -1;
+                if ((int32_t)d >= 0) {
+                    uint32_t q = (d * kHashMul) >> t.shift;
+                    const uint32_t limit = t.mask < kMaxProbes ? t.mask + 1 : kMaxProbes;
+                    for (uint32_t n = 0; n < limit; ++n) {
+                        const unsigned long long v = slots[q];
+                        if ((uint32_t)v == d) {
+                            // (a destination id holds its number; one that only an edge of this call has mentioned
+                            // so far -- pending -- is not a destination: missing)
+                            if (!((uint32_t)(v >> 32) & kPending)) local = (int32_t)(v >> 32);
+                            break;
+                        }
+                        if ((uint32_t)v == kEmpty) break;
+                        q = (q + 1) & t.mask;
+                    }
+                }
+                if (local < 0 && d_status) atomicOr(d_status, FGL_STATUS_MISSING_KEY);
+                dst_inout[e] = local;
+            }
         }
         // (the compare-and-swaps of the edges whose first slot is empty -- most edges of an outer hop -- are issued
         // before any of their results is looked at)
@@ -225,14 +257,22 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
 
 // n_total = n_base + (number of new ids), clamped to the capacity of the unique list.
 __device__ __forceinline__ void publish_node_total(int64_t n_base, int n_new, int64_t capacity,
-                                                   int32_t* __restrict__ d_n_total_out, uint32_t* __restrict__ d_status)
+                                                   int32_t* __restrict__ d_n_total_out, uint32_t* __restrict__ d_status,
+                                                   int32_t* __restrict__ readback = nullptr)
 {
     int64_t total = n_base + (int64_t)n_new;
+    uint32_t overflow = 0u;
     if (total > capacity) {
+        overflow = FGL_STATUS_UNIQ_OVERFLOW;
         if (d_status) atomicOr(d_status, FGL_STATUS_UNIQ_OVERFLOW);
         total = capacity;
     }
     if (d_n_total_out) *d_n_total_out = (int32_t)total;
+    if (readback) {
+        // {node total, status word}: every other bit of the status word was set by an earlier launch of the call
+        readback[0] = (int32_t)total;
+        readback[1] = (int32_t)((d_status ? *d_status : 0u) | overflow);
+    }
 }
 
 // One workgroup: exclusive scan of the per-tile counts of new ids, then
@@ -242,7 +282,7 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
                                                                     const int32_t* __restrict__ d_e, int64_t n_base_h,
                                                                     const int32_t* __restrict__ d_n_base, int64_t capacity,
                                                                     int32_t* __restrict__ d_n_total_out,
-                                                                    uint32_t* __restrict__ d_status)
+                                                                    uint32_t* __restrict__ d_status, int32_t* __restrict__ readback)
 {
     __shared__ int smem[1024 / kWave + 1];
     const int n_tiles = (int)tiles_of(actual_count(e_max, d_e));
@@ -256,7 +296,7 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
         carry += total;
     }
     if (threadIdx.x == 0)
-        publish_node_total(d_n_base ? (int64_t)(*d_n_base) : n_base_h, carry, capacity, d_n_total_out, d_status);
+        publish_node_total(d_n_base ? (int64_t)(*d_n_base) : n_base_h, carry, capacity, d_n_total_out, d_status, readback);
 }
 
 // Up to this many tiles the number pass scans the tile counts itself (every workgroup, into LDS) and
@@ -316,7 +356,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                                                               int32_t* __restrict__ d_n_total_out,
                                                               uint32_t* __restrict__ d_status, const NextHop next,
                                                               uint32_t* __restrict__ clear_words, int64_t n_clear_words,
-                                                              const TransposeRank tr)
+                                                              const TransposeRank tr, int32_t* __restrict__ readback)
 {
     __shared__ int s_prefix[SELF ? kIdmapSelfPrefixTiles : 1];
     __shared__ int smem[kBlock / kWave + 1];
@@ -353,7 +393,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
             run += v[j];
         }
         __syncthreads();
-        if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status);
+        if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status, readback);
     }
     // the last pass of a mini-batch, which no longer reads the table, can leave it empty for the next one
     // (first, so that the stores drain while the edges are being numbered)
@@ -552,7 +592,7 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
                                                                        int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                        int64_t capacity, int32_t* __restrict__ d_n_total_out,
                                                                        uint32_t* __restrict__ d_status, const TransposeRank tr,
-                                                                       const TransposeJob before)
+                                                                       const TransposeJob before, int32_t* __restrict__ readback)
 {
     tjob_fill<kBlock>(before);  // (the hop before, if its transposed block is being built: entries into their rows)
     const int64_t n_e = actual_count(e_max, d_e);
@@ -567,7 +607,7 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-        publish_node_total(n_base, *counter, capacity, d_n_total_out, d_status);
+        publish_node_total(n_base, *counter, capacity, d_n_total_out, d_status, readback);
     }
 }
 
@@ -592,16 +632,20 @@ int launch_idmap_reset(void* d_table, int64_t slots, hipStream_t stream)
 }
 
 int launch_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids, int64_t n_max, const int32_t* d_n,
-                            int32_t* d_uniq, uint32_t* d_status, hipStream_t stream)
+                            int32_t* d_uniq, uint32_t* d_status, hipStream_t stream, uint32_t* d_zero_words, int64_t n_zero_words)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE(n_max >= 0 && n_max <= slots / 2, "idmap_insert_dst: %lld ids do not fit %lld slots at load 1/2", (long long)n_max, (long long)slots);
     FGL_REQUIRE(n_max <= 0x7FFFFFFF, "idmap_insert_dst: too many ids");
-    if (n_max == 0) return FGL_OK;
-    FGL_REQUIRE(d_dst_ids != nullptr, "idmap_insert_dst: null ids");
-    const int64_t blocks = ceil_div(n_max, kBlock);
+    if (d_zero_words == nullptr) n_zero_words = 0;
+    if (n_max == 0 && n_zero_words == 0) return FGL_OK;
+    FGL_REQUIRE(n_max == 0 || d_dst_ids != nullptr, "idmap_insert_dst: null ids");
+    int64_t blocks = ceil_div(n_max, kBlock);
+    const int64_t zero_blocks = ceil_div(n_zero_words, (int64_t)kBlock * 16) < 2048 ? ceil_div(n_zero_words, (int64_t)kBlock * 16) : 2048;
+    if (blocks < zero_blocks) blocks = zero_blocks;
+    if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(idmap_insert_dst_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, make_ref(d_table, slots),
-                       d_dst_ids, n_max, d_n, d_uniq, d_status);
+                       d_dst_ids, n_max, d_n, d_uniq, d_status, d_zero_words, n_zero_words);
     FGL_CHECK_LAUNCH("idmap_insert_dst_kernel");
     return FGL_OK;
 }
@@ -616,6 +660,7 @@ size_t idmap_map_src_workspace_bytes(int64_t n_edges_max)
     c.take<uint16_t>((size_t)tiles * kBlock);   // before8
     c.take<int32_t>((size_t)tiles);             // tile sums
     c.take<int32_t>((size_t)tiles);             // tile prefix
+    c.take<uint32_t>((size_t)(n_edges_max + 3) / 4);  // one byte per edge ("displaced as first mention"), used by fgl_idmap_transfer
     return c.used();
 }
 
@@ -624,7 +669,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          int32_t* d_uniq, int64_t uniq_capacity, int flags, uint32_t* d_status, void* d_ws,
                          size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed, const NextHop* next_hop,
                          bool leave_table_empty, uint8_t* d_lowered, const TransposeJob* rank_job,
-                         const TransposeJob* before_job)
+                         const TransposeJob* before_job, int32_t* d_dst_inout, int32_t* d_readback)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
@@ -667,6 +712,10 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     FGL_REQUIRE(!leave_table_empty || final_call, "idmap_map_src: only a final call can leave the table empty");
 
     if (flags & FGL_IDMAP_ARRIVAL) {
+        if (d_dst_inout != nullptr && n_edges_max > 0) {  // (this numbering's passes do not carry the destination half: a launch of its own)
+            hipLaunchKernelGGL(idmap_lookup_kernel, dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_dst_inout, n_edges_max, d_n_edges, d_status);
+            FGL_CHECK_LAUNCH("idmap_lookup_kernel");
+        }
         // the counter of new ids: *d_n_total_out itself when the caller vouches that it holds zero (the all-hops
         // entry point zeroes its counts when it resets the table), else one int of the (otherwise unused)
         // tile-sum array, zeroed by a launch of its own
@@ -687,7 +736,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                                d_status, next, tr, scan_job);
         FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
         hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, tr, fill_job);
+                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, tr, fill_job, d_readback);
         FGL_CHECK_LAUNCH("idmap_relabel_publish_kernel");
         // (the second pass reads the table, so emptying it takes a launch of its own here)
         if (leave_table_empty) return launch_fill_u32(t.words, slots * 2, kEmpty, stream);
@@ -699,18 +748,19 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     // (small inputs need the workgroups more than the edges in flight per lane)
     if (n_edges_max > kArrivalSmallEdges)
         hipLaunchKernelGGL(idmap_insert_src_kernel<FGL_INSERT_ITEMS>, dim3(stride_grid(n_edges_max, kBlock * FGL_INSERT_ITEMS) + scan_blocks),
-                           dim3(kBlock), 0, stream, t, d_src_in, n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job);
+                           dim3(kBlock), 0, stream, t, d_src_in, n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job,
+                           d_dst_inout);
     else
-    hipLaunchKernelGGL(idmap_insert_src_kernel<1>, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
-                       n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job);
+        hipLaunchKernelGGL(idmap_insert_src_kernel<1>, dim3(edge_blocks + scan_blocks), dim3(kBlock), 0, stream, t, d_src_in,
+                           n_edges_max, d_n_edges, slot_of, d_src_out, lowered, d_status, tr, scan_job, d_dst_inout);
     FGL_CHECK_LAUNCH("idmap_insert_src_kernel");
     hipLaunchKernelGGL(idmap_mark_kernel, dim3(tile_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
                        slot_of, lowered, first_of, flags8, before8, sums, fill_job);
     FGL_CHECK_LAUNCH("idmap_mark_kernel");
-#define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS)                                                              \
+#define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS, READBACK)                                                              \
     hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
-                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words, tr)
+                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words, tr, READBACK)
     // emptying the table rides on the last pass: enough workgroups for a fill of that size
     uint32_t* clear_words = leave_table_empty ? t.words : nullptr;
     const int64_t n_clear_words = leave_table_empty ? slots * 2 : 0;
@@ -722,14 +772,14 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     // compute unit, each looping over several tiles of edges, instead of one per 256 edges
     if (tiles <= kIdmapSelfPrefixTiles && edge_blocks > FGL_NUMBER_SELF_MAX_BLOCKS) edge_blocks = FGL_NUMBER_SELF_MAX_BLOCKS;
     if (tiles <= kIdmapSelfPrefixTiles) {
-        if (final_call) FGL_LAUNCH_NUMBER(true, false, nullptr, d_n_total_out, d_status);
-        else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status);
+        if (final_call) FGL_LAUNCH_NUMBER(true, false, nullptr, d_n_total_out, d_status, d_readback);
+        else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status, d_readback);
     } else {
         hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max,
-                           d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status);
+                           d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, d_readback);
         FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
-        if (final_call) FGL_LAUNCH_NUMBER(false, false, prefix, nullptr, nullptr);
-        else FGL_LAUNCH_NUMBER(false, true, prefix, nullptr, nullptr);
+        if (final_call) FGL_LAUNCH_NUMBER(false, false, prefix, nullptr, nullptr, nullptr);
+        else FGL_LAUNCH_NUMBER(false, true, prefix, nullptr, nullptr, nullptr);
     }
 #undef FGL_LAUNCH_NUMBER
     FGL_CHECK_LAUNCH("idmap_number_kernel");
@@ -767,7 +817,7 @@ FGL_EXPORT int fgl_idmap_reset(void* d_table, int64_t slots, void* stream) { ret
 FGL_EXPORT int fgl_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids, int64_t n_max,
                                     const int32_t* d_n, int32_t* d_uniq, uint32_t* d_status, void* stream)
 {
-    return launch_idmap_insert_dst(d_table, slots, d_dst_ids, n_max, d_n, d_uniq, d_status, as_stream(stream));
+    return launch_idmap_insert_dst(d_table, slots, d_dst_ids, n_max, d_n, d_uniq, d_status, as_stream(stream), nullptr, 0);
 }
 
 FGL_EXPORT size_t fgl_idmap_map_src_workspace_bytes(int64_t n_edges_max) { return idmap_map_src_workspace_bytes(n_edges_max < 0 ? 0 : n_edges_max); }
@@ -781,7 +831,41 @@ FGL_EXPORT int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_
     FGL_REQUIRE(!leave_empty || (flags & FGL_IDMAP_FINAL), "idmap_map_src: FGL_IDMAP_LEAVE_TABLE_EMPTY needs FGL_IDMAP_FINAL");
     return launch_idmap_map_src(d_table, slots, d_src_in, d_src_out, n_edges_max, d_n_edges, n_base, d_n_base,
                                 d_n_total_out, d_uniq, uniq_capacity, flags & ~FGL_IDMAP_LEAVE_TABLE_EMPTY, d_status, d_ws, ws_bytes,
-                                as_stream(stream), false, nullptr, leave_empty, nullptr, nullptr, nullptr);
+                                as_stream(stream), false, nullptr, leave_empty, nullptr, nullptr, nullptr, nullptr);
+}
+
+FGL_EXPORT int fgl_idmap_transfer(void* d_table, int64_t slots, const int32_t* d_dst_unique, int64_t n_dst,
+                                  int32_t* d_src_edges, int32_t* d_dst_edges, int64_t n_edges, int32_t* d_uniq,
+                                  int64_t uniq_capacity, int flags, int32_t* d_n_total_out, uint32_t* d_status,
+                                  int32_t* d_readback, void* d_ws, size_t ws_bytes, void* stream)
+{
+    FGL_REQUIRE(n_dst >= 0 && n_edges >= 0, "idmap_transfer: negative size");
+    FGL_REQUIRE(n_edges == 0 || (d_src_edges && d_dst_edges), "idmap_transfer: null edge array");
+    FGL_REQUIRE(d_src_edges == nullptr || d_src_edges != d_dst_edges, "idmap_transfer: the two edge arrays must be distinct");
+    FGL_REQUIRE(d_uniq != nullptr && uniq_capacity >= n_dst, "idmap_transfer: the unique list cannot hold the destination ids");
+    const bool leave_empty = (flags & FGL_IDMAP_LEAVE_TABLE_EMPTY) != 0;
+    FGL_REQUIRE(!leave_empty || (flags & FGL_IDMAP_FINAL), "idmap_transfer: FGL_IDMAP_LEAVE_TABLE_EMPTY needs FGL_IDMAP_FINAL");
+    if (d_ws == nullptr || ws_bytes < idmap_map_src_workspace_bytes(n_edges)) {
+        set_error("idmap_transfer: workspace too small (%zu < %zu)", ws_bytes, idmap_map_src_workspace_bytes(n_edges));
+        return FGL_ERR_WORKSPACE;
+    }
+    // the last piece of the workspace: one byte per edge that lets the mark pass skip most of its table reads;
+    // cleared by the launch that inserts the destination ids
+    const int64_t tiles = ceil_div(n_edges > 0 ? n_edges : 1, kTile);
+    Carver c(d_ws);
+    c.take<uint32_t>((size_t)n_edges);
+    c.take<uint32_t>((size_t)n_edges);
+    c.take<uint8_t>((size_t)tiles * kBlock);
+    c.take<uint16_t>((size_t)tiles * kBlock);
+    c.take<int32_t>((size_t)tiles);
+    c.take<int32_t>((size_t)tiles);
+    uint32_t* lowered_words = c.take<uint32_t>((size_t)(n_edges + 3) / 4);
+    int rc = launch_idmap_insert_dst(d_table, slots, d_dst_unique, n_dst, nullptr, d_uniq, d_status, as_stream(stream), lowered_words,
+                                     (n_edges + 3) / 4);
+    if (rc != FGL_OK) return rc;
+    return launch_idmap_map_src(d_table, slots, d_src_edges, d_src_edges, n_edges, nullptr, n_dst, nullptr, d_n_total_out, d_uniq,
+                                uniq_capacity, flags & ~FGL_IDMAP_LEAVE_TABLE_EMPTY, d_status, d_ws, ws_bytes, as_stream(stream), false,
+                                nullptr, leave_empty, reinterpret_cast<uint8_t*>(lowered_words), nullptr, nullptr, d_dst_edges, d_readback);
 }
 
 FGL_EXPORT int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t n_max, const int32_t* d_n,

@@ -13,7 +13,7 @@ int launch_exclusive_sum(const int32_t* d_in, int64_t n_max, const int32_t* d_n,
 // scan to the tiles the actual count occupies
 int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_prefix, int32_t* total_a,
                        int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n, int tile_items,
-                       hipStream_t stream);
+                       hipStream_t stream, int32_t* readback = nullptr, const uint32_t* d_status = nullptr);
 int launch_fill_u32(uint32_t* p, int64_t n, uint32_t value, hipStream_t stream);
 
 // Row start of a node whose id lies outside the graph / whose insert found the table full: how a launch that
@@ -92,18 +92,20 @@ int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_
                         int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
                         hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next,
                         uint8_t* d_zero_per_edge = nullptr,   // (optional) one byte per output edge, cleared along with the writes
-                        const TransposeSteps* steps = nullptr);  // (optional) zero this hop's counters, tile sums of the hop before
+                        const TransposeSteps* steps = nullptr,   // (optional) zero this hop's counters, tile sums of the hop before
+                        int32_t* d_readback = nullptr);          // (optional) {edge count, status word} once both are final; may be host memory
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                   int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws, size_t ws_bytes,
-                  hipStream_t stream, const uint32_t* d_stream_add = nullptr);
+                  hipStream_t stream, const uint32_t* d_stream_add = nullptr, int32_t* d_readback = nullptr);
 
 // id-map (fgl_idmap.hip)
 size_t idmap_map_src_workspace_bytes(int64_t n_edges_max);
 int launch_idmap_reset(void* d_table, int64_t slots, hipStream_t stream);
 int launch_idmap_insert_dst(void* d_table, int64_t slots, const int32_t* d_dst_ids, int64_t n_max,
-                            const int32_t* d_n, int32_t* d_uniq, uint32_t* d_status, hipStream_t stream);
+                            const int32_t* d_n, int32_t* d_uniq, uint32_t* d_status, hipStream_t stream,
+                            uint32_t* d_zero_words, int64_t n_zero_words);  // (optional) scratch words to clear on the way
 int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int32_t* d_src_out,
                          int64_t n_edges_max, const int32_t* d_n_edges, int64_t n_base, const int32_t* d_n_base,
                          int32_t* d_n_total_out, int32_t* d_uniq, int64_t uniq_capacity, int flags,
@@ -113,7 +115,9 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          bool leave_table_empty,          // final calls only: every slot of the table is empty when the call's work is done
                          uint8_t* d_lowered,              // (may be null) n_edges_max bytes, zero on entry: lets the mark pass skip most table reads
                          const TransposeJob* rank_job = nullptr,     // (may be null) the edges take their ranks in this block's transposed rows
-                         const TransposeJob* before_job = nullptr);  // (may be null) scan and fill steps of the hop before, carried by the first two passes
+                         const TransposeJob* before_job = nullptr,   // (may be null) scan and fill steps of the hop before, carried by the first two passes
+                         int32_t* d_dst_inout = nullptr,             // (may be null) n_edges_max ids that are in the table already: relabelled in place by the first pass
+                         int32_t* d_readback = nullptr);             // (may be null) {node total, status word} once both are final; may be host memory
 
 // deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
 size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);

@@ -106,24 +106,34 @@ __global__ __launch_bounds__(TS) void sample_degree_kernel(const void* __restric
 template <int TS>
 __device__ __forceinline__ int tile_base(int lane_sum_of_earlier_tiles, const int32_t* __restrict__ tile_prefix, int64_t tile,
                                          int64_t n_tiles, int64_t n, int tile_total, int* smem,
-                                         int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+                                         int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
+                                         int32_t* __restrict__ readback, const uint32_t* __restrict__ d_status)
 {
     if (tile_prefix) return tile_prefix[tile];
     const int base = block_sum_of_lanes<TS>(lane_sum_of_earlier_tiles, smem);
     if (tile == n_tiles - 1 && threadIdx.x == 0) {
         block_ptr[n] = base + tile_total;
         if (n_edges_out) *n_edges_out = base + tile_total;
+        if (readback) {  // (nothing in a launch that is handed a read-back pointer sets status bits: they are final)
+            readback[0] = base + tile_total;
+            readback[1] = d_status ? (int32_t)*d_status : 0;
+        }
     }
     return base;
 }
 
 // The launch for zero seeds still has to publish the (empty) totals when no scan launch does.
 __device__ __forceinline__ void publish_empty(const int32_t* __restrict__ tile_prefix, int64_t n_tiles,
-                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out)
+                                              int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
+                                              int32_t* __restrict__ readback, const uint32_t* __restrict__ d_status)
 {
     if (tile_prefix == nullptr && n_tiles == 0 && blockIdx.x == 0 && threadIdx.x == 0) {
         block_ptr[0] = 0;
         if (n_edges_out) *n_edges_out = 0;
+        if (readback) {
+            readback[0] = 0;
+            readback[1] = d_status ? (int32_t)*d_status : 0;
+        }
     }
 }
 
@@ -169,7 +179,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
                                                           int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
                                                           uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
                                                           int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge,
-                                                          const TransposeSteps steps)
+                                                          const TransposeSteps steps, int32_t* __restrict__ readback)
 {
     extern __shared__ uint32_t s_sel[];  // [fanout][TS] picked positions
     __shared__ int s_scan[TS / kWave + 1];
@@ -185,7 +195,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
     tjob_tile_sums<TS>(steps.before);
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
-    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
+    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out, readback, d_status);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i = tile * TS + tid;
         int deg = 0, seed = 0;
@@ -201,7 +211,7 @@ __global__ __launch_bounds__(TS) void sample_edges_kernel(const int32_t* __restr
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
+        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out, readback, d_status);
         s_off[tid] = ex;
         if (tid == 0) s_off[TS] = total;
         s_row[tid] = row;
@@ -278,7 +288,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
                                                               int32_t* __restrict__ block_ptr, int32_t* __restrict__ n_edges_out,
                                                               uint32_t* __restrict__ d_status, int next_fanout, int next_tile_seeds,
                                                               int32_t* __restrict__ next_tile_sums, uint8_t* __restrict__ zero_per_edge,
-                                                              const TransposeSteps steps)
+                                                              const TransposeSteps steps, int32_t* __restrict__ readback)
 {
     extern __shared__ int32_t s_stage[];  // [TS*fanout] sampled ids (+ [TS*fanout] seed ids when dst_out is wanted)
     __shared__ int s_scan[TS / kWave + 1];
@@ -292,7 +302,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
     tjob_tile_sums<TS>(steps.before);
     const int64_t n = actual_count(n_max, d_n);
     const int64_t n_tiles = (n + TS - 1) / TS;
-    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out);
+    publish_empty(tile_prefix, n_tiles, block_ptr, n_edges_out, readback, d_status);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t i = tile * TS + tid;
         int deg = 0, seed = 0;
@@ -308,7 +318,7 @@ __global__ __launch_bounds__(TS) void sample_edges_reg_kernel(const int32_t* __r
         const int k = deg < fanout ? deg : fanout;
         int total;
         const int ex = block_exclusive_scan<TS>(k, s_scan, &total);
-        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out);
+        const int base = tile_base<TS>(sum_before, tile_prefix, tile, n_tiles, n, total, s_scan, block_ptr, n_edges_out, readback, d_status);
         if (i < n) block_ptr[i] = base + ex;
 
         uint32_t sel[F];
@@ -383,7 +393,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
                            uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                            int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, hipStream_t stream,
                            const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge,
-                           const TransposeSteps* steps_in)
+                           const TransposeSteps* steps_in, int32_t* d_readback)
 {
     const int64_t tiles = ceil_div(n_seeds_max > 0 ? n_seeds_max : 1, TS);
     unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
@@ -408,7 +418,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
     // publishes the totals), which saves the scan launch in between
     if (tiles > kSampleSelfPrefixTiles) {
         int rc = launch_tile_prefix(sums, (int)tiles, prefix, d_n_edges_out, nullptr, d_block_ptr, n_seeds_max, d_n_seeds,
-                                    TS, stream);
+                                    TS, stream, d_readback, d_status);
         if (rc != FGL_OK) return rc;
     } else {
         prefix = nullptr;
@@ -424,7 +434,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
     hipLaunchKernelGGL((sample_edges_reg_kernel<TS, F>), dim3(grid), dim3(TS), lds_reg, stream, d_indices, d_seeds,   \
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,                   \
                        (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, \
-                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps)
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps, d_readback)
         if (fanout <= 8) FGL_LAUNCH_REG(8);
         else if (fanout <= 16) FGL_LAUNCH_REG(16);
         else FGL_LAUNCH_REG(32);
@@ -436,7 +446,7 @@ static int launch_edges_ts(const int32_t* d_indices, const int32_t* d_seeds, int
     hipLaunchKernelGGL((sample_edges_kernel<TS, 16>), dim3(grid), dim3(TS), lds, stream, d_indices, d_seeds,
                        n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, (uint32_t)rng_seed,
                        (uint32_t)(rng_seed >> 32), stream_id, d_stream_add, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out,
-                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps);
+                       d_status, next_fanout, next_ts, next_sums, d_zero_per_edge, steps, d_readback);
     FGL_CHECK_LAUNCH("sample_edges_kernel");
     return FGL_OK;
 }
@@ -446,22 +456,22 @@ int launch_sample_edges(const int32_t* d_indices, const int32_t* d_seeds, int64_
                         int32_t* tile_prefix, uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out,
                         int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status,
                         hipStream_t stream, const uint32_t* d_stream_add, const NextHop* next, uint8_t* d_zero_per_edge,
-                        const TransposeSteps* steps)
+                        const TransposeSteps* steps, int32_t* d_readback)
 {
     if (sample_tile_seeds(fanout, n_seeds_max) == 256)
         return launch_edges_ts<256>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
                                     rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
-                                    d_stream_add, next, d_zero_per_edge, steps);
+                                    d_stream_add, next, d_zero_per_edge, steps, d_readback);
     return launch_edges_ts<64>(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, tile_sums, tile_prefix,
                                rng_seed, stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream,
-                               d_stream_add, next, d_zero_per_edge, steps);
+                               d_stream_add, next, d_zero_per_edge, steps, d_readback);
 }
 
 int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                   const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                   uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
                   int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws, size_t ws_bytes,
-                  hipStream_t stream, const uint32_t* d_stream_add)
+                  hipStream_t stream, const uint32_t* d_stream_add, int32_t* d_readback)
 {
     FGL_REQUIRE(n_seeds_max >= 0 && n_nodes >= 0, "sample_node: negative size");
     FGL_REQUIRE(fanout >= 1 && fanout <= FGL_MAX_FANOUT, "sample_node: fanout %d outside [1, %d]", fanout, FGL_MAX_FANOUT);
@@ -490,7 +500,7 @@ int launch_sample(const void* d_indptr, int indptr_is64, const int32_t* d_indice
     FGL_CHECK_LAUNCH("sample_degree_kernel");
     return launch_sample_edges(d_indices, d_seeds, n_seeds_max, d_n_seeds, fanout, row_start, deg, sums, prefix, rng_seed,
                                stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, stream, d_stream_add,
-                               nullptr, nullptr);
+                               nullptr, nullptr, nullptr, d_readback);
 }
 
 }  // namespace fgl
@@ -506,12 +516,12 @@ FGL_EXPORT size_t fgl_sample_workspace_bytes(int64_t n_seeds_max, int fanout)
 FGL_EXPORT int fgl_sample_node(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,
                                const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                                uint64_t rng_seed, uint32_t stream_id, int32_t* d_src_out, int32_t* d_dst_out,
-                               int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, void* d_ws,
-                               size_t ws_bytes, void* stream)
+                               int32_t* d_block_ptr, int32_t* d_n_edges_out, uint32_t* d_status, int32_t* d_readback,
+                               void* d_ws, size_t ws_bytes, void* stream)
 {
     return launch_sample(d_indptr, indptr_is64, d_indices, n_nodes, d_seeds, n_seeds_max, d_n_seeds, fanout, rng_seed,
                          stream_id, d_src_out, d_dst_out, d_block_ptr, d_n_edges_out, d_status, d_ws, ws_bytes,
-                         as_stream(stream));
+                         as_stream(stream), nullptr, d_readback);
 }
 
 FGL_EXPORT int fgl_sample_node_static(const void* d_indptr, int indptr_is64, const int32_t* d_indices, int64_t n_nodes,

@@ -47,7 +47,9 @@ __global__ __launch_bounds__(1024) void scan_tile_prefix_kernel(const int32_t* _
                                                                 int32_t* __restrict__ total_a,
                                                                 int32_t* __restrict__ total_b,
                                                                 int32_t* __restrict__ at_count_base, int64_t n_max,
-                                                                const int32_t* __restrict__ d_n, int tile_items)
+                                                                const int32_t* __restrict__ d_n, int tile_items,
+                                                                int32_t* __restrict__ readback,
+                                                                const uint32_t* __restrict__ d_status)
 {
     __shared__ int smem[1024 / kWave + 1];
     if (tile_items > 0) {
@@ -67,15 +69,19 @@ __global__ __launch_bounds__(1024) void scan_tile_prefix_kernel(const int32_t* _
         if (total_a) *total_a = carry;
         if (total_b) *total_b = carry;
         if (at_count_base) at_count_base[actual_count(n_max, d_n)] = carry;
+        if (readback) {  // {total, status word as it stands}: see fgl_sample_node's d_readback
+            readback[0] = carry;
+            readback[1] = d_status ? (int32_t)*d_status : 0;
+        }
     }
 }
 
 int launch_tile_prefix(const int32_t* tile_sums, int n_tiles, int32_t* tile_prefix, int32_t* total_a,
                        int32_t* total_b, int32_t* at_count_base, int64_t n_max, const int32_t* d_n, int tile_items,
-                       hipStream_t stream)
+                       hipStream_t stream, int32_t* readback, const uint32_t* d_status)
 {
     hipLaunchKernelGGL(scan_tile_prefix_kernel, dim3(1), dim3(1024), 0, stream, tile_sums, n_tiles, tile_prefix,
-                       total_a, total_b, at_count_base, n_max, d_n, tile_items);
+                       total_a, total_b, at_count_base, n_max, d_n, tile_items, readback, d_status);
     FGL_CHECK_LAUNCH("scan_tile_prefix_kernel");
     return FGL_OK;
 }

@@ -37,7 +37,7 @@ SIGNATURES = {
     "fgl_exclusive_sum_i32": (_i32, [_vp, _i64, _vp, _vp, _vp, _sz, _vp]),
     "fgl_cal_deg": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp]),
     "fgl_sample_workspace_bytes": (_sz, [_i64, _i32]),
-    "fgl_sample_node": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fgl_sample_node": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_sample_node_static": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _u64, _u32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "fgl_table_size": (_i64, [_i64, _i32]),
     "fgl_idmap_slots": (_i64, [_i64]),
@@ -46,6 +46,7 @@ SIGNATURES = {
     "fgl_idmap_insert_dst": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp]),
     "fgl_idmap_map_src_workspace_bytes": (_sz, [_i64]),
     "fgl_idmap_map_src": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _sz, _vp]),
+    "fgl_idmap_transfer": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]),
     "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _vp, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp,

@@ -88,7 +88,7 @@ def sample_node(src_edges, dst_edges, edge_ptr, seed_nodes, dst_nodes, neighbor_
         L.check(lib.fgl_sample_node(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(src_edges),
                                     int(edge_ptr.size(0)) - 1, L.ptr(seed_nodes), n_seeds, None, fanout,
                                     _rng_state["seed"], stream_id, L.ptr(src_out), L.ptr(dst_out), L.ptr(block_ptr),
-                                    meta.data_ptr(), meta.data_ptr() + 4, L.ptr(ws), ws.numel(), L.stream_handle()))
+                                    meta.data_ptr(), meta.data_ptr() + 4, None, L.ptr(ws), ws.numel(), L.stream_handle()))
         n_edges, status = meta.tolist()  # the host read-back the reference also does (sample.cu:202)
     _raise_status(status, "sample_node")
     edges_num = meta[:1]
@@ -135,15 +135,12 @@ def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_it
         if known_empty < slots:
             L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
         _tables[key] = (table, 0)
-        L.check(lib.fgl_idmap_insert_dst(L.ptr(table), slots, L.ptr(dst_edges_unique), n_dst, None, L.ptr(uniq),
-                                         status_ptr, st))
-        # the destination half first (its ids are all in the table by now), then the source half, whose last pass
+        # destination ids in, then three passes over the edges (the destination half rides on the first); the last
         # writes nothing back into the table (no later call looks these ids up) and empties it
-        L.check(lib.fgl_idmap_lookup(L.ptr(table), slots, L.ptr(dst_edges), n_edges, None, status_ptr, st))
-        L.check(lib.fgl_idmap_map_src(L.ptr(table), slots, L.ptr(src_edges), L.ptr(src_edges), n_edges, None, n_dst,
-                                      None, meta.data_ptr(), L.ptr(uniq), capacity,
-                                      L.IDMAP_ORDERED | L.IDMAP_FINAL | L.IDMAP_LEAVE_TABLE_EMPTY, status_ptr,
-                                      L.ptr(ws), ws.numel(), st))
+        L.check(lib.fgl_idmap_transfer(L.ptr(table), slots, L.ptr(dst_edges_unique), n_dst, L.ptr(src_edges), L.ptr(dst_edges),
+                                       n_edges, L.ptr(uniq), capacity,
+                                       L.IDMAP_ORDERED | L.IDMAP_FINAL | L.IDMAP_LEAVE_TABLE_EMPTY, meta.data_ptr(), status_ptr,
+                                       None, L.ptr(ws), ws.numel(), st))
         _tables[key] = (table, max(known_empty, slots))
         n_total, status = meta.tolist()  # host read-back, as id_map.cu:454,491
     _raise_status(status, "transfer_edge_id")

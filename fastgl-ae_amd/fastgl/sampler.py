@@ -219,6 +219,7 @@ class FusedMapSampler:
         self.output_nodes = None
         self._states = {}       # shape of a mini-batch -> _ShapeState
         self._side = None        # second stream of iter_batches
+        self._pinned_counts = None  # host buffer of the per-batch size read-back
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
         self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
@@ -343,7 +344,7 @@ class FusedMapSampler:
         if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and pending["caps"] is not None:
             state.nodes_seen = None
             pending = self._launch_fused(pending["seeds"], pending["stream_base"], worst_case=True, state=state)
-            c = pending["out"][4].tolist()
+            c = self._read_counts(pending["out"][4])
             status = c[2 * H + 1]
         if status:
             ops._raise_status(status, "sample_blocks")
@@ -386,9 +387,17 @@ class FusedMapSampler:
         self.batches += 1
         return PendingBatch(self, self._launch_fused(seeds, stream_base))
 
+    def _read_counts(self, counts):
+        """The batch's sizes on the host: one copy into a pinned buffer that the sampler keeps, one wait."""
+        if self._pinned_counts is None or self._pinned_counts.numel() != counts.numel():
+            self._pinned_counts = torch.empty(counts.numel(), dtype=torch.int32, pin_memory=True)
+        self._pinned_counts.copy_(counts, non_blocking=True)
+        torch.cuda.current_stream(counts.device).synchronize()
+        return self._pinned_counts.tolist()
+
     def _sample_fused(self, seeds, stream_base):
         pending = self._launch_fused(seeds, stream_base)
-        return self._finish_fused(pending, pending["out"][4].tolist())  # the one host synchronisation of the mini-batch
+        return self._finish_fused(pending, self._read_counts(pending["out"][4]))  # the one host synchronisation of the mini-batch
 
     def _side_stream(self, dev):
         if self._side is None:

@@ -113,6 +113,10 @@ int fgl_cal_deg(const int32_t* d_ids, int64_t n_ids_max, const int32_t* d_n_ids,
  * replacement (Floyd) from Philox4x32-10 keyed by (rng_seed, stream_id, s): what a node
  * draws does not depend on its position in the seed list.
  * d_n_edges_out (optional) receives the edge count as int32.
+ * d_readback (optional): two int32 that the call writes once both are final -- {edge count, status word} -- for a
+ * caller that must know the size at once (as the reference's operator does, sample.cu:202).  It may point to
+ * pinned host memory that the device can write (hipHostMalloc): the caller then only waits for the stream and reads
+ * the two words, with no copy to enqueue behind the kernels.
  * d_src_out / d_dst_out need room for n_seeds_max * fanout entries.
  * ------------------------------------------------------------------------------- */
 size_t fgl_sample_workspace_bytes(int64_t n_seeds_max, int fanout);
@@ -120,7 +124,7 @@ int fgl_sample_node(const void* d_indptr, int indptr_is64, const int32_t* d_indi
                     const int32_t* d_seeds, int64_t n_seeds_max, const int32_t* d_n_seeds, int fanout,
                     uint64_t rng_seed, uint32_t stream_id,
                     int32_t* d_src_out, int32_t* d_dst_out, int32_t* d_block_ptr, int32_t* d_n_edges_out,
-                    uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream);
+                    uint32_t* d_status, int32_t* d_readback, void* d_ws, size_t ws_bytes, void* stream);
 
 /* sample_node without a workspace argument.  Has no counterpart in the reference; it is for callers
  * that cannot allocate device memory at the point of the call (code under HIP graph capture, tight
@@ -173,6 +177,22 @@ int fgl_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, int
                       int64_t n_base, const int32_t* d_n_base, int32_t* d_n_total_out,
                       int32_t* d_uniq, int64_t uniq_capacity, int flags,
                       uint32_t* d_status, void* d_ws, size_t ws_bytes, void* stream);
+
+/* transfer_edge_id -- the whole device part of fastgl.transfer_edge_id (aggregate_acc.cpp:467-489,
+ * id_map.cu:386-493) on a table that holds nothing: the destination ids get the local ids 0..n_dst-1 and go to
+ * d_uniq[0..n_dst); d_src_edges and d_dst_edges (n_edges global ids each, distinct arrays) are relabelled in place;
+ * new source ids are numbered from n_dst on and appended to d_uniq; *d_n_total_out = n_dst + their number.
+ * A destination id of an edge that is not in d_dst_unique becomes -1 and sets FGL_STATUS_MISSING_KEY.
+ * Four launches with first-occurrence numbering (the destination half rides on the first pass over the
+ * edges), against the reference's table allocation, fill and four kernels per call.  flags and workspace
+ * (fgl_idmap_map_src_workspace_bytes(n_edges)) as for fgl_idmap_map_src; a caller that keeps the table between
+ * calls passes FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY and never fills it again.
+ * d_readback (optional): {node total, status word}, written once both are final; may be device-writable pinned host
+ * memory, as for fgl_sample_node (the reference reads the same size back at id_map.cu:454,491). */
+int fgl_idmap_transfer(void* d_table, int64_t slots, const int32_t* d_dst_unique, int64_t n_dst,
+                       int32_t* d_src_edges, int32_t* d_dst_edges, int64_t n_edges, int32_t* d_uniq,
+                       int64_t uniq_capacity, int flags, int32_t* d_n_total_out, uint32_t* d_status,
+                       int32_t* d_readback, void* d_ws, size_t ws_bytes, void* stream);
 
 /* relabel ids that are already in the table, in place (the dst half of
  * transfer_edge_id_kernel, id_map.cu:377-381).  A missing id becomes -1 and sets

@@ -77,7 +77,7 @@ def test_argument_errors_are_reported_not_launched():
     fan = (C.c_int32 * 1)(0)
     assert lib.fgl_sample_blocks_plan(10, 10, fan, 1, None, 0, None, None, None, None, None) == 1
     assert b"fanout" in lib.fgl_last_error()
-    assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, 0, None) == 1
+    assert lib.fgl_sample_node(None, 1, None, 10, None, 5, None, 500, 0, 0, None, None, None, None, None, None, None, 0, None) == 1
     assert lib.fgl_idmap_reset(None, 100, None) == 1      # not a power of two / null table
     assert lib.fgl_aggregate(None, None, 4, None, None, 8, 8, 7, 0, 0, None, None, None, 1, None, -1, None, -1, None, 8, None) == 1
     assert b"dtype" in lib.fgl_last_error()
@@ -196,7 +196,7 @@ def test_size_limits_are_stated_before_anything_is_launched():
     lib = fastgl.lib()
     fake = C.c_void_p(0x1000)  # never dereferenced: every call below fails its size checks first
     # seeds x fanout beyond int32 edge offsets
-    assert lib.fgl_sample_node(fake, 1, fake, 10, fake, 20_000_000, None, 192, 0, 0, fake, None, fake, None, None, fake, 1 << 40, None) == 1
+    assert lib.fgl_sample_node(fake, 1, fake, 10, fake, 20_000_000, None, 192, 0, 0, fake, None, fake, None, None, None, fake, 1 << 40, None) == 1
     assert b"overflows int32" in lib.fgl_last_error()
     # a hop of the all-hops plan that could produce more than 2^31 edges
     fan = (C.c_int32 * 2)(192, 192)

@@ -118,3 +118,57 @@ def test_sample_chi_square_on_device(cuda):
     expect = n * fanout / deg
     stat = ((counts - expect) ** 2 / expect).sum() * (deg - 1) / (deg - fanout)
     assert stats.chi2.sf(stat, deg - 1) > 1e-4
+
+
+@pytest.mark.parametrize("where", ["pinned_host", "device"])
+def test_sizes_written_where_the_caller_reads_them(cuda, small_graph, where):
+    """d_readback of fgl_sample_node / fgl_idmap_transfer: {size, status word}, written by the call's own launches --
+    into pinned host memory (no copy to enqueue: wait, read) or into device memory.  With and without a status bit;
+    zero seeds; more than a million seeds (the size then comes from the scan launch)."""
+    from fastgl import _lib as L
+    lib = L.lib()
+    print("read-back pair in %s memory" % where, flush=True)
+    indptr, indices = small_graph
+    ptr, idx = torch.from_numpy(indptr).to(cuda), dev_i32(indices, cuda)
+    n_nodes = indptr.size - 1
+    rb = torch.full((2,), -7, dtype=torch.int32, pin_memory=True) if where == "pinned_host" else torch.full((2,), -7, dtype=torch.int32, device=cuda)
+    st = L.stream_handle()
+    rng = np.random.default_rng(9)
+    for n_seeds, fanout, bad in ((3000, 7, False), (3000, 7, True), (0, 5, False), (1_100_000, 2, False)):
+        seeds = rng.integers(0, n_nodes, size=n_seeds).astype(np.int32)
+        if bad:
+            seeds[17] = n_nodes + 5
+        d_seeds = dev_i32(seeds, cuda)
+        cap = max(n_seeds * fanout, 1)
+        src, bptr = torch.empty(cap, dtype=torch.int32, device=cuda), torch.empty(n_seeds + 1, dtype=torch.int32, device=cuda)
+        meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+        ws = torch.empty(max(lib.fgl_sample_workspace_bytes(n_seeds, fanout), 256), dtype=torch.uint8, device=cuda)
+        rb.fill_(-7)
+        torch.cuda.synchronize()
+        L.check(lib.fgl_sample_node(L.ptr(ptr), 1, L.ptr(idx), n_nodes, L.ptr(d_seeds), n_seeds, None, fanout, 3, 1, L.ptr(src), None,
+                                    L.ptr(bptr), meta.data_ptr(), meta.data_ptr() + 4, rb.data_ptr(), L.ptr(ws), ws.numel(), st))
+        torch.cuda.synchronize()
+        assert rb.tolist() == meta.tolist() == [int(bptr[-1]), 8 if bad else 0]
+    # the fused id-map: node total and status
+    for missing in (False, True):
+        dst_unique = np.arange(100, 164, dtype=np.int32)
+        src_e = rng.integers(0, 500, size=1000).astype(np.int32)
+        dst_e = np.sort(rng.integers(100, 164, size=1000)).astype(np.int32)
+        if missing:
+            dst_e[5] = 99
+        slots = lib.fgl_idmap_slots(64 + 1000)
+        table = torch.full((slots,), -1, dtype=torch.int64, device=cuda)
+        uniq = torch.empty(64 + 1000, dtype=torch.int32, device=cuda)
+        meta = torch.zeros(2, dtype=torch.int32, device=cuda)
+        ws = torch.empty(max(lib.fgl_idmap_map_src_workspace_bytes(1000), 256), dtype=torch.uint8, device=cuda)
+        d_src, d_dst = dev_i32(src_e, cuda), dev_i32(dst_e, cuda)
+        rb.fill_(-7)
+        torch.cuda.synchronize()
+        L.check(lib.fgl_idmap_transfer(L.ptr(table), slots, L.ptr(dev_i32(dst_unique, cuda)), 64, L.ptr(d_src), L.ptr(d_dst), 1000,
+                                       L.ptr(uniq), 64 + 1000, L.IDMAP_ORDERED | L.IDMAP_FINAL | L.IDMAP_LEAVE_TABLE_EMPTY,
+                                       meta.data_ptr(), meta.data_ptr() + 4, rb.data_ptr(), L.ptr(ws), ws.numel(), st))
+        torch.cuda.synchronize()
+        n_total = 64 + np.setdiff1d(src_e, dst_unique).size
+        assert rb.tolist() == meta.tolist() == [n_total, 4 if missing else 0]
+        assert bool((table == -1).all())  # left empty for the next call
+        assert np.array_equal(uniq[:n_total].cpu().numpy()[d_src.cpu().numpy()], src_e)

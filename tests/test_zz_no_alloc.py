@@ -27,7 +27,7 @@ def _both(cuda, ptr, idx, seeds, fanout, rng_seed, stream_id):
             L.check(lib.fgl_sample_node_static(*head, st))
         else:
             ws = torch.empty(max(lib.fgl_sample_workspace_bytes(n, fanout), 256), dtype=torch.uint8, device=cuda)
-            L.check(lib.fgl_sample_node(*head, L.ptr(ws), ws.numel(), st))
+            L.check(lib.fgl_sample_node(*head, None, L.ptr(ws), ws.numel(), st))
         torch.cuda.synchronize()
         outs.append((src.cpu().numpy(), dst.cpu().numpy(), bptr.cpu().numpy(), meta.cpu().numpy()))
     return outs
