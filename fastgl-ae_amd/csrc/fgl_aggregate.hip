@@ -213,17 +213,64 @@ struct LaneSlice {
     }
 };
 
-// acc += sum over the entries [a, b) of one row (a < b), all modes except FGL_AGG_EDGE.
-template <typename T, int VEC, int LPR, int MODE, bool ALL_FULL>
-__device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, VEC>& ls, int gl, int64_t row, int a, int b,
-                                           float (&acc)[VEC])
+// part += the weighted rows of one chunk of at most LPR entries, whose ids and weights the group's lanes hold
+// (lane t: entry t).  Four row loads are issued before the first FMA; the tail of the list goes together as well
+// (measured: longer or predicated unrolls gain nothing on long lists and lose up to 2x on the one- and two-entry
+// lists of a transposed block).
+template <typename T, int VEC, int LPR, bool ALL_FULL>
+__device__ __forceinline__ void accumulate_chunk(const LaneSlice<T, VEC>& ls, const T* __restrict__ X, int64_t ldx, int my_col,
+                                                 float my_w, int cnt, float (&part)[VEC])
 {
     using IO = RowIO<T, VEC>;
-    const int32_t* __restrict__ indices = g.indices;
-    const T* __restrict__ X = static_cast<const T*>(g.x);
-    const int64_t ldx = g.ldx;
     const int col0 = ls.col0;
     const bool live = ls.live;
+    int t = 0;
+    for (; t + 4 <= cnt; t += 4) {
+        const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
+        const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
+        const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
+        const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
+        if (live) {
+            const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
+            const typename IO::Raw r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
+            const typename IO::Raw r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
+            const typename IO::Raw r3 = ls.template load_row<ALL_FULL>(X + (int64_t)c3 * ldx + col0);
+            IO::fma(part, w0, r0);
+            IO::fma(part, w1, r1);
+            IO::fma(part, w2, r2);
+            IO::fma(part, w3, r3);
+        }
+    }
+    // the last one to three entries: their loads are issued together as well (most lists of a
+    // transposed block have only this tail)
+    const int rem = cnt - t;
+    if (rem > 0) {
+        const int c0 = __shfl(my_col, t, LPR);
+        const int c1 = __shfl(my_col, rem > 1 ? t + 1 : t, LPR);
+        const int c2 = __shfl(my_col, rem > 2 ? t + 2 : t, LPR);
+        const float w0 = __shfl(my_w, t, LPR);
+        const float w1 = __shfl(my_w, rem > 1 ? t + 1 : t, LPR);
+        const float w2 = __shfl(my_w, rem > 2 ? t + 2 : t, LPR);
+        if (live) {
+            const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
+            typename IO::Raw r1 = r0, r2 = r0;
+            if (rem > 1) r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
+            if (rem > 2) r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
+            IO::fma(part, w0, r0);
+            if (rem > 1) IO::fma(part, w1, r1);
+            if (rem > 2) IO::fma(part, w2, r2);
+        }
+    }
+}
+
+// acc += sum over the entries [a, b) of one row (a < b), all modes except FGL_AGG_EDGE.
+// first_col (optional): the ids of the row's first chunk, already loaded (lane t: entry a + t).
+template <typename T, int VEC, int LPR, int MODE, bool ALL_FULL>
+__device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, VEC>& ls, int gl, int64_t row, int a, int b,
+                                           float (&acc)[VEC], const int* first_col = nullptr)
+{
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
     float row_factor = 1.0f;
     if (MODE == FGL_AGG_MEAN) row_factor = 1.0f / (float)(b - a);
     if (MODE == FGL_AGG_GCN) row_factor = 1.0f / sqrtf((float)g.row_norm[row]);
@@ -233,12 +280,9 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
         int my_col = 0;
         float my_w = 0.0f;
         if (gl < cnt) {
-            my_col = indices[base + gl];
+            my_col = (first_col != nullptr && base == a) ? *first_col : indices[base + gl];
             my_w = edge_weight<MODE>(my_col, row_factor, g.col_norm, g.col_norm_is_ptr);
         }
-        // four row loads are issued before the first FMA; the tail of the list goes one by one
-        // (measured: longer or predicated unrolls gain nothing on long lists and lose up to 2x
-        // on the one- and two-entry lists of a transposed block).
         // Two-level summation: each chunk of LPR entries is summed on its own and then added to
         // the row total, so the rounding error of a row with thousands of entries (a hub in a
         // transposed block) grows like LPR + n/LPR instead of n.  Rows of at most LPR entries --
@@ -246,43 +290,7 @@ __device__ __forceinline__ void gather_row(const AggArgs& g, const LaneSlice<T, 
         float part[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) part[i] = 0.0f;
-        int t = 0;
-        for (; t + 4 <= cnt; t += 4) {
-            const int c0 = __shfl(my_col, t, LPR), c1 = __shfl(my_col, t + 1, LPR);
-            const int c2 = __shfl(my_col, t + 2, LPR), c3 = __shfl(my_col, t + 3, LPR);
-            const float w0 = __shfl(my_w, t, LPR), w1 = __shfl(my_w, t + 1, LPR);
-            const float w2 = __shfl(my_w, t + 2, LPR), w3 = __shfl(my_w, t + 3, LPR);
-            if (live) {
-                const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
-                const typename IO::Raw r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
-                const typename IO::Raw r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
-                const typename IO::Raw r3 = ls.template load_row<ALL_FULL>(X + (int64_t)c3 * ldx + col0);
-                IO::fma(part, w0, r0);
-                IO::fma(part, w1, r1);
-                IO::fma(part, w2, r2);
-                IO::fma(part, w3, r3);
-            }
-        }
-        // the last one to three entries: their loads are issued together as well (most lists of a
-        // transposed block have only this tail)
-        const int rem = cnt - t;
-        if (rem > 0) {
-            const int c0 = __shfl(my_col, t, LPR);
-            const int c1 = __shfl(my_col, rem > 1 ? t + 1 : t, LPR);
-            const int c2 = __shfl(my_col, rem > 2 ? t + 2 : t, LPR);
-            const float w0 = __shfl(my_w, t, LPR);
-            const float w1 = __shfl(my_w, rem > 1 ? t + 1 : t, LPR);
-            const float w2 = __shfl(my_w, rem > 2 ? t + 2 : t, LPR);
-            if (live) {
-                const typename IO::Raw r0 = ls.template load_row<ALL_FULL>(X + (int64_t)c0 * ldx + col0);
-                typename IO::Raw r1 = r0, r2 = r0;
-                if (rem > 1) r1 = ls.template load_row<ALL_FULL>(X + (int64_t)c1 * ldx + col0);
-                if (rem > 2) r2 = ls.template load_row<ALL_FULL>(X + (int64_t)c2 * ldx + col0);
-                IO::fma(part, w0, r0);
-                if (rem > 1) IO::fma(part, w1, r1);
-                if (rem > 2) IO::fma(part, w2, r2);
-            }
-        }
+        accumulate_chunk<T, VEC, LPR, ALL_FULL>(ls, X, g.ldx, my_col, my_w, cnt, part);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] += part[i];
     }
@@ -415,6 +423,76 @@ __global__ __launch_bounds__(kBlock) void aggregate_kernel(const AggArgs g)
         else gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc);
     }
     if (live) ls.store(out + row * ldo + col0, acc);
+}
+
+// The same mapping as a loop: a fixed number of lane groups, each taking rows g, g + G, g + 2G, ... and fetching the
+// row after next's two offsets and the next row's neighbour ids while the current row's data is in flight, so that
+// a row's chain offsets -> ids -> data is not walked from its start for every row.  Same sums in the same order.
+// An experiment, not built by default (make HIPFLAGS_EXTRA="-DFGL_AGG_PIPE=1 -DFGL_AGG_PIPE_BLOCKS=8192" builds it in):
+// measured on the outermost block of a 111 M-node graph's mini-batches (1.5 M gathered rows of 512 B, and of 256 B
+// in bf16) it runs 0-3 % slower than one lane group per row with 2048-8192 persistent workgroups -- the gather is
+// bound by the rate at which the memory system serves random rows, and the thousands of resident waves of the
+// plain mapping already hide a single row's chain.
+#ifndef FGL_AGG_PIPE
+#define FGL_AGG_PIPE 0
+#endif
+#ifndef FGL_AGG_PIPE_BLOCKS
+#define FGL_AGG_PIPE_BLOCKS 4096
+#endif
+template <typename T, int VEC, int LPR, int MODE>
+__global__ __launch_bounds__(kBlock) void aggregate_pipe_kernel(const AggArgs g)
+{
+    using IO = RowIO<T, VEC>;
+    constexpr int kGroups = kBlock / LPR;
+    const int32_t* __restrict__ indptr = g.indptr;
+    const int32_t* __restrict__ indices = g.indices;
+    const T* __restrict__ X = static_cast<const T*>(g.x);
+    T* __restrict__ out = static_cast<T*>(g.out);
+    const int64_t ldx = g.ldx, ldo = g.ldo;
+    const int64_t n_rows = actual_count(g.n_rows_max, g.d_n_rows);
+    const int gl = (int)threadIdx.x % LPR;
+    const int64_t stride = (int64_t)gridDim.x * kGroups;
+    const LaneSlice<T, VEC> ls((int)blockIdx.y, LPR, gl, g.D);
+    const bool all_full = all_lanes_full<T, VEC>(g.D);
+    int64_t row = (int64_t)blockIdx.x * kGroups + (int)threadIdx.x / LPR;
+    int64_t nrow = row + stride;
+    int a = 0, b = 0, na = 0, nb = 0;
+    if (row < n_rows) {
+        a = indptr[row];
+        b = indptr[row + 1];
+    }
+    if (nrow < n_rows) {
+        na = indptr[nrow];
+        nb = indptr[nrow + 1];
+    }
+    int my_col = (row < n_rows && gl < b - a) ? indices[a + gl] : 0;
+    while (row < n_rows) {  // (uniform over a lane group; a wave's groups may leave at different times)
+        const int64_t nnrow = nrow + stride;
+        int nna = 0, nnb = 0;
+        if (nnrow < n_rows) {
+            nna = indptr[nnrow];
+            nnb = indptr[nnrow + 1];
+        }
+        const int n_col = (nrow < n_rows && gl < nb - na) ? indices[na + gl] : 0;
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+        if (a == b) {
+            if (ls.live && g.zero_policy == FGL_ZERO_COPY_SELF) IO::fma(acc, 1.0f, ls.load(X + row * ldx + ls.col0));
+        } else if (all_full) {
+            gather_row<T, VEC, LPR, MODE, true>(g, ls, gl, row, a, b, acc, &my_col);
+        } else {
+            gather_row<T, VEC, LPR, MODE, false>(g, ls, gl, row, a, b, acc, &my_col);
+        }
+        if (ls.live) ls.store(out + row * ldo + ls.col0, acc);
+        row = nrow;
+        a = na;
+        b = nb;
+        nrow = nnrow;
+        na = nna;
+        nb = nnb;
+        my_col = n_col;
+    }
 }
 
 // ---- few rows, long lists: several lane groups share a row -----------------------------------------
@@ -1115,6 +1193,22 @@ static int launch_agg_mode(int mode, bool long_rows_possible, dim3 grid, hipStre
 {
     const bool second_pass = long_rows_possible;
     g.skip_rows_longer_than = second_pass ? kLongRowEntries : 0x7FFFFFFF;
+    if constexpr (FGL_AGG_PIPE != 0) {
+      if (!second_pass && mode != FGL_AGG_EDGE && (int64_t)grid.x > FGL_AGG_PIPE_BLOCKS) {
+        note_mapping("aggregate_pipe_kernel", LPR, 1, false);
+        const dim3 pgrid(FGL_AGG_PIPE_BLOCKS, grid.y);
+#define FGL_LAUNCH_PIPE(M) hipLaunchKernelGGL((aggregate_pipe_kernel<T, VEC, LPR, M>), pgrid, dim3(kBlock), 0, stream, g)
+        switch (mode) {
+            case FGL_AGG_SUM: FGL_LAUNCH_PIPE(FGL_AGG_SUM); break;
+            case FGL_AGG_MEAN: FGL_LAUNCH_PIPE(FGL_AGG_MEAN); break;
+            case FGL_AGG_GCN: FGL_LAUNCH_PIPE(FGL_AGG_GCN); break;
+            default: FGL_LAUNCH_PIPE(FGL_AGG_COLMEAN); break;
+        }
+#undef FGL_LAUNCH_PIPE
+        FGL_CHECK_LAUNCH("aggregate_pipe_kernel");
+        return FGL_OK;
+      }
+    }
     note_mapping("aggregate_kernel", LPR, 1, second_pass);
 #define FGL_LAUNCH_MODE(M)                                                                                         \
     do {                                                                                                           \
