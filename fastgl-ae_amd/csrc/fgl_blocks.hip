@@ -142,7 +142,10 @@ static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
 // hop h (entry n_hops: after the last hop).  The plan is the worst case clipped to it.
 // Hops of at least this many edges (by the plan's bound) count their transposed rows with kTransposeSplit
 // counters per column: a hub column of such a hop is mentioned thousands of times.
-constexpr int64_t kTransposeSplitMinEdges = (int64_t)1 << 20;
+#ifndef FGL_TRANSPOSE_SPLIT_MIN_EDGES
+#define FGL_TRANSPOSE_SPLIT_MIN_EDGES (1 << 20)
+#endif
+constexpr int64_t kTransposeSplitMinEdges = FGL_TRANSPOSE_SPLIT_MIN_EDGES;
 constexpr int kTransposeSplit = 8;
 
 static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, int n_hops, const int64_t* node_capacity,
@@ -403,7 +406,7 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         job_before.side_blocks = side_blocks_for(job_before.cols_max * job_before.split + 1, kTjobTile, 8192);
         hipLaunchKernelGGL(transpose_step_kernel<0>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
         hipLaunchKernelGGL(transpose_step_kernel<1>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
-        job_before.side_blocks = side_blocks_for(job_before.rows_max, kBlock / 16, 8192);
+        job_before.side_blocks = side_blocks_for(job_before.rows_max, kBlock / 16, 16384);
         hipLaunchKernelGGL(transpose_step_kernel<2>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
         FGL_CHECK_LAUNCH("transpose_step_kernel");
     }

@@ -707,7 +707,7 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
     if (before.cnt != nullptr) {
         scan_job.side_first = fill_job.side_first = 0;
         scan_blocks = scan_job.side_blocks = side_blocks_for(before.cols_max * before.split + 1, kTjobTile);
-        fill_blocks_t = fill_job.side_blocks = side_blocks_for(before.rows_max, kBlock / 16);
+        fill_blocks_t = fill_job.side_blocks = side_blocks_for(before.rows_max, kBlock / 16, 16384);
     }
     FGL_REQUIRE(!leave_table_empty || final_call, "idmap_map_src: only a final call can leave the table empty");
 

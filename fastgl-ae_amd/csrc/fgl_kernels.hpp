@@ -57,7 +57,7 @@ struct TransposeJob {
 };
 // Side workgroups for a step over n_items, items_per_block at a time: never more than the work needs, and few
 // enough that they are an appendix to the launch that carries them.
-inline int side_blocks_for(int64_t n_items, int64_t items_per_block, int cap = 1024)
+inline int side_blocks_for(int64_t n_items, int64_t items_per_block, int cap = 8192)
 {
     int64_t b = (n_items + items_per_block - 1) / items_per_block;
     if (b < 1) b = 1;
