@@ -122,7 +122,7 @@ def run_c4(args, edge_weighted=True):
     # The transposed block's longest row: the transpose leaves it on the device (the backward launches below find it there
     # and pay a second, empty launch that looks for hub rows); a caller that has read it back -- a block that is
     # transposed once and used many times, or one whose sizes travel to the host anyway -- passes it as a bound.
-    t_longest = int(t_ptr.fgl_longest_row.item())
+    t_longest = max(int(t_ptr.fgl_longest_row.item()), 32)  # (the transpose reports lengths beyond 32 entries only)
     deg = torch.full((n_dst,), k, dtype=torch.int32, device=dev)
     E = n_dst * k
     ev = lambda: torch.cuda.Event(enable_timing=True)
@@ -1117,7 +1117,8 @@ def run_graph_workload(args, workload, light=False):
                                     "frac_of_peak_by_traffic = the counter-derived bytes / the same time / peak; "
                                     "traffic = bytes per launch that the L2s fetch and write (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled): "
                                     "repeated rows that hit in L2 are not in it, hits in the memory-side Infinity Cache still are",
-                     "kernel": "aggregate_kernel<float,4,32,MEAN> (outermost block, forward)",
+                     "kernel": ("aggregate_kernel<float,4,32,MEAN>" if w["dtype"] == "f32" and D == 128 else
+                                "aggregate_kernel, %s rows of %d columns, MEAN" % (w["dtype"], D)) + " (outermost block, forward)",
                      "bytes_per_launch": bytes_agg0 / K, "us_per_launch": t_kernel0 / K * 1e3},
         "cpu_baseline": cpu,
         "parity_checked": parity,

@@ -135,8 +135,9 @@ def test_sample_blocks_golden(cuda, oracle, fused):
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("fanouts,batch", [([15, 10, 5], 1024), ([10, 10, 10, 10, 10], 64), ([3], 1), ([64, 2], 300),
-                                           # batches of 8192 and more seeds with small and mid fanouts (a third mini-batch is all hubs)
-                                           ([3, 16], 8192), ([3, 17], 500), ([2, 8], 8192), ([2, 5], 8193), ([4, 1], 1)])
+                                           # batches of 8192 and more seeds with small and mid fanouts, a single hop of fanout 16; a third
+                                           # mini-batch is all hubs
+                                           ([3, 16], 8192), ([3, 17], 500), ([2, 8], 8192), ([2, 5], 8193), ([4, 1], 1), ([16], 700)])
 def test_sample_blocks_vs_oracle(cuda, oracle, small_graph, fused, fanouts, batch):
     import fastgl
     print("sample_blocks %s batch=%d fused=%s" % (fanouts, batch, fused), flush=True)
