@@ -331,11 +331,24 @@ def run_ceiling(args):
                     idx64 = idx.long()
                     t = timed(lambda: torch.index_select(table, 0, idx64, out=out))
                     case["torch_index_select_GBps"] = 2 * n_out * row_bytes / t / 1e9
+                else:
+                    # the same gather-and-sum by a kernel that is not this library's: torch's embedding_bag
+                    # (same bytes counted; it also writes a bag index per entry, which is not)
+                    try:
+                        idx64 = idx.long()
+                        off64 = ptr[:-1].long()
+                        bag = lambda: torch.nn.functional.embedding_bag(idx64, table, off64, mode="sum")
+                        t = timed(bag)
+                        case["torch_embedding_bag_k13_GBps"] = moved / t / 1e9
+                        del bag
+                    except Exception as e:  # (a dtype the library kernel does not take)
+                        case["torch_embedding_bag_k13_GBps"] = None
+                        log("embedding_bag: %s" % str(e).splitlines()[0])
             rows_out.append(case)
             log("%-4s rows of %4d B: 1 source per row %5.0f GB/s (%.1f G rows/s; torch.index_select %5.0f GB/s) | "
-                "13 sources per row %5.0f GB/s (%.1f G rows/s)"
+                "13 sources per row %5.0f GB/s (%.1f G rows/s; torch embedding_bag %5.0f GB/s)"
                 % (case["dtype"], row_bytes, case["k1_GBps"], case["k1_Grows_per_s"], case["torch_index_select_GBps"],
-                   case["k13_GBps"], case["k13_Grows_per_s"]))
+                   case["k13_GBps"], case["k13_Grows_per_s"], case["torch_embedding_bag_k13_GBps"] or 0.0))
             del table, out
             torch.cuda.empty_cache()
     a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -836,6 +849,36 @@ def run_graph_workload(args, workload, light=False):
         log("id order %s: %.3g sampled edges/s (sample+idmap %.3f ms)" % (other_order, value_other, alt_ms / args.steps))
         del alt, rec_alt
 
+    # ---- the same steps with a sampler that hands over the blocks only (transposed="none"): the transposed inner
+    # blocks are then built by the batch transpose behind the forward pass, five launches, as a caller without
+    # the all-in-one call would; shows what carrying them inside the sampling call costs that stage and saves the step
+    blocks_only = None
+    if sampler_mode == "eager" and other_order_on and L > 1:
+        keep_main = list(keep)
+        alt = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order, transposed="none").set_graph(edge_ptr, edge_src)
+        for i in range(args.warmup):
+            step(i, None, alt)
+        torch.cuda.synchronize()
+        rec_alt = []
+        for i in range(args.steps):
+            step(args.warmup + i, rec_alt, alt)
+        torch.cuda.synchronize()
+        keep[:] = keep_main
+        alt_edges = sum(r[0][0] for r in rec_alt)
+        t01 = sum(r[1][0].elapsed_time(r[1][1]) for r in rec_alt)
+        t34 = sum(r[1][3].elapsed_time(r[1][4]) for r in rec_alt)
+        t04 = sum(r[1][0].elapsed_time(r[1][4]) for r in rec_alt)
+        blocks_only = {"value": alt_edges / (t01 * 1e-3), "sample_idmap_ms": t01 / args.steps,
+                       "default_gpu_ms_per_step": sum(r[1][0].elapsed_time(r[1][4]) for r in rec) / args.steps,
+                       "transpose_agg_bwd_inner_ms": t34 / args.steps, "gpu_ms_per_step": t04 / args.steps,
+                       "what": "the sampler hands over the blocks without their transposed form "
+                               "(FusedMapSampler(transposed='none')); the inner blocks are transposed by "
+                               "fgl_block_transpose_batch in front of the backward gathers"}
+        log("blocks only: %.3g sampled edges/s (sample+idmap %.3f ms, transpose+bwd %.3f ms, GPU time of a step %.3f ms)"
+            % (blocks_only["value"], blocks_only["sample_idmap_ms"], blocks_only["transpose_agg_bwd_inner_ms"],
+               blocks_only["gpu_ms_per_step"]))
+        del alt, rec_alt
+
     # ---- the same mini-batches through the two other forms of the sampler (context for `value`) -------------
     # value_sample_blocks: FusedMapSampler.sample_blocks(), i.e. the fused call followed at once by the one
     # read-back of the batch's sizes (the host's wait is inside the interval).
@@ -1109,6 +1152,7 @@ def run_graph_workload(args, workload, light=False):
         "value_sample_blocks": value_sample_blocks,
         "value_drop_in_api": value_drop_in,
         "value_other_id_order": {"id_order": other_order, "value": value_other},
+        "value_blocks_only": blocks_only,
         "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
