@@ -1140,7 +1140,7 @@ def run_graph_workload(args, workload, light=False):
                    "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
                    "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
                            "feature table); block transpose + bwd gather on the inner blocks; no dense layers",
-                   "readback": ("the batch's sizes reach the host on a second stream while the outermost aggregation runs "
+                   "readback": ("the batch's sizes are stored into pinned host memory by the sampling kernels; the host waits for them while the outermost aggregation runs "
                                 "(sample_idmap = the sampling kernels' own time)") if args.readback == "hidden" else
                                "the batch's sizes are read back before anything else is enqueued (inside sample_idmap)"},
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,

@@ -205,12 +205,17 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
 
 // The three closing steps of a transposed block as launches of their own: for the last hop of a call, which has no
 // later hop whose launches could carry them.
+// The last of them also hands the call's counts to the host, if asked: everything in them is final by then.
 template <int STEP>
-__global__ __launch_bounds__(kBlock) void transpose_step_kernel(const TransposeJob j)
+__global__ __launch_bounds__(kBlock) void transpose_step_kernel(const TransposeJob j, int32_t* __restrict__ readback,
+                                                                const int32_t* __restrict__ counts, int n_counts)
 {
     if (STEP == 0) tjob_tile_sums<kBlock>(j);
     if (STEP == 1) tjob_scan<kBlock>(j);
-    if (STEP == 2) tjob_fill<kBlock>(j);
+    if (STEP == 2) {
+        if (readback != nullptr && blockIdx.x == 0 && (int)threadIdx.x < n_counts) readback[threadIdx.x] = counts[threadIdx.x];
+        tjob_fill<kBlock>(j);
+    }
 }
 
 // ---- R-MAT -------------------------------------------------------------------------
@@ -271,8 +276,8 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
                                  int64_t table_slots,
                                  int32_t* d_uniq, int64_t uniq_capacity, int32_t* const* block_ptr,
                                  int32_t* const* src_local, int32_t* const* src_global, int32_t* const* t_ptr,
-                                 int32_t* const* t_dst, int32_t* const* t_edge, int32_t* d_counts, void* d_ws,
-                                 size_t ws_bytes, void* stream)
+                                 int32_t* const* t_dst, int32_t* const* t_edge, int32_t* d_counts, int32_t* d_readback,
+                                 void* d_ws, size_t ws_bytes, void* stream)
 {
     // the hops whose transposed block is wanted: those with a row-pointer output
     uint32_t transpose_hops = 0;
@@ -394,20 +399,27 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         // the node count this hop may grow to: what the next hop's buffers (or the unique list) hold;
         // growing past it is reported as FGL_STATUS_UNIQ_OVERFLOW and the count is clamped
         const int64_t grow_to = (!last && p.cap_dst[h + 1] < p.cap_uniq) ? p.cap_dst[h + 1] : p.cap_uniq;
+        // the host's copy of the counts: written by whichever launch makes the last of them final -- the last hop's
+        // node total, or (if the last hop's transposed block is wanted) its longest row, below
+        const bool counts_final_here = last && steps.zero.cnt == nullptr;
         rc = launch_idmap_map_src(d_table, table_slots, sampled, src_local[h], p.cap_edges[h], d_n_edges, 0, d_n_dst,
                                   d_counts + h + 1, d_uniq, grow_to, order | (last ? FGL_IDMAP_FINAL : 0), d_status,
                                   ws.idmap_ws, p.idmap_bytes, s, /*counter_is_zeroed=*/true, last ? nullptr : &next,
-                                  /*leave_table_empty=*/last && leave_empty, ws.lowered, &steps.zero, &job_before);
+                                  /*leave_table_empty=*/last && leave_empty, ws.lowered, &steps.zero, &job_before, nullptr,
+                                  counts_final_here ? d_readback : nullptr, d_counts, n_counts);
         if (rc != FGL_OK) return rc;
         job_before = steps.zero;
     }
     if (job_before.cnt != nullptr) {  // the last hop's transposed block: no later launch to carry its closing steps
         job_before.side_first = 0;
         job_before.side_blocks = side_blocks_for(job_before.cols_max * job_before.split + 1, kTjobTile, 8192);
-        hipLaunchKernelGGL(transpose_step_kernel<0>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
-        hipLaunchKernelGGL(transpose_step_kernel<1>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
+        hipLaunchKernelGGL(transpose_step_kernel<0>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before,
+                           nullptr, nullptr, 0);
+        hipLaunchKernelGGL(transpose_step_kernel<1>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before,
+                           nullptr, nullptr, 0);
         job_before.side_blocks = side_blocks_for(job_before.rows_max, kBlock / 16, 16384);
-        hipLaunchKernelGGL(transpose_step_kernel<2>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before);
+        hipLaunchKernelGGL(transpose_step_kernel<2>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before,
+                           d_readback, d_counts, n_counts);
         FGL_CHECK_LAUNCH("transpose_step_kernel");
     }
     return FGL_OK;

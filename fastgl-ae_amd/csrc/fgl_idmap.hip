@@ -256,9 +256,14 @@ __global__ __launch_bounds__(kBlock) void idmap_mark_kernel(TableRef t, int64_t 
 }
 
 // n_total = n_base + (number of new ids), clamped to the capacity of the unique list.
+// readback (optional, may be host memory that the device can write): where the host reads the call's sizes.
+// Without rb_counts: two words, {node total, status word}.  With rb_counts (the all-hops call's count array, which
+// holds both d_n_total_out and the status word): a copy of its rb_n words as they stand now -- the other entries
+// were final before this launch began.
 __device__ __forceinline__ void publish_node_total(int64_t n_base, int n_new, int64_t capacity,
                                                    int32_t* __restrict__ d_n_total_out, uint32_t* __restrict__ d_status,
-                                                   int32_t* __restrict__ readback = nullptr)
+                                                   int32_t* __restrict__ readback = nullptr,
+                                                   const int32_t* __restrict__ rb_counts = nullptr, int rb_n = 0)
 {
     int64_t total = n_base + (int64_t)n_new;
     uint32_t overflow = 0u;
@@ -268,10 +273,19 @@ __device__ __forceinline__ void publish_node_total(int64_t n_base, int n_new, in
         total = capacity;
     }
     if (d_n_total_out) *d_n_total_out = (int32_t)total;
-    if (readback) {
-        // {node total, status word}: every other bit of the status word was set by an earlier launch of the call
+    if (readback == nullptr) return;
+    // (every other bit of the status word was set by an earlier launch of the call)
+    const int32_t status = (int32_t)((d_status ? *d_status : 0u) | overflow);
+    if (rb_counts == nullptr) {
         readback[0] = (int32_t)total;
-        readback[1] = (int32_t)((d_status ? *d_status : 0u) | overflow);
+        readback[1] = status;
+        return;
+    }
+    for (int i = 0; i < rb_n; ++i) {
+        int32_t v = rb_counts[i];
+        if (rb_counts + i == d_n_total_out) v = (int32_t)total;
+        if (rb_counts + i == reinterpret_cast<const int32_t*>(d_status)) v = status;
+        readback[i] = v;
     }
 }
 
@@ -282,7 +296,8 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
                                                                     const int32_t* __restrict__ d_e, int64_t n_base_h,
                                                                     const int32_t* __restrict__ d_n_base, int64_t capacity,
                                                                     int32_t* __restrict__ d_n_total_out,
-                                                                    uint32_t* __restrict__ d_status, int32_t* __restrict__ readback)
+                                                                    uint32_t* __restrict__ d_status, int32_t* __restrict__ readback,
+                                                                    const int32_t* __restrict__ rb_counts, int rb_n)
 {
     __shared__ int smem[1024 / kWave + 1];
     const int n_tiles = (int)tiles_of(actual_count(e_max, d_e));
@@ -296,7 +311,7 @@ __global__ __launch_bounds__(1024) void idmap_prefix_publish_kernel(const int32_
         carry += total;
     }
     if (threadIdx.x == 0)
-        publish_node_total(d_n_base ? (int64_t)(*d_n_base) : n_base_h, carry, capacity, d_n_total_out, d_status, readback);
+        publish_node_total(d_n_base ? (int64_t)(*d_n_base) : n_base_h, carry, capacity, d_n_total_out, d_status, readback, rb_counts, rb_n);
 }
 
 // Up to this many tiles the number pass scans the tile counts itself (every workgroup, into LDS) and
@@ -356,7 +371,8 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
                                                               int32_t* __restrict__ d_n_total_out,
                                                               uint32_t* __restrict__ d_status, const NextHop next,
                                                               uint32_t* __restrict__ clear_words, int64_t n_clear_words,
-                                                              const TransposeRank tr, int32_t* __restrict__ readback)
+                                                              const TransposeRank tr, int32_t* __restrict__ readback,
+                                                              const int32_t* __restrict__ rb_counts, int rb_n)
 {
     __shared__ int s_prefix[SELF ? kIdmapSelfPrefixTiles : 1];
     __shared__ int smem[kBlock / kWave + 1];
@@ -393,7 +409,7 @@ __global__ __launch_bounds__(kBlock) void idmap_number_kernel(TableRef t, const 
             run += v[j];
         }
         __syncthreads();
-        if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status, readback);
+        if (blockIdx.x == 0 && threadIdx.x == 0) publish_node_total(n_base, total, capacity, d_n_total_out, d_status, readback, rb_counts, rb_n);
     }
     // the last pass of a mini-batch, which no longer reads the table, can leave it empty for the next one
     // (first, so that the stores drain while the edges are being numbered)
@@ -592,7 +608,8 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
                                                                        int64_t n_base_h, const int32_t* __restrict__ d_n_base,
                                                                        int64_t capacity, int32_t* __restrict__ d_n_total_out,
                                                                        uint32_t* __restrict__ d_status, const TransposeRank tr,
-                                                                       const TransposeJob before, int32_t* __restrict__ readback)
+                                                                       const TransposeJob before, int32_t* __restrict__ readback,
+                                                                       const int32_t* __restrict__ rb_counts, int rb_n)
 {
     tjob_fill<kBlock>(before);  // (the hop before, if its transposed block is being built: entries into their rows)
     const int64_t n_e = actual_count(e_max, d_e);
@@ -607,7 +624,7 @@ __global__ __launch_bounds__(kBlock) void idmap_relabel_publish_kernel(TableRef 
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         const int64_t n_base = d_n_base ? (int64_t)(*d_n_base) : n_base_h;
-        publish_node_total(n_base, *counter, capacity, d_n_total_out, d_status, readback);
+        publish_node_total(n_base, *counter, capacity, d_n_total_out, d_status, readback, rb_counts, rb_n);
     }
 }
 
@@ -669,7 +686,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          int32_t* d_uniq, int64_t uniq_capacity, int flags, uint32_t* d_status, void* d_ws,
                          size_t ws_bytes, hipStream_t stream, bool counter_is_zeroed, const NextHop* next_hop,
                          bool leave_table_empty, uint8_t* d_lowered, const TransposeJob* rank_job,
-                         const TransposeJob* before_job, int32_t* d_dst_inout, int32_t* d_readback)
+                         const TransposeJob* before_job, int32_t* d_dst_inout, int32_t* d_readback,
+                         const int32_t* d_readback_counts, int n_readback_counts)
 {
     FGL_REQUIRE(d_table != nullptr && valid_slots(slots), "idmap: slot count %lld is not a power of two in [64, 2^31]", (long long)slots);
     FGL_REQUIRE((flags & ~(FGL_IDMAP_ARRIVAL | FGL_IDMAP_FINAL)) == 0, "idmap_map_src: unknown flags %d", flags);
@@ -736,7 +754,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                                d_status, next, tr, scan_job);
         FGL_CHECK_LAUNCH("idmap_insert_arrival_kernel");
         hipLaunchKernelGGL(idmap_relabel_publish_kernel, dim3(edge_blocks + fill_blocks_t), dim3(kBlock), 0, stream, t, n_edges_max, d_n_edges,
-                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, tr, fill_job, d_readback);
+                           slot_of, d_src_out, counter, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, tr, fill_job, d_readback,
+                           d_readback_counts, n_readback_counts);
         FGL_CHECK_LAUNCH("idmap_relabel_publish_kernel");
         // (the second pass reads the table, so emptying it takes a launch of its own here)
         if (leave_table_empty) return launch_fill_u32(t.words, slots * 2, kEmpty, stream);
@@ -760,7 +779,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
 #define FGL_LAUNCH_NUMBER(SELF, WB, PREFIX, TOTAL, STATUS, READBACK)                                                              \
     hipLaunchKernelGGL((idmap_number_kernel<SELF, WB>), dim3(edge_blocks), dim3(kBlock), 0, stream, t, d_src_in,        \
                        n_edges_max, d_n_edges, n_base, d_n_base, slot_of, first_of, flags8, before8, sums, PREFIX, d_uniq, \
-                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words, tr, READBACK)
+                       uniq_capacity, d_src_out, TOTAL, STATUS, next, clear_words, n_clear_words, tr, READBACK, d_readback_counts,   \
+                       n_readback_counts)
     // emptying the table rides on the last pass: enough workgroups for a fill of that size
     uint32_t* clear_words = leave_table_empty ? t.words : nullptr;
     const int64_t n_clear_words = leave_table_empty ? slots * 2 : 0;
@@ -776,7 +796,8 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
         else FGL_LAUNCH_NUMBER(true, true, nullptr, d_n_total_out, d_status, d_readback);
     } else {
         hipLaunchKernelGGL(idmap_prefix_publish_kernel, dim3(1), dim3(1024), 0, stream, sums, prefix, n_edges_max,
-                           d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, d_readback);
+                           d_n_edges, n_base, d_n_base, uniq_capacity, d_n_total_out, d_status, d_readback, d_readback_counts,
+                           n_readback_counts);
         FGL_CHECK_LAUNCH("idmap_prefix_publish_kernel");
         if (final_call) FGL_LAUNCH_NUMBER(false, false, prefix, nullptr, nullptr, nullptr);
         else FGL_LAUNCH_NUMBER(false, true, prefix, nullptr, nullptr, nullptr);

@@ -117,7 +117,9 @@ int launch_idmap_map_src(void* d_table, int64_t slots, const int32_t* d_src_in, 
                          const TransposeJob* rank_job = nullptr,     // (may be null) the edges take their ranks in this block's transposed rows
                          const TransposeJob* before_job = nullptr,   // (may be null) scan and fill steps of the hop before, carried by the first two passes
                          int32_t* d_dst_inout = nullptr,             // (may be null) n_edges_max ids that are in the table already: relabelled in place by the first pass
-                         int32_t* d_readback = nullptr);             // (may be null) {node total, status word} once both are final; may be host memory
+                         int32_t* d_readback = nullptr,              // (may be null) {node total, status word} once both are final; may be host memory
+                         const int32_t* d_readback_counts = nullptr, // (may be null) instead of those two words: a copy of this array, which holds
+                         int n_readback_counts = 0);                 //   *d_n_total_out and the status word, taken when the node total is final
 
 // deterministic block transpose (fgl_transpose_sort.hip): fills t_indices / t_edge given the offsets
 size_t sorted_transpose_workspace_bytes(int64_t n_cols, int64_t n_edges);

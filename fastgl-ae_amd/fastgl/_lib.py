@@ -19,7 +19,7 @@ CSRC_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "csrc"))
 F32, BF16 = 0, 1
 AGG_SUM, AGG_MEAN, AGG_GCN, AGG_COLMEAN, AGG_EDGE, AGG_COLMEAN_PTR = 0, 1, 2, 3, 4, 5
 ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
-ABI_VERSION = 10  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
+ABI_VERSION = 11  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL, IDMAP_LEAVE_TABLE_EMPTY = 0, 1, 2, 8
 BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
@@ -50,7 +50,7 @@ SIGNATURES = {
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]),
     "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _vp, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
-                                 _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+                                 _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_block_transpose_workspace_bytes": (_sz, [_i64, _i64, _i32]),
     "fgl_block_transpose": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp, _sz, _vp]),
     "fgl_block_transpose_batch_workspace_bytes": (_sz, [_i32, _vp, _vp]),

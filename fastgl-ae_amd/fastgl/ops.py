@@ -505,7 +505,7 @@ class BlocksPlan:
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
-                        keep_global=(0,), table_slots=None, id_order="first", stream_offset=None):
+                        keep_global=(0,), table_slots=None, id_order="first", stream_offset=None, readback=None):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
@@ -522,7 +522,10 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     their inserts land (the reference's rule, and about a tenth faster; any run is a valid map, equal to every other after
     sorting the new ids).
     ``stream_offset``: one-element int32 device tensor added to ``stream_base`` when the kernels run (for
-    callers that capture this call in a graph and advance the random stream between replays)."""
+    callers that capture this call in a graph and advance the random stream between replays).
+    ``readback``: a pinned int32 host tensor of ``3*n_hops + 2`` elements; the kernels store a copy of
+    ``counts`` there when the last of them is final, so the caller's read-back is a wait for the stream and a
+    look at that tensor, with no copy to enqueue."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
     _check_input(indices, "indices", _I32)
     _check_input(seeds, "seeds", _I32)
@@ -532,6 +535,9 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     if int(seeds.numel()) != plan.n_seeds:
         raise RuntimeError("plan was made for %d seeds, got %d" % (plan.n_seeds, seeds.numel()))
     H = plan.n_hops
+    if readback is not None and not (readback.dtype == torch.int32 and readback.is_pinned() and readback.is_contiguous()
+                                     and readback.numel() >= 3 * H + 2):
+        raise RuntimeError("readback must be a contiguous pinned int32 host tensor of at least %d elements" % (3 * H + 2))
     keep = {(h + H) % H for h in keep_global}
     slots = plan.slots if table_slots is None else min(int(table_slots), plan.slots)
     lib = L.lib()
@@ -559,7 +565,8 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,
                                       int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(stream_base) & 0xFFFFFFFF, L.ptr(stream_offset),
                                       flags, L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
-                                      arr(src_local), arr(src_global), t_arr(0), t_arr(1), t_arr(2), L.ptr(counts), L.ptr(plan.ws),
+                                      arr(src_local), arr(src_global), t_arr(0), t_arr(1), t_arr(2), L.ptr(counts),
+                                      None if readback is None else readback.data_ptr(), L.ptr(plan.ws),
                                       plan.ws.numel(), L.stream_handle()))
         plan.empty_slots = slots
     return uniq, block_ptr, src_local, src_global, counts, transposed

@@ -127,10 +127,26 @@ class _ShapeState:
         self.graphs = None      # (plan, table slots) -> captured launch sequences, see FusedMapSampler._replay
 
 
+class _HostCounts:
+    """Pinned host words that the kernels of a mini-batch write its sizes into (``readback`` of
+    ``ops.sample_blocks_fused``).  A sampler keeps a few and hands them out in turn; one that is still waiting to be
+    read is never handed out again."""
+
+    def __init__(self, n_words):
+        self.words = torch.empty(n_words, dtype=torch.int32, pin_memory=True)
+        self.busy = False
+
+    def read(self):
+        """The words as a list; the caller has waited for the kernels that write them."""
+        values = self.words.tolist()
+        self.busy = False
+        return values
+
+
 class PendingBatch:
     """A mini-batch whose kernels are enqueued and whose sizes are still on the device
-    (``FusedMapSampler.begin_sample``).  The sizes travel to a pinned host buffer on a second stream as soon as
-    the sampling kernels are done, whatever the caller enqueues behind them in the meantime."""
+    (``FusedMapSampler.begin_sample``).  The sampling kernels store the sizes into pinned host memory themselves;
+    an event recorded behind them tells ``finish`` when, whatever the caller enqueues in the meantime."""
 
     def __init__(self, sampler, pending):
         self._sampler, self._pending = sampler, pending
@@ -142,17 +158,14 @@ class PendingBatch:
         self.outer_n_dst_bound = int(bptr[H - 1].numel()) - 1
         self.outer_fanout = int(sampler.fanouts[0])
         self.redone = False
-        dev = counts.device
-        main = torch.cuda.current_stream(dev)
-        side = sampler._side_stream(dev)
-        sampled = torch.cuda.Event()
-        sampled.record(main)
-        side.wait_event(sampled)
-        self._host = torch.empty(counts.numel(), dtype=torch.int32, pin_memory=True)
-        with torch.cuda.stream(side):
-            self._host.copy_(counts, non_blocking=True)
-            self._arrived = torch.cuda.Event()
-            self._arrived.record(side)
+        self._arrived = torch.cuda.Event()
+        self._arrived.record(torch.cuda.current_stream(counts.device))
+
+    def __del__(self):  # a batch that was begun and dropped: its host words go back to the sampler
+        try:
+            self._pending["host"].busy = False
+        except Exception:  # noqa: BLE001 -- interpreter shutdown
+            pass
 
     def finish(self):
         """The second half: wait for the sizes, then ``(input_nodes, output_nodes, blocks)`` as ``sample_blocks``
@@ -161,7 +174,7 @@ class PendingBatch:
         kernels never leave their bounds)."""
         outer_ptr = self.outer_edge_ptr.data_ptr()
         self._arrived.synchronize()
-        result = self._sampler._finish_fused(self._pending, self._host.tolist())
+        result = self._sampler._finish_fused(self._pending, self._pending["host"].read())
         self.redone = result[2][0].edge_ptr.data_ptr() != outer_ptr
         return result
 
@@ -219,7 +232,8 @@ class FusedMapSampler:
         self.output_nodes = None
         self._states = {}       # shape of a mini-batch -> _ShapeState
         self._side = None        # second stream of iter_batches
-        self._pinned_counts = None  # host buffer of the per-batch size read-back
+        self._host_counts = []   # pinned words for the per-batch size read-back, handed out in turn (_HostCounts)
+        self._host_turn = 0
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
         self.edge_ptr, self.edge_src, self.edge_dst = edge_ptr, edge_src, edge_dst
@@ -283,11 +297,30 @@ class FusedMapSampler:
         if caps is not None:
             slots = min(slots, max(lib.fgl_idmap_slots(2 * state.nodes_seen[-1]), lib.fgl_idmap_slots(n_seeds)))
         if self.graph_slots and caps is not None:  # steady state only: the worst-case plan (first batch, redo) runs eagerly
-            out = self._replay(state, plan, slots, seeds, stream_base)
+            out, host = self._replay(state, plan, slots, seeds, stream_base)
         else:
+            host = self._take_host_counts(3 * len(hop_fanouts) + 2)
             out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
-                                          keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order)
-        return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state)
+                                          keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
+                                          readback=host.words)
+        return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state, host=host)
+
+    def _take_host_counts(self, n_words, ring=8):
+        """Pinned words for one mini-batch's sizes: the next of a small ring that is not waiting to be read (a batch
+        begun and not finished keeps its own); a fresh allocation if all are."""
+        if self._host_counts and self._host_counts[0].words.numel() != n_words:
+            self._host_counts = []
+        for _ in range(len(self._host_counts)):
+            h = self._host_counts[self._host_turn % len(self._host_counts)]
+            self._host_turn += 1
+            if not h.busy:
+                h.busy = True
+                return h
+        h = _HostCounts(n_words)
+        h.busy = True
+        if len(self._host_counts) < ring:
+            self._host_counts.append(h)
+        return h
 
     def _replay(self, state, plan, slots, seeds, stream_base):
         """Graph mode: copy the seeds and the random-stream offset into the turn's slot, replay its graph."""
@@ -310,18 +343,19 @@ class FusedMapSampler:
         plan.empty_slots = None
         slot["graph"].replay()
         plan.empty_slots = slots
-        return slot["out"]
+        return slot["out"], slot["host"]
 
     def _capture(self, plan, slots, dev):
         hop_fanouts = list(reversed(self.fanouts))
         slot = dict(seeds=torch.zeros(plan.n_seeds, dtype=torch.int32, device=dev),
-                    offset=torch.zeros(1, dtype=torch.int32, device=dev))
+                    offset=torch.zeros(1, dtype=torch.int32, device=dev),
+                    host=_HostCounts(3 * len(hop_fanouts) + 2))  # (the slot's own: rewritten by every replay, like its outputs)
 
         def enqueue():
             # stream_base 0: the slot's offset carries the mini-batch's stream number
             return ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, slot["seeds"], self.rng_seed, 0,
                                            keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
-                                           stream_offset=slot["offset"])
+                                           stream_offset=slot["offset"], readback=slot["host"].words)
 
         cur = torch.cuda.current_stream(dev)
         warm = torch.cuda.Stream(device=dev)  # default priority
@@ -344,7 +378,7 @@ class FusedMapSampler:
         if status & (ops.L.STATUS_TABLE_FULL | ops.L.STATUS_UNIQ_OVERFLOW) and pending["caps"] is not None:
             state.nodes_seen = None
             pending = self._launch_fused(pending["seeds"], pending["stream_base"], worst_case=True, state=state)
-            c = self._read_counts(pending["out"][4])
+            c = self._read_counts(pending)
             status = c[2 * H + 1]
         if status:
             ops._raise_status(status, "sample_blocks")
@@ -387,17 +421,14 @@ class FusedMapSampler:
         self.batches += 1
         return PendingBatch(self, self._launch_fused(seeds, stream_base))
 
-    def _read_counts(self, counts):
-        """The batch's sizes on the host: one copy into a pinned buffer that the sampler keeps, one wait."""
-        if self._pinned_counts is None or self._pinned_counts.numel() != counts.numel():
-            self._pinned_counts = torch.empty(counts.numel(), dtype=torch.int32, pin_memory=True)
-        self._pinned_counts.copy_(counts, non_blocking=True)
-        torch.cuda.current_stream(counts.device).synchronize()
-        return self._pinned_counts.tolist()
+    def _read_counts(self, pending):
+        """The batch's sizes on the host: the kernels stored them into pinned memory, so one wait for the stream."""
+        torch.cuda.current_stream(pending["out"][4].device).synchronize()
+        return pending["host"].read()
 
     def _sample_fused(self, seeds, stream_base):
         pending = self._launch_fused(seeds, stream_base)
-        return self._finish_fused(pending, self._read_counts(pending["out"][4]))  # the one host synchronisation of the mini-batch
+        return self._finish_fused(pending, self._read_counts(pending))  # the one host synchronisation of the mini-batch
 
     def _side_stream(self, dev):
         if self._side is None:
@@ -425,21 +456,21 @@ class FusedMapSampler:
             side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
             with torch.cuda.stream(side):
                 pending = self._launch_fused(seeds, stream_base)
-                host = torch.empty(3 * H + 2, dtype=torch.int32, pin_memory=True)
-                host.copy_(pending["out"][4], non_blocking=True)
                 done = torch.cuda.Event()
                 done.record(side)
-            return pending, host, done
+            return pending, done
 
         def finish(item):
-            pending, host, done = item
+            pending, done = item
             done.synchronize()
             with torch.cuda.stream(side):  # a batch that outgrew its buffers is redone here, synchronously
-                result = self._finish_fused(pending, host.tolist())
+                result = self._finish_fused(pending, pending["host"].read())
                 redo = torch.cuda.Event()
                 redo.record(side)
             main.wait_event(redo)
-            for t in (result[0],) + tuple(x for b in result[2] for x in (b.edge_ptr, b.src_local, b.src_global) if x is not None):
+            for t in (result[0],) + tuple(x for b in result[2]
+                                          for x in (b.edge_ptr, b.src_local, b.src_global) + tuple(b._transposed or ())
+                                          if x is not None):
                 t.record_stream(main)  # allocated on the side stream, consumed on the caller's
             return result
 

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FGL_ABI_VERSION 10
+#define FGL_ABI_VERSION 11
 
 enum fgl_error {
     FGL_OK = 0,
@@ -243,6 +243,9 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * longest row of hop h's transposed block if that exceeds FGL_SHORT_ROW_ENTRIES, else some value not above it
  * (zero for hops whose transposed block is not built) -- read back with the sizes, it is the host bound that
  * fgl_aggregate's longest_row_max wants.
+ * d_readback (may be NULL): 3*n_hops+2 int32 words of host memory that the device can write (hipHostMalloc); the
+ * launch that makes the last of the counts final stores a copy of d_counts there, so the host's one read per
+ * mini-batch is a wait for the stream (or for an event recorded behind the call) and a load, with no copy to enqueue.
  *
  * Transposed blocks (the column-major companions that the backward kernels gather over, see fgl_block_transpose):
  * t_ptr / t_dst / t_edge are NULL, or arrays of n_hops pointers of which any may be NULL.  Where t_ptr[h] is given
@@ -268,7 +271,7 @@ int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const int32_t* d_in
                       void* d_table, int64_t table_slots, int32_t* d_uniq, int64_t uniq_capacity,
                       int32_t* const* block_ptr, int32_t* const* src_local, int32_t* const* src_global,
                       int32_t* const* t_ptr, int32_t* const* t_dst, int32_t* const* t_edge,
-                      int32_t* d_counts, void* d_ws, size_t ws_bytes, void* stream);
+                      int32_t* d_counts, int32_t* d_readback, void* d_ws, size_t ws_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * block transpose -- the column-major companion of a block CSR, which turns the

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_pure_host_entry_points():
     lib = fastgl.lib()
-    assert lib.fgl_abi_version() == 10
+    assert lib.fgl_abi_version() == 11
     assert fastgl.table_size(40960, 2) == 131072
     assert fastgl.table_size(8110080, 2) == 16777216
     assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25

@@ -187,6 +187,35 @@ def test_transposed_blocks_come_with_the_sample(cuda, oracle, small_graph, which
             assert all(b._transposed is not None for b in blocks)
 
 
+@pytest.mark.parametrize("id_order", ["first", "arrival"])
+@pytest.mark.parametrize("hops", [(), (0, 1), (0, 1, 2)])
+def test_counts_written_where_the_host_reads_them(cuda, small_graph, hops, id_order):
+    """`readback` of the all-hops call: pinned host words that the call's own kernels fill with a copy of its count
+    array once the last count is final (the last hop's node total, or the longest row of the last hop's transposed
+    block when that is built) -- equal to the device array after a wait for the stream, batch after batch; stale
+    contents of the words never survive."""
+    import torch
+    from fastgl import ops
+    print("sample_blocks readback hops=%s %s" % (hops, id_order), flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    n = indptr.size - 1
+    rng = np.random.default_rng(5)
+    plan = ops.BlocksPlan(n, 700, [5, 10, 15], cuda, transpose_hops=hops)
+    host = torch.empty(3 * 3 + 2, dtype=torch.int32, pin_memory=True)
+    for it in range(3):
+        host.fill_(-7)
+        seeds = dev_i32(rng.permutation(n)[:700].astype(np.int32), cuda)
+        out = ops.sample_blocks_fused(plan, ptr, idx, seeds, 9, 64 * it, id_order=id_order, readback=host)
+        torch.cuda.current_stream(cuda).synchronize()
+        got, want = host.tolist(), out[4].cpu().tolist()
+        assert got == want and want[2 * 3 + 1] == 0 and want[0] == 700 and want[3] > want[0]
+        for h in range(3):
+            assert h in hops or want[2 * 3 + 2 + h] == 0
+    with pytest.raises(RuntimeError, match="pinned"):
+        ops.sample_blocks_fused(plan, ptr, idx, seeds, 9, 0, readback=torch.empty(11, dtype=torch.int32))
+
+
 def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     import fastgl
     print("sample_blocks int32 ptr", flush=True)
