@@ -1331,10 +1331,20 @@ static int launch_agg_bundle(int mode, bool long_rows_possible, unsigned gy, hip
 #define FGL_SPLIT_TARGET_WAVES 4096  // groups per row are doubled until the launch has this many waves
 #endif
 // Lists of at most this many entries on average (per row, from the caller's entry count) are taken several
-// rows at a time (aggregate_bundle_kernel).
+// rows at a time (aggregate_bundle_kernel).  Launches of a million rows and more bundle up to longer averages:
+// there the one-group-per-row kernel falls behind (2 M rows of 2.1 entries, 256 bf16 columns: 614 us against
+// 436 us bundled; 1 M rows: 255 against 217; at 3 entries per row 656 against 552 and 272 against 276), while
+// below half a million rows bundling lists of more than two entries costs a few per cent.
 #ifndef FGL_BUNDLE_MAX_AVG_ENTRIES
 #define FGL_BUNDLE_MAX_AVG_ENTRIES 2
 #endif
+static inline bool lists_are_short(int64_t n_entries, int64_t n_rows)
+{
+    if (n_entries < 0 || n_rows < 1024) return false;
+    // twice the largest average that is bundled, so that 2.5 can be said
+    const int64_t twice = n_rows >= ((int64_t)1 << 21) ? 8 : n_rows >= ((int64_t)1 << 20) ? 5 : 2 * FGL_BUNDLE_MAX_AVG_ENTRIES;
+    return 2 * n_entries <= twice * n_rows;
+}
 
 template <typename T, int VEC>
 static int launch_agg_vec(int mode, int64_t longest_row_max, int64_t n_entries_max, hipStream_t stream, const AggArgs& g)
@@ -1343,8 +1353,7 @@ static int launch_agg_vec(int mode, int64_t longest_row_max, int64_t n_entries_m
     int lpr = 8;
     while (lpr < 64 && lpr < lanes_needed) lpr <<= 1;
     // many rows of short lists (a transposed block): several rows per lane group
-    const bool short_lists = n_entries_max >= 0 && g.n_rows_max >= 1024 &&
-                             n_entries_max <= (int64_t)FGL_BUNDLE_MAX_AVG_ENTRIES * g.n_rows_max &&
+    const bool short_lists = lists_are_short(n_entries_max, g.n_rows_max) &&
                              (mode != FGL_AGG_EDGE || (g.unit_dim % VEC == 0 && lanes_needed <= 64));
     // rows wider than one 64-lane group that fill their groups to less than 90 %: flat mapping
     // (602 fp32 columns: 100 -> 80 us; 602 bf16: 59 -> 44 us forward, 135 -> 84 us on the transposed block)
