@@ -108,13 +108,25 @@ void* grown(torch::Tensor& buf, size_t bytes, const torch::Tensor& like)
     return buf.data_ptr();
 }
 
-// {size, status} of the call that has just been enqueued.  The call's own launches wrote both words into the pinned
-// buffer (device-writable host memory), so there is no copy to enqueue: wait for the stream, read.  A non-zero
-// status word is cleared on the device again (the kernels only ever or into it).
-// (Polling hipStreamQuery instead of the blocking wait was measured: 0.34 -> 0.40 ms per three-hop mini-batch.)
+// {size, status} of a call.  The call's own launches write both words into the pinned buffer (device-writable host
+// memory), so there is no copy to enqueue: expect() marks the words as pending before the call is enqueued, and
+// read_back() looks at them until they have been overwritten -- which the launch that knows the size does when it
+// starts, so the host is back at work while the call's last kernel is still running (and falls back to a stream
+// wait after a few milliseconds).  A non-zero status word is cleared on the device again (the kernels only ever
+// or into it).
+// (Polling hipStreamQuery instead was measured: 0.34 -> 0.40 ms per three-hop mini-batch.)
+constexpr int32_t kPendingWord = -1;  // no size and no status word is all ones
+
+int32_t* expect(CallState& st)
+{
+    int32_t* h = st.host.data_ptr<int32_t>();
+    h[0] = h[1] = kPendingWord;
+    return h;
+}
+
 std::pair<int64_t, uint32_t> read_back(CallState& st, void* stream)
 {
-    TORCH_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)) == hipSuccess, "fastgl: waiting for the call's sizes failed");
+    ok(fgl_wait_words(st.host.data_ptr<int32_t>(), 2, kPendingWord, stream, 5000));
     const volatile int32_t* h = st.host.data_ptr<int32_t>();
     const std::pair<int64_t, uint32_t> out{h[0], (uint32_t)h[1]};
     if (out.second != 0) st.meta.zero_();
@@ -195,7 +207,7 @@ std::vector<torch::Tensor> sample_node(torch::Tensor src_edges, torch::Tensor ds
     ok(fgl_sample_node(edge_ptr.data_ptr(), edge_ptr.scalar_type() == torch::kInt64, src_edges.data_ptr<int32_t>(),
                        edge_ptr.size(0) - 1, seed_nodes.data_ptr<int32_t>(), n_seeds, nullptr, neighbor_num, g_rng_seed.load(),
                        g_rng_calls.fetch_add(1), src_out.data_ptr<int32_t>(), dst_out.data_ptr<int32_t>(), block_ptr.data_ptr<int32_t>(),
-                       meta, reinterpret_cast<uint32_t*>(meta) + 1, st.host.data_ptr<int32_t>(), ws, (size_t)st.ws.numel(), stream));
+                       meta, reinterpret_cast<uint32_t*>(meta) + 1, expect(st), ws, (size_t)st.ws.numel(), stream));
     const auto back = read_back(st, stream);  // the read-back of sample.cu:202
     raise_status(back.second, "sample_node");
     // (the edge count as a device tensor, as the reference returns it: the last entry of the block's row pointer)
@@ -242,7 +254,7 @@ std::vector<torch::Tensor> transfer_edge_id(torch::Tensor src_edges, torch::Tens
     // own destination list) nor leaves anything in it
     ok(fgl_idmap_transfer(table, slots, dst_edges_unique.data_ptr<int32_t>(), n_dst, src_edges.data_ptr<int32_t>(),
                           dst_edges.data_ptr<int32_t>(), n_edges, uniq.data_ptr<int32_t>(), capacity,
-                          FGL_IDMAP_ORDERED | FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY, meta, status, st.host.data_ptr<int32_t>(), ws,
+                          FGL_IDMAP_ORDERED | FGL_IDMAP_FINAL | FGL_IDMAP_LEAVE_TABLE_EMPTY, meta, status, expect(st), ws,
                           (size_t)st.ws.numel(), stream));
     st.empty_slots = known_empty;
     const auto back = read_back(st, stream);  // the read-back of id_map.cu:454,491

@@ -5,6 +5,8 @@
 // 256 threads x 8 consecutive items (32 contiguous bytes per lane, 2 KiB per wave).
 #include <stdarg.h>
 
+#include <chrono>
+
 #include "fgl_common.hpp"
 #include "fgl_kernels.hpp"
 
@@ -198,6 +200,34 @@ using namespace fgl;
 
 FGL_EXPORT int fgl_abi_version(void) { return FGL_ABI_VERSION; }
 FGL_EXPORT const char* fgl_last_error(void) { return g_err; }
+
+// Host side of a d_readback: the caller stored `pending` into every word before it enqueued the call; the launch
+// that knows the sizes overwrites them.  Looking at the words themselves returns as soon as they have landed --
+// which is before that launch has finished, and without the wake-up of a stream wait.  Bounded: past spin_limit_us
+// the stream is waited for instead, and words that are still pending then are an error.
+FGL_EXPORT int fgl_wait_words(const int32_t* h_words, int n_words, int32_t pending, void* stream, int64_t spin_limit_us)
+{
+    FGL_REQUIRE(h_words != nullptr && n_words >= 1, "wait_words: nothing to wait for");
+    const volatile int32_t* w = h_words;
+    auto all_there = [&]() {
+        for (int i = 0; i < n_words; ++i)
+            if (w[i] == pending) return false;
+        return true;
+    };
+    if (spin_limit_us > 0) {
+        const auto t0 = std::chrono::steady_clock::now();
+        for (;;) {
+            for (int k = 0; k < 256; ++k) {
+                if (all_there()) return FGL_OK;
+                __builtin_ia32_pause();
+            }
+            if (std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() > spin_limit_us) break;
+        }
+    }
+    FGL_REQUIRE(hipStreamSynchronize(as_stream(stream)) == hipSuccess, "wait_words: waiting for the stream failed");
+    FGL_REQUIRE(all_there(), "wait_words: the stream is idle and the words were not written");
+    return FGL_OK;
+}
 
 FGL_EXPORT size_t fgl_exclusive_sum_workspace_bytes(int64_t n_max) { return scan_workspace_bytes(n_max < 0 ? 0 : n_max); }
 

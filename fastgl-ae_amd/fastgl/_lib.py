@@ -48,6 +48,7 @@ SIGNATURES = {
     "fgl_idmap_map_src": (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _sz, _vp]),
     "fgl_idmap_transfer": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fgl_idmap_lookup": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp]),
+    "fgl_wait_words": (_i32, [_vp, _i32, _i32, _vp, _i64]),
     "fgl_sample_blocks_plan": (_i32, [_i64, _i64, _vp, _i32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]),
     "fgl_sample_blocks": (_i32, [_vp, _i32, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _u64, _u32, _vp, _i32, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -131,13 +131,26 @@ class _HostCounts:
     """Pinned host words that the kernels of a mini-batch write its sizes into (``readback`` of
     ``ops.sample_blocks_fused``).  A sampler keeps a few and hands them out in turn; one that is still waiting to be
     read is never handed out again."""
+    PENDING = -1  # no count and no status word is all ones
 
     def __init__(self, n_words):
         self.words = torch.empty(n_words, dtype=torch.int32, pin_memory=True)
         self.busy = False
+        self.abandoned = False  # handed out, never read: its kernels may still be about to write
+        self.stream = None
+
+    def expect(self, stream):
+        """Before the call is enqueued on ``stream``: every word pending."""
+        self.words.fill_(self.PENDING)
+        self.stream = stream
+        return self.words
 
     def read(self):
-        """The words as a list; the caller has waited for the kernels that write them."""
+        """Waits until the kernels have overwritten every word -- the launch that makes the last count final does so
+        when it starts, so this returns while that launch is still running, without the wake-up of a stream wait
+        (bounded: after a few milliseconds the stream is waited for instead) -- and returns them as a list."""
+        ops.L.check(ops.L.lib().fgl_wait_words(self.words.data_ptr(), int(self.words.numel()), self.PENDING,
+                                               self.stream.cuda_stream, 5000))
         values = self.words.tolist()
         self.busy = False
         return values
@@ -145,8 +158,8 @@ class _HostCounts:
 
 class PendingBatch:
     """A mini-batch whose kernels are enqueued and whose sizes are still on the device
-    (``FusedMapSampler.begin_sample``).  The sampling kernels store the sizes into pinned host memory themselves;
-    an event recorded behind them tells ``finish`` when, whatever the caller enqueues in the meantime."""
+    (``FusedMapSampler.begin_sample``).  The sampling kernels store the sizes into pinned host memory themselves as
+    soon as the last of them is final; ``finish`` waits for those words, whatever the caller enqueues in the meantime."""
 
     def __init__(self, sampler, pending):
         self._sampler, self._pending = sampler, pending
@@ -158,12 +171,14 @@ class PendingBatch:
         self.outer_n_dst_bound = int(bptr[H - 1].numel()) - 1
         self.outer_fanout = int(sampler.fanouts[0])
         self.redone = False
-        self._arrived = torch.cuda.Event()
-        self._arrived.record(torch.cuda.current_stream(counts.device))
 
-    def __del__(self):  # a batch that was begun and dropped: its host words go back to the sampler
+    def __del__(self):
+        # a batch that was begun and dropped: its kernels may still be about to write its host words, so the sampler
+        # waits for them before it hands the words out again
         try:
-            self._pending["host"].busy = False
+            host = self._pending["host"]
+            if host.busy:
+                host.abandoned = True
         except Exception:  # noqa: BLE001 -- interpreter shutdown
             pass
 
@@ -173,7 +188,6 @@ class PendingBatch:
         ones -- anything computed from the ``outer_*`` arrays before is then void (it read valid memory, the
         kernels never leave their bounds)."""
         outer_ptr = self.outer_edge_ptr.data_ptr()
-        self._arrived.synchronize()
         result = self._sampler._finish_fused(self._pending, self._pending["host"].read())
         self.redone = result[2][0].edge_ptr.data_ptr() != outer_ptr
         return result
@@ -232,7 +246,7 @@ class FusedMapSampler:
         self.output_nodes = None
         self._states = {}       # shape of a mini-batch -> _ShapeState
         self._side = None        # second stream of iter_batches
-        self._host_counts = []   # pinned words for the per-batch size read-back, handed out in turn (_HostCounts)
+        self._host_counts = {}   # word count -> pinned words for the per-batch size read-back, handed out in turn (_HostCounts)
         self._host_turn = 0
 
     def set_graph(self, edge_ptr, edge_src, nodes_num=None, edge_dst=None):
@@ -302,24 +316,26 @@ class FusedMapSampler:
             host = self._take_host_counts(3 * len(hop_fanouts) + 2)
             out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
                                           keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
-                                          readback=host.words)
+                                          readback=host.expect(torch.cuda.current_stream(seeds.device)))
         return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state, host=host)
 
-    def _take_host_counts(self, n_words, ring=8):
-        """Pinned words for one mini-batch's sizes: the next of a small ring that is not waiting to be read (a batch
-        begun and not finished keeps its own); a fresh allocation if all are."""
-        if self._host_counts and self._host_counts[0].words.numel() != n_words:
-            self._host_counts = []
-        for _ in range(len(self._host_counts)):
-            h = self._host_counts[self._host_turn % len(self._host_counts)]
+    def _take_host_counts(self, n_words):
+        """Pinned words for one mini-batch's sizes: one of the sampler's that is not waiting to be read (a batch begun
+        and not finished keeps its own), a new one if all are.  They live as long as the sampler: kernels in flight
+        write into them."""
+        rows = self._host_counts.setdefault(n_words, [])
+        for _ in range(len(rows)):
+            h = rows[self._host_turn % len(rows)]
             self._host_turn += 1
+            if h.abandoned:  # (its batch was dropped unread: once its kernels have written, it is free again)
+                h.abandoned = False
+                h.read()
             if not h.busy:
                 h.busy = True
                 return h
         h = _HostCounts(n_words)
         h.busy = True
-        if len(self._host_counts) < ring:
-            self._host_counts.append(h)
+        rows.append(h)
         return h
 
     def _replay(self, state, plan, slots, seeds, stream_base):
@@ -341,6 +357,7 @@ class FusedMapSampler:
         if plan.empty_slots != slots:
             ops.L.check(ops.L.lib().fgl_idmap_reset(ops.L.ptr(plan.table), slots, ops.L.stream_handle()))
         plan.empty_slots = None
+        slot["host"].expect(torch.cuda.current_stream(seeds.device))
         slot["graph"].replay()
         plan.empty_slots = slots
         return slot["out"], slot["host"]
@@ -422,8 +439,7 @@ class FusedMapSampler:
         return PendingBatch(self, self._launch_fused(seeds, stream_base))
 
     def _read_counts(self, pending):
-        """The batch's sizes on the host: the kernels stored them into pinned memory, so one wait for the stream."""
-        torch.cuda.current_stream(pending["out"][4].device).synchronize()
+        """The batch's sizes on the host: the kernels store them into pinned memory, the host waits for the words."""
         return pending["host"].read()
 
     def _sample_fused(self, seeds, stream_base):
@@ -456,13 +472,9 @@ class FusedMapSampler:
             side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
             with torch.cuda.stream(side):
                 pending = self._launch_fused(seeds, stream_base)
-                done = torch.cuda.Event()
-                done.record(side)
-            return pending, done
+            return pending
 
-        def finish(item):
-            pending, done = item
-            done.synchronize()
+        def finish(pending):
             with torch.cuda.stream(side):  # a batch that outgrew its buffers is redone here, synchronously
                 result = self._finish_fused(pending, pending["host"].read())
                 redo = torch.cuda.Event()

@@ -89,6 +89,16 @@ enum fgl_zero_policy {
 int fgl_abi_version(void);
 const char* fgl_last_error(void);
 
+/* Host side of the d_readback arguments below (where the reference copies a count back with cudaMemcpy and waits:
+ * sample.cu:202, id_map.cu:454,491).  The caller stores `pending` -- a value that no size or status word can
+ * take, e.g. -1 -- into each of the n_words host words, enqueues the call, and waits here: the function returns
+ * when every word has been overwritten, which the device does as soon as the sizes are final -- before the
+ * call's last launch has finished, and without the wake-up latency of a stream wait.  It looks at the words for
+ * at most spin_limit_us microseconds (0: not at all), then waits for `stream` (the one the call went to) and
+ * reports words that are still pending as an error.  What the call wrote besides is ordered by the stream, as
+ * always: only the sizes are on the host early. */
+int fgl_wait_words(const int32_t* h_words, int n_words, int32_t pending, void* stream, int64_t spin_limit_us);
+
 /* ---------------------------------------------------------------------------------
  * exclusive_sum  -- replaces fastgl.exclusive_sum (cuda_operators/aggregate_acc.cpp:514-520,
  * utilis.cu:17-41): out[0..n] = exclusive prefix sums of in[0..n-1], out[n] = total.

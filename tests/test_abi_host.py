@@ -36,6 +36,10 @@ def test_pure_host_entry_points():
     assert lib.fgl_idmap_slots(0) == 64 and lib.fgl_idmap_slots(33) == 128 and lib.fgl_idmap_slots(8650752) == 1 << 25
     assert lib.fgl_idmap_table_bytes(1 << 25) == 8 << 25
     assert lib.fgl_exclusive_sum_workspace_bytes(10) > 0
+    # the host side of a read-back, where no device is involved: words that are there already, and bad arguments
+    words = (C.c_int32 * 3)(5, 0, 7)
+    assert lib.fgl_wait_words(words, 3, -1, None, 1000) == 0
+    assert lib.fgl_wait_words(words, 0, -1, None, 1000) != 0 and lib.fgl_wait_words(None, 3, -1, None, 1000) != 0
 
 
 def test_static_scratch_holds_the_workspace_of_its_largest_call():

@@ -216,6 +216,45 @@ def test_counts_written_where_the_host_reads_them(cuda, small_graph, hops, id_or
         ops.sample_blocks_fused(plan, ptr, idx, seeds, 9, 0, readback=torch.empty(11, dtype=torch.int32))
 
 
+def test_waiting_for_the_words_and_dropped_batches(cuda, oracle, small_graph):
+    """The host side of the read-back: `fgl_wait_words` returns once the kernels have overwritten every pending
+    word (also with no spinning at all: the stream wait), and a batch that was begun and dropped unread never
+    hands its sizes to the batch that gets its host words next."""
+    import gc
+    import torch
+    import fastgl
+    from fastgl import ops
+    print("wait_words / dropped pending batches", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    n = indptr.size - 1
+    rng = np.random.default_rng(6)
+    plan = ops.BlocksPlan(n, 500, [5, 10, 15], cuda, transpose_hops=(0, 1))
+    host = torch.empty(11, dtype=torch.int32, pin_memory=True)
+    lib = fastgl.lib()
+    stream = torch.cuda.current_stream(cuda).cuda_stream
+    for spin_us in (5000, 0):
+        host.fill_(-1)
+        seeds = dev_i32(rng.permutation(n)[:500].astype(np.int32), cuda)
+        out = ops.sample_blocks_fused(plan, ptr, idx, seeds, 9, 0, readback=host)
+        assert lib.fgl_wait_words(host.data_ptr(), 11, -1, stream, spin_us) == 0
+        got = host.tolist()
+        assert -1 not in got and got == out[4].cpu().tolist()
+    torch.cuda.synchronize()
+    host.fill_(-1)  # nothing enqueued that would write them: reported after the stream wait, not waited for for ever
+    assert lib.fgl_wait_words(host.data_ptr(), 11, -1, stream, 100) != 0
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=3).set_graph(ptr, idx)
+    batches = [rng.permutation(n)[:600].astype(np.int32) for _ in range(6)]
+    for it, seeds in enumerate(batches):
+        if it % 2 == 0:
+            sampler.begin_sample(dev_i32(seeds, cuda))  # dropped at once, unread
+            gc.collect()
+        else:
+            got = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+            check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], got, 3, it * 64)
+    assert len(sampler._host_counts[11]) <= 2
+
+
 def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     import fastgl
     print("sample_blocks int32 ptr", flush=True)
