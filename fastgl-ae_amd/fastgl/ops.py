@@ -58,6 +58,25 @@ def _raise_status(bits: int, where: str):
 # ---------------------------------------------------------------------------------------
 # drop-in operators
 # ---------------------------------------------------------------------------------------
+_host_words = {}
+
+
+def _expect_sizes(dev, stream):
+    """Two pinned host words per (device, stream) for a call's ``{size, status}``, marked pending: the call's kernels
+    store both there themselves (no copy to enqueue), ``_sizes`` waits for them."""
+    key = (torch.device(dev).index, stream)
+    h = _host_words.get(key)
+    if h is None:
+        h = _host_words[key] = torch.empty(2, dtype=torch.int32, pin_memory=True)
+    h.fill_(-1)  # (no size and no status word is all ones)
+    return h
+
+
+def _sizes(h, stream):
+    L.check(L.lib().fgl_wait_words(h.data_ptr(), 2, -1, stream, 5000))
+    return h.tolist()
+
+
 def sample_node(src_edges, dst_edges, edge_ptr, seed_nodes, dst_nodes, neighbor_num):
     """fastgl.sample_node (aggregate_acc.cpp:491-512): ``-> [src_out, dst_out, edges_num]``.
 
@@ -85,11 +104,13 @@ def sample_node(src_edges, dst_edges, edge_ptr, seed_nodes, dst_nodes, neighbor_
         ws = L.workspace(ws_bytes, dev)
         stream_id = _rng_state["calls"] & 0xFFFFFFFF
         _rng_state["calls"] += 1
+        st = L.stream_handle()
+        host = _expect_sizes(dev, st)
         L.check(lib.fgl_sample_node(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(src_edges),
                                     int(edge_ptr.size(0)) - 1, L.ptr(seed_nodes), n_seeds, None, fanout,
                                     _rng_state["seed"], stream_id, L.ptr(src_out), L.ptr(dst_out), L.ptr(block_ptr),
-                                    meta.data_ptr(), meta.data_ptr() + 4, None, L.ptr(ws), ws.numel(), L.stream_handle()))
-        n_edges, status = meta.tolist()  # the host read-back the reference also does (sample.cu:202)
+                                    meta.data_ptr(), meta.data_ptr() + 4, host.data_ptr(), L.ptr(ws), ws.numel(), st))
+        n_edges, status = _sizes(host, st)  # the host read-back the reference also does (sample.cu:202)
     _raise_status(status, "sample_node")
     edges_num = meta[:1]
     out = [src_out[:n_edges], dst_out[:n_edges], edges_num]
@@ -135,14 +156,15 @@ def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_it
         if known_empty < slots:
             L.check(lib.fgl_idmap_reset(L.ptr(table), slots, st))
         _tables[key] = (table, 0)
+        host = _expect_sizes(dev, st)
         # destination ids in, then three passes over the edges (the destination half rides on the first); the last
         # writes nothing back into the table (no later call looks these ids up) and empties it
         L.check(lib.fgl_idmap_transfer(L.ptr(table), slots, L.ptr(dst_edges_unique), n_dst, L.ptr(src_edges), L.ptr(dst_edges),
                                        n_edges, L.ptr(uniq), capacity,
                                        L.IDMAP_ORDERED | L.IDMAP_FINAL | L.IDMAP_LEAVE_TABLE_EMPTY, meta.data_ptr(), status_ptr,
-                                       None, L.ptr(ws), ws.numel(), st))
+                                       host.data_ptr(), L.ptr(ws), ws.numel(), st))
         _tables[key] = (table, max(known_empty, slots))
-        n_total, status = meta.tolist()  # host read-back, as id_map.cu:454,491
+        n_total, status = _sizes(host, st)  # host read-back, as id_map.cu:454,491
     _raise_status(status, "transfer_edge_id")
     return [src_edges, dst_edges, uniq[:n_total]]
 
