@@ -363,20 +363,24 @@ def test_arrival_order_equals_oracle_after_canonical_sort(cuda, oracle, small_gr
                 assert np.array_equal(uniq[src_l], b.src_global.cpu().numpy())
 
 
-def test_pipelined_iterator_equals_batch_by_batch(cuda, oracle, small_graph):
-    """iter_batches samples ahead on a second stream; every batch must equal the oracle's (and hence
-    sample_blocks'), also while the consumer keeps the main stream busy."""
+@pytest.mark.parametrize("prefetch", [1, 2, 3])
+def test_pipelined_iterator_equals_batch_by_batch(cuda, oracle, small_graph, prefetch):
+    """iter_batches samples up to `prefetch` mini-batches ahead, each on a stream of its own with its own table and
+    scratch; every batch must equal the oracle's (and hence sample_blocks'), also while the consumer keeps the main
+    stream busy, for more batches than lanes and fewer."""
     import fastgl
-    print("sample_blocks pipelined iterator", flush=True)
+    print("sample_blocks pipelined iterator, %d in flight" % prefetch, flush=True)
     indptr, indices = small_graph
     ptr, idx = load_graph(cuda, indptr, indices)
     rng = np.random.default_rng(77)
-    batches = [rng.permutation(indptr.size - 1)[:700].astype(np.int32) for _ in range(6)]
+    batches = [rng.permutation(indptr.size - 1)[:700].astype(np.int32) for _ in range(11)]
     batches[3] = np.argsort(-np.diff(indptr))[:700].astype(np.int32)  # outgrows the buffers sized by experience
+    sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=21).set_graph(ptr, idx)
+    assert len(list(sampler.iter_batches([dev_i32(batches[0], cuda)], prefetch=prefetch))) == 1
     sampler = fastgl.FusedMapSampler([15, 10, 5], rng_seed=21).set_graph(ptr, idx)
     feat = torch.randn(indptr.size - 1, 64, device=cuda)
     n = 0
-    for i, got in enumerate(sampler.iter_batches(dev_i32(b, cuda) for b in batches)):
+    for i, got in enumerate(sampler.iter_batches((dev_i32(b, cuda) for b in batches), prefetch=prefetch)):
         check_blocks(oracle, indptr, indices, batches[i], [15, 10, 5], got, 21, i * 64)
         b0 = got[2][0]
         out = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")  # main-stream consumer
@@ -412,11 +416,13 @@ def test_graph_replay_equals_the_oracle_batch_after_batch(cuda, oracle, small_gr
         out = fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")  # eager work between replays
         want = oracle.aggregate(b0.edge_ptr.cpu().numpy(), b0.src_global.cpu().numpy(), feat.cpu().numpy(), "mean", 1)
         assert np.abs(out.cpu().numpy() - want).max() < 1e-5
-        state = sampler._state_for(seeds_dev[i])
-        if state.graphs is not None:
-            captures.add(state.graphs[0])
-    assert state.graphs is not None and all(slot is not None for slot in state.graphs[2])  # graphs were used
-    assert len(captures) >= 2  # ... and captured anew after the plan changed
+        for lane, state in enumerate(sampler._states.values()):  # (one state per mini-batch in flight when pipelined)
+            if state.graphs is not None:
+                captures.add((lane, state.graphs[0]))
+    states = list(sampler._states.values())
+    assert len(states) == (2 if pipelined else 1)
+    assert all(st.graphs is not None and any(slot is not None for slot in st.graphs[2]) for st in states)  # graphs were used
+    assert len(captures) >= len(states) + 1  # ... and captured anew after a plan changed
 
 
 @pytest.mark.parametrize("fused", [True, False])
@@ -660,7 +666,7 @@ def test_a_short_last_batch_keeps_what_the_full_batches_learned(cuda, oracle, sm
             check_blocks(oracle, indptr, indices, batches[i], [15, 10, 5], got, 2, i * 64)
             full = sampler._state_for(seeds_dev[0])
             plans_full.append({k: id(v) for k, v in full.plans.items()})
-        assert len(sampler._states) == 2
+        assert len({key[:-1] for key in sampler._states}) == 2  # (two shapes; when pipelined, each on both lanes)
         full, short = sampler._state_for(seeds_dev[0]), sampler._state_for(seeds_dev[3])
         assert full.nodes_seen is not None and short.nodes_seen is not None and full.nodes_seen[0] == 600 and short.nodes_seen[0] == 150
         # the full-size shape's sized-by-experience plan of batch 2 is still the one in use at the end
