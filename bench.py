@@ -622,8 +622,9 @@ def main():
     ap.add_argument("--extras", choices=["on", "off"], default="on",
                     help="workload c3 only: also run the aggregation microbench (key c4) and the very large shape (key c5) and "
                          "attach their compact records to the line")
-    ap.add_argument("--overlap", action="store_true",
-                    help="also time the steps with the next batch sampled on a second stream (reported as ms_per_step_overlapped)")
+    ap.add_argument("--prefetch", type=int, default=2,
+                    help="mini-batches that the sampler keeps in flight ahead of the one being aggregated "
+                         "(FusedMapSampler.iter_batches; 0: one mini-batch at a time only)")
     ap.add_argument("--c4-eager", action="store_true",
                     help="workload c4: time launches made one by one through the Python binding instead of replaying them "
                          "from a captured graph (the interval then includes the host's cost per call)")
@@ -683,8 +684,10 @@ def main():
 def light_summary(rec):
     """A workload's record cut down to what rides on another workload's line."""
     r = rec["roofline"]
-    return {"workload": rec["config"]["workload"], "value": rec["value"], "unit": rec["unit"], "dtype": rec["dtype"],
-            "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"], "stages_ms": rec["stages_ms"],
+    return {"workload": rec["config"]["workload"], "value": rec["value"], "value_one_at_a_time": rec["value_one_at_a_time"],
+            "unit": rec["unit"], "dtype": rec["dtype"],
+            "steps": rec["steps"], "warmup": rec["warmup"], "ms_per_step": rec["ms_per_step"],
+            "ms_per_step_one_at_a_time": rec["ms_per_step_one_at_a_time"], "stages_ms": rec["stages_ms"],
             "sampled_edges_per_step": rec["config"]["sampled_edges_per_step"], "graph_edges": rec["config"]["graph_edges"],
             "roofline": {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "kernel", "bytes_per_launch", "us_per_launch")},
             "random_read_Gps": rec["random_read_Gps"]}
@@ -931,9 +934,16 @@ def run_graph_workload(args, workload, light=False):
             log("reference call pattern through the compiled module: %.3g sampled edges/s (%.3f ms per mini-batch)"
                 % (value_drop_in, ms_di))
 
-    # ---- optional: the same steps with sampling of batch i+1 overlapped with aggregation of batch i ----
-    ms_overlapped = None
-    if args.overlap and not light:
+    # ---- the sampler as a prefetching iterator (FusedMapSampler.iter_batches, the role of the DataLoader that the
+    # reference plugs its sampler into: train_fastgl.py:109-122,248-258, prefetch_factor 2): `prefetch` mini-batches are
+    # sampled ahead, each on a stream of its own, so that the small hops of one -- latency chains on a mostly idle
+    # chip -- run under the large kernels of another and under the aggregation.  Two timings, each a pass of its own
+    # (pipeline fill and drain inside the interval), wall clock between two device synchronisations:
+    #   the sampling stage alone (nothing else on the GPU, every mini-batch's read-back included) -> edges per second;
+    #   whole steps (sampling + the aggregation of every block, forward and backward)             -> ms per step.
+    pipelined = None
+    K = args.steps
+    if args.prefetch > 0:
         def aggregate_only(blocks):
             b0 = blocks[0]
             fastgl.aggregate(b0.edge_ptr, b0.src_global, feat, mode="mean", zero_policy="zeros")
@@ -945,16 +955,35 @@ def run_graph_workload(args, workload, light=False):
                 t_ptr, t_idx = b.transposed()
                 fastgl.aggregate(t_ptr, t_idx, grad[:b.num_dst_nodes()], mode="colmean_ptr", zero_policy="zeros",
                                  col_norm=b.edge_ptr)
-        batches = [train[(i % n_batches) * B:(i % n_batches) * B + B] for i in range(args.warmup + args.steps)]
+
+        pipe = fastgl.FusedMapSampler(w["fanouts"], rng_seed=0, id_order=args.id_order).set_graph(edge_ptr, edge_src)
+        batch_of = lambda i: train[(i % n_batches) * B:(i % n_batches) * B + B]
+        for _, _, blocks in pipe.iter_batches([batch_of(i) for i in range(max(args.warmup, 2 * args.prefetch))], prefetch=args.prefetch):
+            aggregate_only(blocks)  # warm-up: every lane has learned its buffer sizes
+        first = pipe.batches
+        n_sampling = max(K, 100 if not light else K)
         torch.cuda.synchronize()
-        for i, (_, _, blocks) in enumerate(sampler.iter_batches(batches)):
-            if i == args.warmup:
-                torch.cuda.synchronize()
-                t_ov = time.perf_counter()
+        t0 = time.perf_counter()
+        pipe_edges = 0
+        for j, (inp, _, blocks) in enumerate(pipe.iter_batches([batch_of(first + i) for i in range(n_sampling)], prefetch=args.prefetch)):
+            pipe_edges += sum(b.num_edges() for b in blocks)
+            if j < 2 and cpu_batches > 0 and not pipe.graph_slots:  # (also held against the oracle below)
+                parity_keep.append(((first + j) % n_batches, ((first + j) * 64) & 0xFFFFFFFF, inp, blocks))
+        torch.cuda.synchronize()
+        t_sampling = time.perf_counter() - t0
+        first = pipe.batches
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _, _, blocks in pipe.iter_batches([batch_of(first + i) for i in range(K)], prefetch=args.prefetch):
             aggregate_only(blocks)
         torch.cuda.synchronize()
-        ms_overlapped = (time.perf_counter() - t_ov) / args.steps * 1e3
-        log("overlapped: %.3f ms per step" % ms_overlapped)
+        t_steps = time.perf_counter() - t0
+        pipelined = {"prefetch": args.prefetch, "value": pipe_edges / t_sampling, "sampling_batches": n_sampling,
+                     "ms_per_batch_sampling": t_sampling / n_sampling * 1e3, "ms_per_step": t_steps / K * 1e3}
+        log("prefetching sampler, %d mini-batches in flight: sampling alone %.3g sampled edges/s (%.3f ms per mini-batch over %d), "
+            "whole steps %.3f ms per step" % (args.prefetch, pipelined["value"], pipelined["ms_per_batch_sampling"], n_sampling,
+                                              pipelined["ms_per_step"]))
+        del pipe
 
     # ---- duration of the dominant kernel -------------------------------------------------
     # The stage interval above starts right after the sampler's host read-back, when the queue
@@ -1120,13 +1149,23 @@ def run_graph_workload(args, workload, light=False):
 
     out = {
         "metric": "sampled edges/s (sample+id_map) + aggregation HBM GB/s (% peak), 1 MI355X",
-        "value": edges_per_s,
+        "value": pipelined["value"] if pipelined else edges_per_s,
         "unit": "sampled edges/s",
         "n_gpus": 1,
         "steps": K,
         "warmup": args.warmup,
-        "ms_per_step": wall / K * 1e3,
-        "ms_per_step_overlapped": ms_overlapped,
+        "ms_per_step": pipelined["ms_per_step"] if pipelined else wall / K * 1e3,
+        "value_is": ("throughput of the sampling stage (all hops, id-map, transposed inner blocks, one host read-back per "
+                     "mini-batch) run as FusedMapSampler.iter_batches runs it in training: %d mini-batches in flight, each on a "
+                     "stream of its own; %d mini-batches, wall clock between two device synchronisations, nothing else on the "
+                     "GPU.  value_one_at_a_time is the same stage with one mini-batch in flight (HIP events around the stage "
+                     "inside sequential steps); ms_per_step is K whole steps with the prefetching sampler, "
+                     "ms_per_step_one_at_a_time the sequential steps that stages_ms is taken from"
+                     % (pipelined["prefetch"], pipelined["sampling_batches"])) if pipelined else
+                    "the sampling stage with one mini-batch in flight (HIP events around the stage inside sequential steps)",
+        "value_one_at_a_time": edges_per_s,
+        "ms_per_step_one_at_a_time": wall / K * 1e3,
+        "pipelined": pipelined,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -1138,11 +1177,13 @@ def run_graph_workload(args, workload, light=False):
                            "(the first hop expands 8192 seeds to ~10 K edges): a mini-batch samples ~1.6 M edges, not the "
                            "8.6 M that the fanouts would allow",
                    "sampler": sampler_mode, "id_order": "first-occurrence (deterministic)" if args.id_order == "first" else "arrival (run-dependent)",
-                   "step": "sample+id-map all hops; mean aggregation fwd on every block (outermost gathers from the full "
-                           "feature table); block transpose + bwd gather on the inner blocks; no dense layers",
+                   "step": "sample+id-map all hops (the transposed inner blocks come out of the same call); mean aggregation fwd on "
+                           "every block (outermost gathers from the full feature table); bwd gather over the transposed inner "
+                           "blocks; no dense layers",
                    "readback": ("the batch's sizes are stored into pinned host memory by the sampling kernels; the host waits for them while the outermost aggregation runs "
                                 "(sample_idmap = the sampling kernels' own time)") if args.readback == "hidden" else
                                "the batch's sizes are read back before anything else is enqueued (inside sample_idmap)"},
+        "stages_ms_are": "per stage of the sequential steps (one mini-batch at a time), HIP events on the launch stream",
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
                       "transpose_agg_bwd_inner": t_bwd / K},
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,
@@ -1153,7 +1194,8 @@ def run_graph_workload(args, workload, light=False):
         "value_drop_in_api": value_drop_in,
         "value_other_id_order": {"id_order": other_order, "value": value_other},
         "value_blocks_only": blocks_only,
-        "speedup_vs_cpu": None if cpu is None else edges_per_s / cpu["value"],
+        "speedup_vs_cpu": None if cpu is None else (pipelined["value"] if pipelined else edges_per_s) / cpu["value"],
+        "speedup_vs_cpu_one_at_a_time": None if cpu is None else edges_per_s / cpu["value"],
         "roofline": {"bound": "hbm", "achieved": agg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": agg_gbps / HBM_PEAK_GBPS,
                      "traffic": traffic_from_profile(workload, bytes_agg0 / K),

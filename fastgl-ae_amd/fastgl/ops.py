@@ -527,7 +527,8 @@ class BlocksPlan:
 
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
-                        keep_global=(0,), table_slots=None, id_order="first", stream_offset=None, readback=None):
+                        keep_global=(0,), table_slots=None, id_order="first", stream_offset=None, readback=None,
+                        launch_stream=None):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
@@ -547,7 +548,9 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     callers that capture this call in a graph and advance the random stream between replays).
     ``readback``: a pinned int32 host tensor of ``3*n_hops + 2`` elements; the kernels store a copy of
     ``counts`` there when the last of them is final, so the caller's read-back is a wait for the stream and a
-    look at that tensor, with no copy to enqueue."""
+    look at that tensor, with no copy to enqueue.
+    ``launch_stream``: a ``torch.cuda.Stream`` to enqueue the kernels on instead of the current one (the outputs are
+    still allocated on the current stream, where their consumer runs; the caller orders the two streams)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
     _check_input(indices, "indices", _I32)
     _check_input(seeds, "seeds", _I32)
@@ -589,7 +592,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
                                       flags, L.ptr(plan.table), slots, L.ptr(uniq), plan.cap_uniq, arr(block_ptr),
                                       arr(src_local), arr(src_global), t_arr(0), t_arr(1), t_arr(2), L.ptr(counts),
                                       None if readback is None else readback.data_ptr(), L.ptr(plan.ws),
-                                      plan.ws.numel(), L.stream_handle()))
+                                      plan.ws.numel(), L.stream_handle() if launch_stream is None else launch_stream.cuda_stream))
         plan.empty_slots = slots
     return uniq, block_ptr, src_local, src_global, counts, transposed
 

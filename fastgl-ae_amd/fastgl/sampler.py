@@ -249,6 +249,7 @@ class FusedMapSampler:
         self.output_nodes = None
         self._states = {}       # shape of a mini-batch -> _ShapeState
         self._lanes = []         # streams of iter_batches, one per mini-batch in flight
+        self._lane_events = []   # per lane: recorded behind the lane's latest mini-batch
         self._host_counts = {}   # word count -> pinned words for the per-batch size read-back, handed out in turn (_HostCounts)
         self._host_turn = 0
 
@@ -301,7 +302,9 @@ class FusedMapSampler:
                 state.nodes_seen = list(first.nodes_seen)
         return state
 
-    def _launch_fused(self, seeds, stream_base, worst_case=False, state=None, lane=0):
+    def _launch_fused(self, seeds, stream_base, worst_case=False, state=None, lane=0, stream=None):
+        """stream: enqueue on this stream instead of the current one (eager path only); the outputs are allocated on
+        the current stream all the same."""
         hop_fanouts = list(reversed(self.fanouts))
         lib = ops.L.lib()
         n_seeds = int(seeds.numel())
@@ -312,7 +315,10 @@ class FusedMapSampler:
         if plan is None:
             n_hops = len(hop_fanouts)
             hops = {"inner": range(n_hops - 1), "all": range(n_hops), "none": ()}[self.transposed]
-            plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps, transpose_hops=hops)
+            # (table and scratch belong to the stream that the kernels run on: when a plan is dropped, its memory
+            # must not reach allocations of another stream while that one may still be using it)
+            with torch.cuda.stream(stream if stream is not None else torch.cuda.current_stream(seeds.device)):
+                plan = ops.BlocksPlan(self.nodes_num, n_seeds, hop_fanouts, seeds.device, node_capacity=caps, transpose_hops=hops)
             state.plans = {k: v for k, v in state.plans.items() if k is None}  # keep the worst-case plan only
             state.plans[caps] = plan
         slots = plan.slots
@@ -322,9 +328,10 @@ class FusedMapSampler:
             out, host = self._replay(state, plan, slots, seeds, stream_base)
         else:
             host = self._take_host_counts(3 * len(hop_fanouts) + 2)
+            run_on = stream if stream is not None else torch.cuda.current_stream(seeds.device)
             out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
                                           keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
-                                          readback=host.expect(torch.cuda.current_stream(seeds.device)))
+                                          readback=host.expect(run_on), launch_stream=stream)
         return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state, host=host)
 
     def _take_host_counts(self, n_words):
@@ -482,35 +489,55 @@ class FusedMapSampler:
             self.batches += 1
             side = self._lane_stream(dev, lane)
             side.wait_stream(main)  # the seeds (and anything else the caller produced) are ready
-            with torch.cuda.stream(side):
-                pending = self._launch_fused(seeds, stream_base, lane=lane)
-            return pending, side
+            if self.graph_slots:  # (a graph replays on the current stream)
+                with torch.cuda.stream(side):
+                    pending = self._launch_fused(seeds, stream_base, lane=lane)
+                pending["on_lane"] = True
+            else:
+                # kernels on the lane's stream, outputs allocated on the caller's (where they are consumed and,
+                # in stream order behind that, freed)
+                pending = self._launch_fused(seeds, stream_base, lane=lane, stream=side)
+            done = self._lane_events[lane]
+            done.record(side)
+            return pending, side, done
 
         def finish(item):
-            pending, side = item
-            with torch.cuda.stream(side):  # a batch that outgrew its buffers is redone here, synchronously
-                result = self._finish_fused(pending, pending["host"].read())
-                done = torch.cuda.Event()
-                done.record(side)
-            main.wait_event(done)
+            pending, side, done = item
+            counts = pending["host"].read()
+            main.wait_event(done)  # whatever the caller enqueues from here on runs behind the mini-batch's kernels
+            if not pending.get("on_lane"):
+                return self._finish_fused(pending, counts)  # (a batch that outgrew its buffers is redone here, on the caller's stream)
+            with torch.cuda.stream(side):
+                result = self._finish_fused(pending, counts)
+                redone = torch.cuda.Event()
+                redone.record(side)
+            main.wait_event(redone)
             for t in (result[0],) + tuple(x for b in result[2]
                                           for x in (b.edge_ptr, b.src_local, b.src_global) + tuple(b._transposed or ())
                                           if x is not None):
-                t.record_stream(main)  # allocated on the lane's stream, consumed on the caller's
+                t.record_stream(main)  # (possibly allocated on the lane's stream; consumed on the caller's)
             return result
 
+        while len(self._lane_events) < prefetch:
+            self._lane_events.append(torch.cuda.Event())
         it = iter(seed_batches)
         in_flight = collections.deque()
         n_launched = 0
-        for seeds in itertools.islice(it, prefetch):
-            in_flight.append(launch(seeds, n_launched % prefetch))
-            n_launched += 1
-        while in_flight:
-            result = finish(in_flight.popleft())
-            for seeds in itertools.islice(it, 1):  # (its lane is the one that has just become free)
+        try:
+            for seeds in itertools.islice(it, prefetch):
                 in_flight.append(launch(seeds, n_launched % prefetch))
                 n_launched += 1
-            yield result
+            while in_flight:
+                result = finish(in_flight.popleft())
+                for seeds in itertools.islice(it, 1):  # (its lane is the one that has just become free)
+                    in_flight.append(launch(seeds, n_launched % prefetch))
+                    n_launched += 1
+                yield result
+        finally:
+            # a consumer that stops early: the mini-batches still in flight write into memory that is about to be
+            # freed on the caller's stream, so that stream waits for them first
+            for _, _, done in in_flight:
+                main.wait_event(done)
 
     def _sample_layerwise(self, seeds, stream_base):
         # the reference loop (FusedMapSampler.py:72-107), one drop-in call per step
