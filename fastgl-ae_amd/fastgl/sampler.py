@@ -228,8 +228,9 @@ class FusedMapSampler:
         # pays off where the GPU would otherwise wait for the host -- one mini-batch at a time from an idle GPU:
         # -11 % at batch 8192, -26 % at batch 1024 -- and not in a loop that keeps the GPU busy, where the launches
         # are hidden behind the previous step's kernels anyway.  The price: outputs live in R fixed slots used in
-        # turn, so the tensors of a mini-batch are overwritten when the R-th mini-batch after it is sampled --
-        # consume (or clone) them before that.
+        # turn, so the tensors of a mini-batch are overwritten when the R-th mini-batch after it is sampled (with
+        # iter_batches: the R-th after it on the same lane, i.e. R * prefetch mini-batches later) -- consume (or
+        # clone) them before that.
         # transposed: which blocks come with their transposed form (what the backward pass of a layer gathers over),
         # built inside the fused sampling call at next to no cost: "inner" = every block but the outermost (the first
         # layer's input needs no gradient), "all", or "none" (built on demand, Block.transposed()).  A deterministic
