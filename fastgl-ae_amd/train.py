@@ -78,10 +78,10 @@ def run(args):
         sync()
         tic = time.time()
         seed_batches = (order[i * args.batch_size:(i + 1) * args.batch_size] for i in range(steps))
-        stream = sampler.iter_batches(seed_batches) if args.prefetch else None
+        stream = sampler.iter_batches(seed_batches, prefetch=args.prefetch) if args.prefetch else None
         for step in range(steps):
             t0 = time.time()
-            if args.prefetch:  # batch step+1 is being sampled on a second stream while this one trains
+            if args.prefetch:  # the next mini-batches are being sampled on streams of their own while this one trains
                 input_nodes, output_nodes, blocks = next(stream)
             else:
                 seeds = order[step * args.batch_size:(step + 1) * args.batch_size]
@@ -167,7 +167,9 @@ def parse_args(argv=None):
     ap.add_argument("--deterministic", type=int, default=0,
                     help="1: order the transposed blocks' lists too, so that the fp32 sums of the backward pass -- and with them "
                          "the whole run -- are reproducible bit for bit (one radix sort per block; needs --id_order first)")
-    ap.add_argument("--prefetch", type=int, default=1, help="1: sample the next mini-batch on a second stream (default)")
+    ap.add_argument("--prefetch", type=int, default=2,
+                    help="mini-batches sampled ahead of the one that trains, each on a stream of its own (the reference's "
+                         "prefetch_factor, train_fastgl.py:109-122); 0: sample and train in turn")
     ap.add_argument("--log_every", type=int, default=10)
     ap.add_argument("--log_path", default="")
     return ap.parse_args(argv)
