@@ -202,6 +202,16 @@ def _check_batch_against_oracle(cuda, oracle, ptr, src, h_ptr, h_src, feat, fano
         assert plan.empty_slots is not None and plan.empty_slots < worst.slots  # a small table, left empty by the batch
         same_as_oracle(got, want, s_i)
         print("steady-state batch %d ok (%d edges)" % (i, sum(b.num_edges() for b in got[2])), flush=True)
+    # ... and as the prefetching iterator runs them: two mini-batches in flight, each on a stream of its own with its
+    # own table and scratch, the main stream busy with a consumer meanwhile
+    first = sampler.batches
+    seed_sets = [pool[(first + j) * 8192:(first + j + 1) * 8192].int() for j in range(4)]
+    for j, got in enumerate(sampler.iter_batches(iter(seed_sets), prefetch=2)):
+        want = oracle.sample_blocks(h_ptr, h_src, seed_sets[j].cpu().numpy(), fanouts, rng_seed, 64 * (first + j))
+        same_as_oracle(got, want, seed_sets[j])
+        fastgl.aggregate(got[2][0].edge_ptr, got[2][0].src_global, feat, mode="mean", zero_policy="zeros")
+    print("prefetching iterator ok", flush=True)
+    del got
     if graph_replay:
         gs = fastgl.FusedMapSampler(fanouts, rng_seed=rng_seed, graph_slots=2).set_graph(ptr, src)
         for i in range(4):  # batch 0 eager (worst-case plan); 1 and 2 capture the two slots; 3 replays slot 0
