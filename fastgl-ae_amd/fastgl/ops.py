@@ -37,6 +37,26 @@ def _check_input(t, name, dtypes=None):
         raise RuntimeError("%s must have dtype in %s, got %s" % (name, [str(d) for d in dtypes], t.dtype))
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev):
+    """Context that makes ``dev`` the current device -- nothing at all when it already is (the usual case: entering
+    and leaving ``torch.cuda.device`` costs several microseconds per call)."""
+    index = dev.index
+    if index is None or index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
+
+
 def _same_device(*tensors):
     dev = tensors[0].device
     for t in tensors[1:]:
@@ -95,7 +115,7 @@ def sample_node(src_edges, dst_edges, edge_ptr, seed_nodes, dst_nodes, neighbor_
     if dst_nodes < n_seeds:
         raise RuntimeError("dst_nodes (%d) is smaller than the number of seeds (%d)" % (dst_nodes, n_seeds))
     lib = L.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         src_out = torch.empty(max(dst_nodes * fanout, 1), dtype=torch.int32, device=dev)
         dst_out = torch.empty(max(dst_nodes * fanout, 1), dtype=torch.int32, device=dev)
         block_ptr = torch.empty(n_seeds + 1, dtype=torch.int32, device=dev)
@@ -142,7 +162,7 @@ def transfer_edge_id(src_edges, dst_edges, dst_edges_unique, dst_nodes, total_it
     max_new = max(0, min(int(unique_num), n_edges))
     capacity = n_dst + max_new
     slots = lib.fgl_idmap_slots(capacity)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         st = L.stream_handle()
         key = (torch.device(dev).index, st)
         table, known_empty = _table(slots, dev)
@@ -189,7 +209,7 @@ def cal_deg(edges, nodes_num):
     _check_input(edges, "edges", _I32)
     n = int(nodes_num)
     dev = edges.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         deg = torch.empty(max(n, 1), dtype=torch.int32, device=dev)[:n]
         L.check(L.lib().fgl_cal_deg(L.ptr(edges), int(edges.numel()), None, L.ptr(deg), n, L.stream_handle()))
     return deg
@@ -201,7 +221,7 @@ def exclusive_sum(in_degs):
     n = int(in_degs.numel())
     dev = in_degs.device
     lib = L.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         out = torch.empty(n + 1, dtype=torch.int32, device=dev)
         ws = L.workspace(lib.fgl_exclusive_sum_workspace_bytes(n), dev)
         L.check(lib.fgl_exclusive_sum_i32(L.ptr(in_degs), n, None, L.ptr(out), L.ptr(ws), ws.numel(), L.stream_handle()))
@@ -379,7 +399,7 @@ def aggregate(indptr, indices, feat, mode="sum", zero_policy="self", row_norm=No
     if z == L.ZERO_COPY_SELF and n > feat.size(0):
         raise RuntimeError("zero_policy 'self' needs feat to have a row for every output row")
     D = int(feat.size(1))
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         if out is None:
             out = torch.empty((n, D), dtype=feat.dtype, device=dev)
         elif out.shape != (n, D) or out.dtype != feat.dtype or out.stride(1) != 1 or not out.is_cuda:
@@ -412,7 +432,7 @@ def edge_softmax(indptr, indices, el, er, negative_slope=0.2, n_rows=None):
     if n < 0 or n > indptr.numel() - 1 or n > er.size(0):
         raise RuntimeError("n_rows (%d) does not match indptr (%d entries) / er (%d rows)" % (n, indptr.numel(), er.size(0)))
     H = int(el.size(1))
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         alpha = torch.empty((int(indices.numel()), H), dtype=torch.float32, device=dev)
         if n > 0 and indices.numel() > 0:
             L.check(L.lib().fgl_edge_softmax(L.ptr(indptr), L.ptr(indices), n, None, L.ptr(el), L.ptr(er), H,
@@ -431,7 +451,7 @@ def block_transpose(indptr, indices, n_rows, n_cols, edge_ids=False, sorted_rows
     n_rows, n_cols = int(n_rows), int(n_cols)
     nnz = int(indices.numel())
     lib = L.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         t_ptr = torch.empty(n_cols + 1, dtype=torch.int32, device=dev)
         t_idx = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz]
         t_edge = torch.empty(max(nnz, 1), dtype=torch.int32, device=dev)[:nnz] if edge_ids else None
@@ -464,7 +484,7 @@ def block_transpose_batch(blocks, edge_ids=False):
         group = small[g:g + L.TRANSPOSE_BATCH_MAX]
         n = len(group)
         dev = _same_device(*[blocks[i][0] for i in group], *[blocks[i][1] for i in group])
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             res = []
             for i in group:
                 indptr, indices, n_rows, n_cols = blocks[i]
@@ -566,7 +586,7 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     keep = {(h + H) % H for h in keep_global}
     slots = plan.slots if table_slots is None else min(int(table_slots), plan.slots)
     lib = L.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         uniq = torch.empty(max(plan.cap_uniq, 1), dtype=torch.int32, device=dev)
         block_ptr = [torch.empty(plan.cap_dst[h] + 1, dtype=torch.int32, device=dev) for h in range(H)]
         src_local = [torch.empty(max(plan.cap_edges[h], 1), dtype=torch.int32, device=dev) for h in range(H)]
