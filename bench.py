@@ -1137,8 +1137,9 @@ def run_graph_workload(args, workload, light=False):
                 first_difference = "seed batch %d, stream %d: %s" % (bi, sb, first_difference)
                 break
         parity = {"batches": len(parity_keep), "ok": first_difference is None,
-                  "what": "the first timed steps' outputs (the steady-state path: learned buffer sizes, small table, no fill, "
-                          "begin_sample/finish) vs the CPU oracle on the same seeds and Philox streams: unique list, block offsets, "
+                  "what": "the first timed sequential steps' outputs (the steady-state path: learned buffer sizes, small table, no "
+                          "fill, begin_sample/finish) and the first two mini-batches of the timed prefetching run (two in flight on "
+                          "two streams) vs the CPU oracle on the same seeds and Philox streams: unique list, block offsets, "
                           "local ids, outermost graph ids, transposed inner blocks; bit-exact"
                           + ("" if args.id_order == "first" else " after sorting the new ids (arrival order)")}
         if first_difference is not None:
