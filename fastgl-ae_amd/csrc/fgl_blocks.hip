@@ -27,12 +27,14 @@ __global__ __launch_bounds__(TS) void blocks_prepare_kernel(TableRef t, const vo
                                                             int64_t n_seeds, int fanout, int32_t* __restrict__ uniq,
                                                             int64_t* __restrict__ row_start, int32_t* __restrict__ deg_out,
                                                             int32_t* __restrict__ tile_sums, int32_t* __restrict__ later_sums,
-                                                            int64_t n_later_sums, int32_t* __restrict__ counts, int n_counts)
+                                                            int64_t n_later_sums, int32_t* __restrict__ counts, int n_counts,
+                                                            int32_t* __restrict__ sort_n_long)
 {
     __shared__ int smem[TS / kWave + 1];
     const int64_t first = (int64_t)blockIdx.x * TS + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * TS;
     for (int64_t i = first; i < n_counts; i += stride) counts[i] = (i == 0) ? (int32_t)n_seeds : 0;
+    if (first < 4) sort_n_long[first] = 0;  // (the counters of the row sort that may close the call)
     for (int64_t i = first; i < n_later_sums; i += stride) later_sums[i] = 0;
     const int64_t n_tiles = (n_seeds + TS - 1) / TS;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -90,6 +92,7 @@ struct BlocksPlan {
     uint32_t transpose_hops;
     int64_t cap_src[32];  // max source nodes (= columns) of hop h
     int split[32];        // counters per column while hop h's transposed rows are being counted
+    int64_t sort_long_max;  // rows of more than 64 entries that the transposed blocks can hold between them
 };
 
 struct BlocksScratch {
@@ -103,6 +106,8 @@ struct BlocksScratch {
     int32_t* t_rank[32];
     int32_t* t_tile_sums[32];
     int32_t* t_split_cnt[32];  // split counters (hops that count with several counters per column)
+    int32_t* sort_long_rows;   // rows left to the second launch of the row sort: pairs (job, row)
+    int32_t* sort_n_long;      // their number, one counter per group of eight transposed blocks (zeroed by the first launch of a call)
 };
 
 static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
@@ -114,8 +119,12 @@ static size_t carve_scratch(const BlocksPlan& p, void* ws, BlocksScratch* out)
     int32_t* tile_prefix = c.take<int32_t>((size_t)p.max_tiles);
     uint8_t* lowered = c.take<uint8_t>((size_t)p.max_edges);
     char* idmap_ws = c.take<char>(p.idmap_bytes);
+    int32_t* sort_long_rows = c.take<int32_t>((size_t)(2 * p.sort_long_max));
+    int32_t* sort_n_long = c.take<int32_t>(4);
     if (out) {
         memset(out, 0, sizeof(*out));
+        out->sort_long_rows = sort_long_rows;
+        out->sort_n_long = sort_n_long;
         out->row_start = row_start;
         out->deg = deg;
         out->tile_sums = tile_sums;
@@ -193,6 +202,9 @@ static int make_plan(int64_t n_nodes, int64_t n_seeds, const int32_t* fanouts, i
         if (h < n_hops && ((transpose_hops >> h) & 1u))
             FGL_REQUIRE(p->cap_src[h] * p->split[h] + 1 <= 0x7FFFFFFF, "sample_blocks: hop %d has too many columns to transpose", h);
     }
+    p->sort_long_max = 0;
+    for (int h = 0; h < n_hops; ++h)
+        if ((transpose_hops >> h) & 1u) p->sort_long_max += p->cap_edges[h] / (kWave + 1) + 1;
     p->table_slots = fgl_idmap_slots(cur);
     FGL_REQUIRE(p->table_slots <= ((int64_t)1 << 31), "sample_blocks: table too large");
     p->n_positions = p->cap_dst[n_hops - 1] > 0 ? p->cap_dst[n_hops - 1] : 1;
@@ -216,6 +228,21 @@ __global__ __launch_bounds__(kBlock) void transpose_step_kernel(const TransposeJ
         if (readback != nullptr && blockIdx.x == 0 && (int)threadIdx.x < n_counts) readback[threadIdx.x] = counts[threadIdx.x];
         tjob_fill<kBlock>(j);
     }
+}
+
+// Every row of the call's transposed blocks into ascending order of its entries' positions in the block (one launch
+// for all of them: blockIdx.y names the block).
+__global__ __launch_bounds__(kBlock) void transpose_sort_rows_kernel(const SortJobs jobs)
+{
+    tjob_sort_rows<kBlock>(jobs, (int)blockIdx.y);
+}
+
+// ... and the rows of more than 64 entries that it listed, a workgroup per row
+__global__ __launch_bounds__(kBlock) void transpose_sort_long_rows_kernel(const SortJobs jobs)
+{
+    __shared__ int s_key[kSortLds];
+    __shared__ int s_val[kSortLds];
+    tjob_sort_long_rows<kBlock>(jobs, s_key, s_val);
 }
 
 // ---- R-MAT -------------------------------------------------------------------------
@@ -293,7 +320,8 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
     const int order = idmap_flags & FGL_IDMAP_ARRIVAL;
     const bool table_is_empty = (idmap_flags & FGL_BLOCKS_TABLE_EMPTY) != 0;
     const bool leave_empty = (idmap_flags & FGL_BLOCKS_LEAVE_TABLE_EMPTY) != 0;
-    FGL_REQUIRE((idmap_flags & ~(FGL_IDMAP_ARRIVAL | FGL_BLOCKS_TABLE_EMPTY | FGL_BLOCKS_LEAVE_TABLE_EMPTY)) == 0,
+    const bool sort_rows = (idmap_flags & FGL_BLOCKS_SORT_TRANSPOSED) != 0;
+    FGL_REQUIRE((idmap_flags & ~(FGL_IDMAP_ARRIVAL | FGL_BLOCKS_TABLE_EMPTY | FGL_BLOCKS_LEAVE_TABLE_EMPTY | FGL_BLOCKS_SORT_TRANSPOSED)) == 0,
                 "sample_blocks: unknown flags %d", idmap_flags);
     FGL_REQUIRE(d_indptr && d_indices && d_table && d_uniq && block_ptr && src_local && d_counts, "sample_blocks: null pointer");
     FGL_REQUIRE(n_seeds == 0 || d_seeds != nullptr, "sample_blocks: null seeds");
@@ -358,11 +386,11 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         if (ts0 == 256)
             hipLaunchKernelGGL(blocks_prepare_kernel<256>, dim3((unsigned)blocks), dim3(256), 0, s, t, d_indptr, indptr_is64, n_nodes,
                                d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
-                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts, ws.sort_n_long);
         else
             hipLaunchKernelGGL(blocks_prepare_kernel<64>, dim3((unsigned)blocks), dim3(64), 0, s, t, d_indptr, indptr_is64, n_nodes,
                                d_seeds, n_seeds, fanouts[0], d_uniq, ws.row_start, ws.deg, ws.tile_sums,
-                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts);
+                               ws.tile_sums + p.tile_first[1], n_later, d_counts, n_counts, ws.sort_n_long);
         FGL_CHECK_LAUNCH("blocks_prepare_kernel");
     }
 
@@ -421,6 +449,33 @@ FGL_EXPORT int fgl_sample_blocks(const void* d_indptr, int indptr_is64, const in
         hipLaunchKernelGGL(transpose_step_kernel<2>, dim3((unsigned)job_before.side_blocks), dim3(kBlock), 0, s, job_before,
                            d_readback, d_counts, n_counts);
         FGL_CHECK_LAUNCH("transpose_step_kernel");
+    }
+    if (sort_rows && transpose_hops != 0) {
+        // rows of the transposed blocks in a fixed order: two more launches per eight blocks -- every row of up to
+        // 64 entries, then the longer ones that the first launch has listed
+        SortJobs jobs;
+        memset(&jobs, 0, sizeof(jobs));
+        jobs.long_rows = ws.sort_long_rows;
+        jobs.long_max = p.sort_long_max;
+        int n_jobs = 0, round = 0;
+        int64_t most_cols = 1;
+        for (int h = 0; h <= n_hops; ++h) {
+            if (h < n_hops && ((transpose_hops >> h) & 1u)) {
+                jobs.job[n_jobs++] = make_job(h);
+                if (p.cap_src[h] > most_cols) most_cols = p.cap_src[h];
+            }
+            if (n_jobs == 8 || (h == n_hops && n_jobs > 0)) {
+                jobs.n_long = ws.sort_n_long + round++;
+                const int64_t gx = ceil_div(most_cols, kBlock) < 4096 ? ceil_div(most_cols, kBlock) : 4096;
+                hipLaunchKernelGGL(transpose_sort_rows_kernel, dim3((unsigned)gx, (unsigned)n_jobs), dim3(kBlock), 0, s, jobs);
+                const int64_t gl = p.sort_long_max < 2048 ? p.sort_long_max : 2048;
+                hipLaunchKernelGGL(transpose_sort_long_rows_kernel, dim3((unsigned)(gl > 0 ? gl : 1)), dim3(kBlock), 0, s, jobs);
+                FGL_CHECK_LAUNCH("transpose_sort_rows_kernel");
+                n_jobs = 0;
+                most_cols = 1;
+                memset(jobs.job, 0, sizeof(jobs.job));
+            }
+        }
     }
     return FGL_OK;
 }

@@ -169,6 +169,239 @@ __device__ __forceinline__ void tjob_fill(const TransposeJob& j)
     }
 }
 
+// ---- rows in a fixed order ------------------------------------------------------------------------------------
+// The fill step leaves the entries of a transposed row in the order in which their atomics landed.  Sorting every
+// row by the position of its entries in the block (t_edge; ascending positions = ascending destination rows,
+// the order a stable counting sort gives) makes the transposed block, and with it the fp32 sums of every gather
+// over it, the same from run to run.  Rows are short with few exceptions, so the work is dealt by length:
+//   up to 8 entries     the row's lane sorts it in registers;
+//   up to 64            the row's wave, one entry per lane, by shuffles;
+//   longer rows         are listed by that pass and dealt out, one workgroup per row, by a second launch (hubs sit
+//                       next to each other in the numbering: left to the workgroup that finds them they would queue
+//                       up behind each other): up to kSortLds entries in LDS, beyond that kSortLds / 2 entries at a
+//                       time and then odd-even rounds of merging neighbouring pieces (as many rounds as pieces: a
+//                       hub of a whole graph taken as one block).
+// Keys are distinct (positions), or -- without t_edge -- destination rows, whose ties are interchangeable.
+constexpr int kSortLds = 4096;
+constexpr int kSortMax = 0x7FFFFFFF;
+
+struct SortJobs {
+    TransposeJob job[8];
+    int32_t* long_rows;   // pairs (job, row) of the rows left to the second launch
+    int32_t* n_long;      // how many (zero when the first launch starts; may exceed long_max: then rows were dropped
+    int64_t long_max;     //   from the list -- which its size, one per 65 entries, rules out)
+};
+
+__device__ __forceinline__ void sort_exchange(int& ka, int& va, int& kb, int& vb)
+{
+    if (kb < ka) {
+        const int k = ka, v = va;
+        ka = kb;
+        va = vb;
+        kb = k;
+        vb = v;
+    }
+}
+
+// bitonic sort of n (a power of two, <= kSortLds) pairs in LDS by the whole workgroup; `merge_only`: the two
+// halves are sorted already (ascending), only the last merge is needed
+template <int NT>
+__device__ __forceinline__ void sort_lds(int* s_key, int* s_val, int n, bool merge_only)
+{
+    if (merge_only) {  // (a bitonic merge wants the second half descending)
+        for (int i = threadIdx.x; i < n / 4; i += NT) {
+            const int a = n / 2 + i, b = n - 1 - i;
+            const int k = s_key[a], v = s_val[a];
+            s_key[a] = s_key[b];
+            s_val[a] = s_val[b];
+            s_key[b] = k;
+            s_val[b] = v;
+        }
+        __syncthreads();
+    }
+    for (int k = merge_only ? n : 2; k <= n; k <<= 1) {
+        for (int jj = k >> 1; jj > 0; jj >>= 1) {
+            for (int t = threadIdx.x; t < n / 2; t += NT) {
+                const int i = 2 * t - (t & (jj - 1));  // the lower index of the t-th pair at distance jj
+                const int o = i + jj;
+                const bool up = (i & k) == 0 || k == n;  // (the last merge is ascending throughout)
+                int ka = s_key[i], va = s_val[i], kb = s_key[o], vb = s_val[o];
+                if (up ? kb < ka : ka < kb) {
+                    s_key[i] = kb;
+                    s_val[i] = vb;
+                    s_key[o] = ka;
+                    s_val[o] = va;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void sort_load(int* s_key, int* s_val, int at, const int32_t* key, const int32_t* val, int64_t a,
+                                          int64_t first, int64_t len, int n)
+{
+    for (int i = threadIdx.x; i < n; i += NT) {
+        const int64_t e = first + i;
+        s_key[at + i] = e < len ? key[a + e] : kSortMax;
+        s_val[at + i] = (val != nullptr && e < len) ? val[a + e] : 0;
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void sort_store(const int* s_key, const int* s_val, int at, int32_t* key, int32_t* val, int64_t a,
+                                           int64_t first, int64_t len, int n)
+{
+    for (int i = threadIdx.x; i < n; i += NT) {
+        const int64_t e = first + i;
+        if (e < len) {
+            key[a + e] = s_key[at + i];
+            if (val != nullptr) val[a + e] = s_val[at + i];
+        }
+    }
+}
+
+// one row of more than 64 entries, by the whole workgroup
+template <int NT>
+__device__ __forceinline__ void sort_row_block(int* s_key, int* s_val, int32_t* key, int32_t* val, int64_t a, int64_t len)
+{
+    if (len <= kSortLds) {
+        int n = 128;
+        while (n < len) n <<= 1;
+        sort_load<NT>(s_key, s_val, 0, key, val, a, 0, len, n);
+        __syncthreads();
+        sort_lds<NT>(s_key, s_val, n, false);
+        sort_store<NT>(s_key, s_val, 0, key, val, a, 0, len, n);
+        __syncthreads();
+        return;
+    }
+    constexpr int kPiece = kSortLds / 2;
+    const int64_t pieces = (len + kPiece - 1) / kPiece;
+    for (int64_t p = 0; p < pieces; ++p) {
+        sort_load<NT>(s_key, s_val, 0, key, val, a, p * kPiece, len, kPiece);
+        __syncthreads();
+        sort_lds<NT>(s_key, s_val, kPiece, false);
+        sort_store<NT>(s_key, s_val, 0, key, val, a, p * kPiece, len, kPiece);
+        __syncthreads();
+    }
+    // odd-even rounds: neighbouring pieces are merged and split again, smaller half first; the padding of the last
+    // piece sorts to its end, which is never stored
+    for (int64_t round = 0; round < pieces; ++round) {
+        for (int64_t p = round & 1; p + 1 < pieces; p += 2) {
+            sort_load<NT>(s_key, s_val, 0, key, val, a, p * kPiece, len, kSortLds);
+            __syncthreads();
+            sort_lds<NT>(s_key, s_val, kSortLds, true);
+            sort_store<NT>(s_key, s_val, 0, key, val, a, p * kPiece, len, kSortLds);
+            __syncthreads();
+        }
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void tjob_sort_rows(const SortJobs& jobs, int job_index)
+{
+    const TransposeJob& j = jobs.job[job_index];
+    if (j.t_ptr == nullptr) return;
+    int32_t* key = j.t_edge ? j.t_edge : j.t_dst;
+    int32_t* val = j.t_edge ? j.t_dst : nullptr;
+    const int64_t n_cols = actual_count(j.cols_max, j.d_n_cols);
+    const int64_t n_edges = actual_count(j.edges_max, j.d_n_edges);
+    const int lane = lane_id();
+    // Neighbouring rows go to different waves (row r to wave r mod the number of waves): the long rows of a block
+    // sit next to each other -- hubs are met early and numbered early -- and a wave takes its rows of 9..64 entries
+    // one after the other.
+    const int64_t n_waves = (int64_t)gridDim.x * (NT / kWave);
+    const int64_t wave = (int64_t)blockIdx.x * (NT / kWave) + threadIdx.x / kWave;
+    for (int64_t first = 0; first < n_cols; first += n_waves * kWave) {  // (uniform over the launch)
+        const int64_t c = first + wave + n_waves * lane;
+        int64_t a = 0, b = 0;
+        if (c < n_cols) {
+            a = j.t_ptr[c];
+            b = j.t_ptr[c + 1];
+            if (b > n_edges) b = n_edges;
+            if (a > b) a = b;
+        }
+        const int64_t len = b - a;
+        if (len >= 2 && len <= 8) {  // in registers: a sorting network for eight
+            int k[8], v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                k[i] = i < len ? key[a + i] : kSortMax;
+                v[i] = (val != nullptr && i < len) ? val[a + i] : 0;
+            }
+#define FGL_CX(x, y) sort_exchange(k[x], v[x], k[y], v[y])
+            FGL_CX(0, 1); FGL_CX(2, 3); FGL_CX(4, 5); FGL_CX(6, 7);
+            FGL_CX(0, 2); FGL_CX(1, 3); FGL_CX(4, 6); FGL_CX(5, 7);
+            FGL_CX(1, 2); FGL_CX(5, 6); FGL_CX(0, 4); FGL_CX(3, 7);
+            FGL_CX(1, 5); FGL_CX(2, 6);
+            FGL_CX(1, 4); FGL_CX(3, 6);
+            FGL_CX(2, 4); FGL_CX(3, 5);
+            FGL_CX(3, 4);
+#undef FGL_CX
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i < len) {
+                    key[a + i] = k[i];
+                    if (val != nullptr) val[a + i] = v[i];
+                }
+        }
+        // rows of 9..64 entries: the wave takes them one after the other, an entry per lane
+        unsigned long long todo = __ballot(len > 8 && len <= kWave);
+        while (todo != 0) {
+            const int r = __ffsll((long long)todo) - 1;
+            todo &= todo - 1;
+            const int64_t ra = __shfl(a, r, kWave);
+            const int rl = (int)__shfl(len, r, kWave);
+            int kk = lane < rl ? key[ra + lane] : kSortMax;
+            int vv = (val != nullptr && lane < rl) ? val[ra + lane] : 0;
+#pragma unroll
+            for (int k2 = 2; k2 <= kWave; k2 <<= 1) {
+#pragma unroll
+                for (int jj = k2 >> 1; jj > 0; jj >>= 1) {
+                    const int ok = __shfl_xor(kk, jj, kWave);
+                    const int ov = __shfl_xor(vv, jj, kWave);
+                    const bool up = (lane & k2) == 0;
+                    const bool lower = (lane & jj) == 0;
+                    const bool take = (lower == up) ? (ok < kk) : (ok > kk);
+                    if (take) {
+                        kk = ok;
+                        vv = ov;
+                    }
+                }
+            }
+            if (lane < rl) {
+                key[ra + lane] = kk;
+                if (val != nullptr) val[ra + lane] = vv;
+            }
+        }
+        // longer rows: listed for the second launch
+        if (len > kWave) {
+            const int64_t at = atomicAdd(jobs.n_long, 1);
+            if (at < jobs.long_max) {
+                jobs.long_rows[2 * at] = job_index;
+                jobs.long_rows[2 * at + 1] = (int32_t)c;
+            }
+        }
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void tjob_sort_long_rows(const SortJobs& jobs, int* s_key, int* s_val)
+{
+    int64_t n = *jobs.n_long;
+    if (n > jobs.long_max) n = jobs.long_max;
+    for (int64_t q = blockIdx.x; q < n; q += gridDim.x) {
+        const TransposeJob& j = jobs.job[jobs.long_rows[2 * q] & 7];
+        const int64_t c = jobs.long_rows[2 * q + 1];
+        const int64_t n_edges = actual_count(j.edges_max, j.d_n_edges);
+        int64_t a = j.t_ptr[c], b = j.t_ptr[c + 1];
+        if (b > n_edges) b = n_edges;
+        if (a > b) a = b;
+        sort_row_block<NT>(s_key, s_val, j.t_edge ? j.t_edge : j.t_dst, j.t_edge ? j.t_dst : nullptr, a, b - a);
+    }
+}
+
 #endif  // __HIPCC__
 
 }  // namespace fgl

@@ -22,7 +22,7 @@ ZERO_COPY_SELF, ZERO_ZEROS = 0, 1
 ABI_VERSION = 11  # FGL_ABI_VERSION of include/fastgl_hip.h that the signatures below follow
 STATUS_TABLE_FULL, STATUS_UNIQ_OVERFLOW, STATUS_MISSING_KEY, STATUS_BAD_SEED, STATUS_BAD_ID = 1, 2, 4, 8, 16
 IDMAP_ORDERED, IDMAP_ARRIVAL, IDMAP_FINAL, IDMAP_LEAVE_TABLE_EMPTY = 0, 1, 2, 8
-BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY = 4, 8
+BLOCKS_TABLE_EMPTY, BLOCKS_LEAVE_TABLE_EMPTY, BLOCKS_SORT_TRANSPOSED = 4, 8, 16
 MAX_FANOUT = 192
 SHORT_ROW_ENTRIES = 32
 TRANSPOSE_BATCH_MAX, TRANSPOSE_BATCH_MAX_EDGES, TRANSPOSE_BATCH_MAX_COLS = 8, 1 << 20, 1 << 23

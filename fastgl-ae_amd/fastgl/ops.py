@@ -548,7 +548,7 @@ class BlocksPlan:
 
 def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: int, stream_base: int,
                         keep_global=(0,), table_slots=None, id_order="first", stream_offset=None, readback=None,
-                        launch_stream=None):
+                        launch_stream=None, sort_transposed=False):
     """All hops of one mini-batch in one enqueue (no host synchronisation inside).
 
     Returns device tensors sized by the plan's bounds: ``(uniq, block_ptr[h], src_local[h],
@@ -569,6 +569,8 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
     ``readback``: a pinned int32 host tensor of ``3*n_hops + 2`` elements; the kernels store a copy of
     ``counts`` there when the last of them is final, so the caller's read-back is a wait for the stream and a
     look at that tensor, with no copy to enqueue.
+    ``sort_transposed``: the rows of the transposed blocks come out in ascending order of their entries' positions in
+    the block (run-to-run identical arrays and, with them, fp32 sums of the backward gathers; one more launch).
     ``launch_stream``: a ``torch.cuda.Stream`` to enqueue the kernels on instead of the current one (the outputs are
     still allocated on the current stream, where their consumer runs; the caller orders the two streams)."""
     _check_input(edge_ptr, "edge_ptr", _PTR)
@@ -605,6 +607,8 @@ def sample_blocks_fused(plan: BlocksPlan, edge_ptr, indices, seeds, rng_seed: in
         flags = {"first": L.IDMAP_ORDERED, "arrival": L.IDMAP_ARRIVAL}[id_order] | L.BLOCKS_LEAVE_TABLE_EMPTY
         if plan.empty_slots == slots:
             flags |= L.BLOCKS_TABLE_EMPTY
+        if sort_transposed:
+            flags |= L.BLOCKS_SORT_TRANSPOSED
         plan.empty_slots = None
         L.check(lib.fgl_sample_blocks(L.ptr(edge_ptr), int(edge_ptr.dtype == torch.int64), L.ptr(indices),
                                       int(edge_ptr.numel()) - 1, L.ptr(seeds), plan.n_seeds, plan._fan, H, plan._node_cap,

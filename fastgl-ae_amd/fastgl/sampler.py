@@ -219,7 +219,8 @@ class FusedMapSampler:
             raise ValueError("id_order must be 'first' or 'arrival'")
         self.id_order = id_order  # numbering of new node ids (fused path): see ops.sample_blocks_fused
         # deterministic=True also fixes the order inside each block's transposed lists, so that the
-        # fp32 sums of the backward pass are reproducible bit for bit (costs one radix sort per block)
+        # fp32 sums of the backward pass are reproducible bit for bit (one more launch per mini-batch for the transposed
+        # blocks that the sampling call builds, a stable sort for those built on demand)
         self.deterministic = bool(deterministic)
         if self.deterministic and id_order != "first":
             raise ValueError("deterministic=True needs id_order='first'")
@@ -234,10 +235,11 @@ class FusedMapSampler:
         # transposed: which blocks come with their transposed form (what the backward pass of a layer gathers over),
         # built inside the fused sampling call at next to no cost: "inner" = every block but the outermost (the first
         # layer's input needs no gradient), "all", or "none" (built on demand, Block.transposed()).  A deterministic
-        # sampler orders its transposed lists and builds them on demand.
+        # sampler has the call sort their rows as well (one more launch); blocks whose transposed form is built on
+        # demand get theirs from a stable sort.
         if transposed not in ("inner", "all", "none"):
             raise ValueError("transposed must be 'inner', 'all' or 'none'")
-        self.transposed = "none" if self.deterministic else transposed
+        self.transposed = transposed
         self.graph_slots = int(graph_slots)
         if self.graph_slots < 0 or self.graph_slots == 1:
             raise ValueError("graph_slots must be 0 (off) or at least 2")
@@ -332,7 +334,7 @@ class FusedMapSampler:
             run_on = stream if stream is not None else torch.cuda.current_stream(seeds.device)
             out = ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, seeds, self.rng_seed, stream_base,
                                           keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
-                                          readback=host.expect(run_on), launch_stream=stream)
+                                          readback=host.expect(run_on), launch_stream=stream, sort_transposed=self.deterministic)
         return dict(seeds=seeds, stream_base=stream_base, caps=caps, out=out, state=state, host=host)
 
     def _take_host_counts(self, n_words):
@@ -388,7 +390,8 @@ class FusedMapSampler:
             # stream_base 0: the slot's offset carries the mini-batch's stream number
             return ops.sample_blocks_fused(plan, self.edge_ptr, self.edge_src, slot["seeds"], self.rng_seed, 0,
                                            keep_global=(len(hop_fanouts) - 1,), table_slots=slots, id_order=self.id_order,
-                                           stream_offset=slot["offset"], readback=slot["host"].words)
+                                           stream_offset=slot["offset"], readback=slot["host"].words,
+                                           sort_transposed=self.deterministic)
 
         cur = torch.cuda.current_stream(dev)
         warm = torch.cuda.Stream(device=dev)  # default priority

@@ -84,6 +84,10 @@ enum fgl_zero_policy {
                                           on the same slots): the call's fill launch is skipped */
 #define FGL_BLOCKS_LEAVE_TABLE_EMPTY 8 /* the last pass of the call also empties the table again (it no longer reads
                                           it), so that the next call may say FGL_BLOCKS_TABLE_EMPTY */
+#define FGL_BLOCKS_SORT_TRANSPOSED 16  /* the rows of the transposed blocks that the call builds come out sorted by the
+                                          position of their entries in the block (= by destination row), instead of in the
+                                          order in which the entries' atomics landed: the same arrays from run to run, and
+                                          with them the same fp32 sums in every gather over them; one more launch per call */
 #define FGL_MAX_FANOUT 192
 
 int fgl_abi_version(void);
@@ -261,7 +265,8 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * t_ptr / t_dst / t_edge are NULL, or arrays of n_hops pointers of which any may be NULL.  Where t_ptr[h] is given
  * (int32[cap_src[h]+1], cap_src[h] = cap_dst[h+1], or cap_uniq for the last hop) the call also builds hop h's
  * transposed block: t_ptr[h] = row pointer over the hop's source nodes, t_dst[h] int32[cap_edges[h]] (required
- * then) = the destination rows each source node feeds, unordered within a row, t_edge[h] (optional) = the
+ * then) = the destination rows each source node feeds (unordered within a row unless FGL_BLOCKS_SORT_TRANSPOSED is
+ * given), t_edge[h] (optional) = the
  * position in src_local[h] of every transposed entry.  Sizes are the call's own device-side counts, so nothing
  * waits for the host.  The work rides on launches the call makes anyway -- a hop's edges take their place in their
  * transposed rows as the id-map numbers them, and the next hop's launches turn the counts into offsets and

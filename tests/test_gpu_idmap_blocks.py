@@ -255,6 +255,51 @@ def test_waiting_for_the_words_and_dropped_batches(cuda, oracle, small_graph):
     assert len(sampler._host_counts[11]) <= 2
 
 
+def test_sorted_transposed_blocks_equal_the_stable_transpose(cuda, oracle):
+    """FGL_BLOCKS_SORT_TRANSPOSED (a deterministic sampler): every row of the transposed blocks that the call builds is in
+    ascending order of its entries' positions -- the arrays equal the oracle's stable counting sort entry for entry, run
+    after run.  A hand-built graph gives rows of every length class of the sort: 1, 2..8, 9..64, 65..4096 and beyond
+    (merged in pieces), and one node that nobody samples."""
+    import fastgl
+    print("sample_blocks sorted transposed rows", flush=True)
+    rng = np.random.default_rng(3)
+    n = 30_000
+    # node v < 24 000 has the single neighbour hub(v): hubs 0..5 are mentioned 9 000, 5 000, 3 000, 700, 40 and 6 times,
+    # the other nodes point at random targets (rows of one or two entries)
+    counts = [9000, 5000, 3000, 700, 40, 6]
+    target = np.concatenate([np.full(c, h) for h, c in enumerate(counts)] + [rng.integers(100, n, 24_000 - sum(counts))]).astype(np.int32)
+    rows = [[int(t)] for t in target] + [[] for _ in range(n - 24_000)]
+    indptr, indices = _csr_from_rows(rows)
+    ptr, idx = load_graph(cuda, indptr, indices)
+    seeds = rng.permutation(24_000)[:20_000].astype(np.int32)
+    for which in ("inner", "all"):
+        first = None
+        for run in range(2):
+            sampler = fastgl.FusedMapSampler([3, 2], rng_seed=4, deterministic=True, transposed=which).set_graph(ptr, idx)
+            inp, _, blocks = sampler.sample_blocks(None, dev_i32(seeds, cuda))
+            w_inp, w_blocks = oracle.sample_blocks(indptr, indices, seeds, [3, 2], 4, 0)
+            assert np.array_equal(inp.cpu().numpy(), w_inp)
+            got = []
+            for b, w in zip(blocks, w_blocks):
+                if b._transposed is None:
+                    continue
+                t_ptr, t_dst, t_edge = (t.cpu().numpy() for t in b.transposed(edge_ids=True))
+                w_ptr, w_idx = oracle.transpose(w["indptr"], w["src_local"], w["n_src"])
+                assert np.array_equal(t_ptr, w_ptr) and np.array_equal(t_dst, w_idx)
+                row_of = np.repeat(np.arange(w["n_src"]), np.diff(w_ptr))
+                order = np.lexsort((t_edge, row_of))
+                assert np.array_equal(order, np.arange(t_edge.size))  # positions ascend within every row
+                assert np.array_equal(w["src_local"][t_edge], row_of)
+                got.append((t_dst, t_edge))
+            assert len(got) == (1 if which == "inner" else 2)
+            longest = max(int(np.diff(oracle.transpose(w["indptr"], w["src_local"], w["n_src"])[0]).max()) for w in w_blocks[1:])
+            assert longest > 4096  # the piecewise merge ran
+            if first is None:
+                first = got
+            else:
+                assert all(np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) for a, b in zip(first, got))
+
+
 def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     import fastgl
     print("sample_blocks int32 ptr", flush=True)
