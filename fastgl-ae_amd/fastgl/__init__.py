@@ -29,7 +29,7 @@ from .ops import (  # noqa: F401
     table_size,
     transfer_edge_id,
 )
-from .sampler import Block, FusedMapSampler, PendingBatch, transpose_blocks  # noqa: F401
+from .sampler import Block, DataLoader, FusedMapSampler, PendingBatch, transpose_blocks  # noqa: F401
 from .conv import (  # noqa: F401
     GAT,
     GCN,

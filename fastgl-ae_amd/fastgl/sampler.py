@@ -571,3 +571,47 @@ class FusedMapSampler:
         finally:
             ops._rng_state.update(saved)
         return seed_nodes_acc, raw_seed_nodes, blocks
+
+
+class DataLoader:
+    """Mini-batch iterator with the constructor that the reference's trainer uses for DGL's ``DataLoader``
+    (train_fastgl.py:248-258: ``DataLoader(g, train_nids, sampler, use_ddp=..., batch_size=..., shuffle=True,
+    drop_last=False, prefetch_factor=..., num_workers=...)``) and the same iteration protocol
+    (``for step, (input_nodes, output_nodes, blocks) in enumerate(dataloader)``, train_fastgl.py:346), without DGL.
+    Every epoch it cuts the (optionally shuffled) seed ids into batches and hands them to
+    ``sampler.iter_batches(..., prefetch=prefetch_factor)``: ``prefetch_factor`` mini-batches are sampled ahead on the
+    GPU, each on a stream of its own, where DGL would run CPU workers.  ``g`` is ignored, as the reference's sampler
+    ignores it (train_fastgl.py:245-246); ``num_workers`` is accepted and unused (sampling runs on the GPU);
+    ``use_ddp`` must be false (one GPU)."""
+
+    def __init__(self, g, nids, sampler, use_ddp=False, batch_size=1, shuffle=False, drop_last=False, prefetch_factor=2,
+                 num_workers=0, seed=0, **unused):
+        if use_ddp:
+            raise NotImplementedError("one GPU: seed shards per rank are the trainer's business")
+        if int(batch_size) < 1:
+            raise ValueError("batch_size must be positive")
+        self.nids = nids
+        self.sampler = sampler
+        self.batch_size = int(batch_size)
+        self.shuffle = bool(shuffle)
+        self.drop_last = bool(drop_last)
+        self.prefetch_factor = max(0, int(prefetch_factor if prefetch_factor is not None else 0))
+        self.seed = int(seed)
+        self.epoch = 0
+
+    def __len__(self):
+        n = int(self.nids.numel())
+        return n // self.batch_size if self.drop_last else -(-n // self.batch_size)
+
+    def __iter__(self):
+        ids = self.nids
+        if self.shuffle:  # a fresh, seeded permutation per epoch
+            gen = torch.Generator(device=ids.device).manual_seed(self.seed + self.epoch)
+            ids = ids[torch.randperm(int(ids.numel()), generator=gen, device=ids.device)]
+        self.epoch += 1
+        B = self.batch_size
+        batches = (ids[i * B:(i + 1) * B] for i in range(len(self)))
+        if self.prefetch_factor > 0 and getattr(self.sampler, "fused", False):
+            return self.sampler.iter_batches(batches, prefetch=self.prefetch_factor)
+        return (self.sampler.sample_blocks(None, b) for b in batches)
+

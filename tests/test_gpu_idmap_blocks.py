@@ -300,6 +300,41 @@ def test_sorted_transposed_blocks_equal_the_stable_transpose(cuda, oracle):
                 assert all(np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) for a, b in zip(first, got))
 
 
+def test_dataloader_with_the_trainers_constructor(cuda, oracle, small_graph):
+    """fastgl.DataLoader, constructed and iterated as the reference's trainer does with DGL's (train_fastgl.py:248-258,346):
+    every seed once per epoch, a different order every epoch, a short last batch unless drop_last, each mini-batch equal
+    to the oracle's for its seeds and its place in the sampler's sequence of random streams."""
+    import fastgl
+    print("DataLoader", flush=True)
+    indptr, indices = small_graph
+    ptr, idx = load_graph(cuda, indptr, indices)
+    train = dev_i32(np.random.default_rng(8).permutation(indptr.size - 1)[:2500].astype(np.int32), cuda)
+    sampler = fastgl.FusedMapSampler([15, 10, 5], replace=False, rng_seed=6).set_graph(ptr, idx)
+    loader = fastgl.DataLoader(None, train, sampler, use_ddp=False, batch_size=600, shuffle=True, drop_last=False,
+                               prefetch_factor=2, num_workers=0)
+    assert len(loader) == 5
+    orders = []
+    n_batch = 0
+    for epoch in range(2):
+        seen = []
+        for step, (input_nodes, output_nodes, blocks) in enumerate(loader):
+            seeds = output_nodes.cpu().numpy()
+            assert seeds.size == (600 if step < 4 else 100)
+            check_blocks(oracle, indptr, indices, seeds, [15, 10, 5], (input_nodes, output_nodes, blocks), 6, 64 * n_batch)
+            seen.append(seeds)
+            n_batch += 1
+        assert step == 4
+        order = np.concatenate(seen)
+        assert np.array_equal(np.sort(order), np.sort(train.cpu().numpy()))
+        orders.append(order)
+    assert not np.array_equal(orders[0], orders[1])
+    assert len(fastgl.DataLoader(None, train, sampler, batch_size=600, drop_last=True)) == 4
+    plain = fastgl.DataLoader(None, train, sampler, batch_size=1000, prefetch_factor=0)
+    assert [int(o.numel()) for _, o, _ in plain] == [1000, 1000, 500]
+    with pytest.raises(NotImplementedError):
+        fastgl.DataLoader(None, train, sampler, use_ddp=True)
+
+
 def test_sample_blocks_int32_ptr_and_long_seeds(cuda, oracle, small_graph):
     import fastgl
     print("sample_blocks int32 ptr", flush=True)
