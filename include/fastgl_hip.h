@@ -220,10 +220,11 @@ int fgl_idmap_lookup(const void* d_table, int64_t slots, int32_t* d_ids, int64_t
  * the numbering persisting across hops (hop h's unique list is hop h+1's seed list).
  * Hops are indexed in sampling order: hop 0 expands the raw seeds with fanouts[0];
  * idmap_flags is FGL_IDMAP_ORDERED or FGL_IDMAP_ARRIVAL (the last hop adds FGL_IDMAP_FINAL by itself), optionally
- * or'ed with FGL_BLOCKS_TABLE_EMPTY and / or FGL_BLOCKS_LEAVE_TABLE_EMPTY.
+ * or'ed with FGL_BLOCKS_TABLE_EMPTY, FGL_BLOCKS_LEAVE_TABLE_EMPTY and / or FGL_BLOCKS_SORT_TRANSPOSED.
  * Launches for H hops, first-occurrence numbering: one that starts the batch (counts, seeds into the table, the
  * first hop's row offsets) and four per hop (sample, insert, mark, number) = 4H + 1, plus a table fill unless the
- * caller vouches for an empty table, plus one scan per hop beyond a million seeds or four million edges.  Each
+ * caller vouches for an empty table, plus one scan per hop beyond a million seeds or four million edges, plus three
+ * if the last hop's transposed block is wanted, plus two with FGL_BLOCKS_SORT_TRANSPOSED.  Each
  * hop's passes also prepare the next hop's sampling (row starts, degrees and per-tile edge counts of the nodes
  * they touch), so no hop after the first reads the graph's offsets in a pass of its own.
  * (The reference lists fanouts the other way round and iterates reversed(); the caller
