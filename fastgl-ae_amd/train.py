@@ -66,26 +66,23 @@ def run(args):
     optimizer = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
     sync = torch.cuda.synchronize
 
-    n_train = train_nids.numel()
-    steps = (n_train + args.batch_size - 1) // args.batch_size
+    # the reference wraps its sampler in DGL's DataLoader (train_fastgl.py:248-258); here the library's own, with the same
+    # arguments: a seeded shuffle per epoch, prefetch_factor mini-batches sampled ahead on streams of their own
+    dataloader = fastgl.DataLoader(None, train_nids, sampler, use_ddp=False, batch_size=args.batch_size, shuffle=True,
+                                   drop_last=False, prefetch_factor=args.prefetch, num_workers=0, seed=args.seed + 1000)
+    steps = len(dataloader)
     epochs = []
     losses = []
     for epoch in range(args.num_epoch + 1):  # the first epoch is the warm-up (train_fastgl.py:96-97)
-        gen = torch.Generator(device=device).manual_seed(args.seed + 1000 + epoch)
-        order = train_nids[torch.randperm(n_train, generator=gen, device=device)]
         t = dict(sample=0.0, copy=0.0, forward=0.0, backward=0.0)
         n_edges = n_inputs = 0
         sync()
         tic = time.time()
-        seed_batches = (order[i * args.batch_size:(i + 1) * args.batch_size] for i in range(steps))
-        stream = sampler.iter_batches(seed_batches, prefetch=args.prefetch) if args.prefetch else None
+        batches = iter(dataloader)
         for step in range(steps):
             t0 = time.time()
-            if args.prefetch:  # the next mini-batches are being sampled on streams of their own while this one trains
-                input_nodes, output_nodes, blocks = next(stream)
-            else:
-                seeds = order[step * args.batch_size:(step + 1) * args.batch_size]
-                input_nodes, output_nodes, blocks = sampler.sample_blocks(None, seeds)
+            input_nodes, output_nodes, blocks = next(batches)
+            if not args.prefetch:
                 sync()
             t1 = time.time()
             fastgl.transpose_blocks(blocks[1:])  # the backward pass of every layer but the first gathers over the transposed block
@@ -166,7 +163,7 @@ def parse_args(argv=None):
     ap.add_argument("--id_order", default="first", choices=["first", "arrival"])
     ap.add_argument("--deterministic", type=int, default=0,
                     help="1: order the transposed blocks' lists too, so that the fp32 sums of the backward pass -- and with them "
-                         "the whole run -- are reproducible bit for bit (one radix sort per block; needs --id_order first)")
+                         "the whole run -- are reproducible bit for bit (two more launches per mini-batch; needs --id_order first)")
     ap.add_argument("--prefetch", type=int, default=2,
                     help="mini-batches sampled ahead of the one that trains, each on a stream of its own (the reference's "
                          "prefetch_factor, train_fastgl.py:109-122); 0: sample and train in turn")
