@@ -594,6 +594,18 @@ def compare_with_oracle(O, np, g_inp, g_blocks, w_inp, w_blocks, exact_order=Tru
     return None
 
 
+def sampling_stage_bytes(blocks, ptr_bytes):
+    """Algorithmic bytes of sampling + id-map for one mini-batch: per hop with S seeds, E sampled edges and U new ids,
+    sampling reads a seed id and two row offsets per seed and one graph entry per edge and writes the edge's source and the
+    block's row offsets, the id-map reads the source, touches one 8-byte slot and writes the local id per edge, and per new
+    id fills a slot and writes the unique list."""
+    total = 0
+    for b in blocks:
+        S, E, U = b.num_dst_nodes(), b.num_edges(), b.num_src_nodes() - b.num_dst_nodes()
+        total += S * (4 + 2 * ptr_bytes) + (S + 1) * 4 + E * (4 + 4) + E * (4 + 8 + 4) + U * (8 + 4)
+    return total
+
+
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
@@ -786,6 +798,8 @@ def run_graph_workload(args, workload, light=False):
     parity_keep = []  # (seed batch, random stream, outputs) of the first timed steps, compared with the oracle in the CPU leg
     N_PARITY = 4
 
+    stage_bytes = []  # algorithmic bytes of the sampling stage, per recorded step (of every sampler that ran the steps)
+
     def step(i, rec=None, sampler=sampler):
         seeds = train[(i % n_batches) * B:(i % n_batches) * B + B]
         stream_base = (sampler.batches * 64) & 0xFFFFFFFF  # the Philox streams this mini-batch draws from
@@ -823,6 +837,7 @@ def run_graph_workload(args, workload, light=False):
         e4.record()
         if rec is not None:
             rec.append(((sum(b.num_edges() for b in blocks), b0.num_edges(), b0.num_dst_nodes()), (e0, e1, e2, e3, e4)))
+            stage_bytes.append(sampling_stage_bytes(blocks, 8 if edge_ptr.dtype == torch.int64 else 4))
             keep.append(b0.clone() if sampler.graph_slots else b0)  # (a graph-replay slot is overwritten two batches on)
             del keep[:-4]  # a few outermost blocks are kept for the kernel-time replay below
             if sampler is main_sampler and len(parity_keep) < N_PARITY and cpu_batches > 0:
@@ -1098,6 +1113,7 @@ def run_graph_workload(args, workload, light=False):
         bytes_agg0 += e_ * D * esz + nd * D * esz + 4 * e_ + 4 * (nd + 1)  # gathered rows + output + indices + offsets
     K = args.steps
     edges_per_s = tot_edges / (t_sample * 1e-3)
+    stage_bytes_per_batch = sum(stage_bytes[:len(rec)]) / max(1, len(rec))  # (the main sampler's steps come first)
     agg_gbps = replay_bytes / (t_kernel0 * 1e-3) / 1e9
     bytes_agg0 = replay_bytes
     log("last batch blocks:", last_blocks)
@@ -1200,6 +1216,15 @@ def run_graph_workload(args, workload, light=False):
         "stages_ms_are": "per stage of the sequential steps (one mini-batch at a time), HIP events on the launch stream",
         "stages_ms": {"sample_idmap": t_sample / K, "agg_fwd_outer": t_agg0 / K, "agg_fwd_inner": t_fwd_in / K,
                       "transpose_agg_bwd_inner": t_bwd / K},
+        "sampling": {"algorithmic_bytes_per_mini_batch": stage_bytes_per_batch,
+                     "algorithmic_bytes_per_edge": stage_bytes_per_batch / (tot_edges / K),
+                     "GBps_one_at_a_time": stage_bytes_per_batch / (t_sample / K * 1e-3) / 1e9,
+                     "GBps": (stage_bytes_per_batch / (pipelined["ms_per_batch_sampling"] * 1e-3) / 1e9) if pipelined else None,
+                     "frac_peak": (stage_bytes_per_batch / (pipelined["ms_per_batch_sampling"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+                                  if pipelined else stage_bytes_per_batch / (t_sample / K * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "bound": "not bytes: the rate of random accesses (one 4-byte graph read per edge, ~38 G/s here: random_read_Gps) "
+                              "and of atomics (one 64-bit compare-and-swap per new id, 23-25 G/s on this chip); the byte rate is "
+                              "reported because the stage is priced per edge in bytes elsewhere"},
         "aggregation": {"GBps": agg_gbps, "frac_peak": agg_gbps / HBM_PEAK_GBPS,
                         "stream_copy_GBps": stream_gbps, "frac_of_stream_copy": agg_gbps / stream_gbps},
         "random_read_Gps": random_read_gps,
